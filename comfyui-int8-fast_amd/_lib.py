@@ -1,0 +1,295 @@
+"""ctypes binding of libi8f_gfx950.so (the C ABI declared in include/i8f.h).
+
+This is the only place the package touches the native library.  There is no
+fallback: if the library is missing or the tensors are not on a gfx950 device,
+the functions raise.  Tensors are torch tensors used as device memory; the
+library launches on torch's current HIP stream.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libi8f_gfx950.so")
+
+BF16, F16, F32 = 0, 1, 2
+SCALE_TENSOR, SCALE_ROW = 0, 1
+EPI_TORCH, EPI_FUSED = 0, 1
+
+_DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
+
+_lib = None
+
+
+class I8FError(RuntimeError):
+    """A call into libi8f_gfx950.so returned a negative status."""
+
+    def __init__(self, what: str, status: int, text: str, hip_error: int = 0):
+        self.status = status
+        self.hip_error = hip_error
+        extra = f", hipError {hip_error}" if hip_error else ""
+        super().__init__(f"{what}: status {status} ({text}{extra})")
+
+
+def lib() -> ctypes.CDLL:
+    """Load the library once.  Raises RuntimeError with the build command if it is not there."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python {os.path.join(_HERE, 'build.py')}` "
+            "(needs hipcc; the INT8 path has no other implementation)."
+        )
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+    L.i8f_version.restype = i32
+    L.i8f_status_string.restype = ctypes.c_char_p
+    L.i8f_status_string.argtypes = [i32]
+    L.i8f_last_hip_error.restype = i32
+    L.i8f_quant_rowwise.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, vp]
+    L.i8f_rotate128.argtypes = [vp, i32, i64, i64, i64, vp, vp]
+    L.i8f_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp, vp]
+    L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
+    L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
+    L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
+    L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
+    for name in ("i8f_quant_rowwise", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8",
+                 "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
+        getattr(L, name).restype = i32
+    _lib = L
+    return L
+
+
+EXPORTS = (
+    "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
+    "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+)
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        L = lib()
+        text = L.i8f_status_string(status).decode()
+        raise I8FError(what, status, text, L.i8f_last_hip_error() if status == -3 else 0)
+
+
+def _dev(t: torch.Tensor, name: str) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} is on {t.device}: the INT8 engine runs on a gfx950 GPU only (no CPU path)")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dt}; expected bfloat16, float16 or float32") from None
+
+
+def _rows(x: torch.Tensor, name: str) -> torch.Tensor:
+    """A 2-D view whose rows are contiguous (row stride may exceed K)."""
+    if x.dim() != 2:
+        raise ValueError(f"{name} must be 2-D, got shape {tuple(x.shape)}")
+    if x.shape[1] > 1 and x.stride(1) != 1:
+        x = x.contiguous()
+    if x.shape[0] > 1 and x.stride(0) < x.shape[1]:
+        x = x.contiguous()
+    return x
+
+
+def _scale(ws, N: int, device):
+    """-> (device tensor or None, host float, mode).  Python floats travel by value."""
+    if isinstance(ws, torch.Tensor):
+        if ws.numel() == 1 and not ws.is_cuda:
+            return None, float(ws.item()), SCALE_TENSOR
+        if ws.device != device:
+            ws = ws.to(device, non_blocking=True)
+        ws = ws.reshape(-1)
+        if ws.dtype != torch.float32:
+            ws = ws.float()
+        ws = ws.contiguous()
+        if ws.numel() == 1:
+            return ws, 0.0, SCALE_TENSOR
+        if ws.numel() != N:
+            raise ValueError(f"weight scale has {ws.numel()} elements, expected 1 or {N}")
+        return ws, 0.0, SCALE_ROW
+    return None, float(ws), SCALE_TENSOR
+
+
+# --------------------------------------------------------------------------- entry points
+def quant_rowwise(x: torch.Tensor, rotate: bool = False):
+    """x [M,K] (bf16/fp16/fp32, cuda) -> (int8 [M,K], float32 [M,1]); rotate=True applies the 128-block Hadamard first."""
+    _dev(x, "x")
+    x = _rows(x, "x")
+    M, K = x.shape
+    if rotate and K % 128:
+        raise ValueError(f"rotation needs K % 128 == 0, got K={K}")
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    s = torch.empty((M, 1), dtype=torch.float32, device=x.device)
+    ldx = x.stride(0) if M > 1 else K
+    with torch.cuda.device(x.device):
+        _check(lib().i8f_quant_rowwise(_ptr(x), dtype_code(x.dtype), M, K, ldx, 128 if rotate else 0, _ptr(q), _ptr(s),
+                                       _stream(x)), "i8f_quant_rowwise")
+    return q, s
+
+
+def rotate128(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    _dev(x, "x")
+    x = _rows(x, "x")
+    M, K = x.shape
+    if K % 128:
+        raise ValueError(f"rotation needs K % 128 == 0, got K={K}")
+    if out is None:
+        out = torch.empty((M, K), dtype=x.dtype, device=x.device)
+    elif out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous() or out.device != x.device:
+        raise ValueError("out must be a contiguous tensor like x")
+    ldx = x.stride(0) if M > 1 else K
+    with torch.cuda.device(x.device):
+        _check(lib().i8f_rotate128(_ptr(x), dtype_code(x.dtype), M, K, ldx, _ptr(out), _stream(x)), "i8f_rotate128")
+    return out
+
+
+def _i8_matrix(t: torch.Tensor, name: str) -> torch.Tensor:
+    _dev(t, name)
+    if t.dtype != torch.int8 or t.dim() != 2:
+        raise TypeError(f"{name} must be a 2-D int8 tensor, got {t.dtype} {tuple(t.shape)}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def gemm_i32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """a [M,K] int8, w [N,K] int8 -> int32 [M,N] = a @ w.T"""
+    a, w = _i8_matrix(a, "a"), _i8_matrix(w, "w")
+    M, K = a.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise ValueError(f"K mismatch: a has {K}, w has {K2}")
+    acc = torch.empty((M, N), dtype=torch.int32, device=a.device)
+    with torch.cuda.device(a.device):
+        _check(lib().i8f_gemm_i32(_ptr(a), _ptr(w), M, N, K, _ptr(acc), _stream(a)), "i8f_gemm_i32")
+    return acc
+
+
+def _bias_arg(bias, N, device):
+    if bias is None:
+        return None, BF16
+    if bias.device != device:
+        bias = bias.to(device, non_blocking=True)
+    bias = bias.reshape(-1).contiguous()
+    if bias.numel() != N:
+        raise ValueError(f"bias has {bias.numel()} elements, expected {N}")
+    return bias, dtype_code(bias.dtype)
+
+
+def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None):
+    """Quantised activations (a int8 [M,K], a_scale [M,1]) times int8 weight [N,K] with the fused dequant epilogue."""
+    a, w = _i8_matrix(a, "a"), _i8_matrix(w, "w")
+    M, K = a.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise ValueError(f"K mismatch: a has {K}, w has {K2}")
+    _dev(a_scale, "a_scale")
+    a_scale = a_scale.reshape(-1)
+    if a_scale.numel() != M or a_scale.dtype != torch.float32:
+        raise ValueError("a_scale must be float32 with M elements")
+    a_scale = a_scale.contiguous()
+    ws, ws_host, mode = _scale(w_scale, N, a.device)
+    bias, bcode = _bias_arg(bias, N, a.device)
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    with torch.cuda.device(a.device):
+        _check(lib().i8f_linear_w8a8(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
+                                     _ptr(out), dtype_code(out.dtype), M, N, K, order, _stream(a)), "i8f_linear_w8a8")
+    return out
+
+
+def linear_w8a16_small_m(x, w, w_scale, bias=None):
+    """x [M<=16,K] float, w int8 [N,K] -> [M,N] in x's dtype (weight dequantised on the fly)."""
+    _dev(x, "x")
+    x = _rows(x, "x")
+    w = _i8_matrix(w, "w")
+    M, K = x.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise ValueError(f"K mismatch: x has {K}, w has {K2}")
+    ws, ws_host, mode = _scale(w_scale, N, x.device)
+    bias, bcode = _bias_arg(bias, N, x.device)
+    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    ldx = x.stride(0) if M > 1 else K
+    with torch.cuda.device(x.device):
+        _check(lib().i8f_linear_w8a16_small_m(_ptr(x), dtype_code(x.dtype), M, K, ldx, _ptr(w), _ptr(ws), ws_host, mode,
+                                              _ptr(bias), bcode, _ptr(out), N, _stream(x)), "i8f_linear_w8a16_small_m")
+    return out
+
+
+def _f32_matrix(t, name, device):
+    if t.device != device:
+        t = t.to(device)
+    if t.dtype != torch.float32:
+        t = t.float()
+    if t.dim() != 2:
+        raise ValueError(f"{name} must be 2-D")
+    return t.contiguous()
+
+
+def sr_quant_delta(x, scale, noise):
+    """Stochastic rounding of x / scale to int8 with the supplied uniform noise (both [N,K] float32)."""
+    _dev(x, "x")
+    x = _f32_matrix(x, "x", x.device)
+    noise = _f32_matrix(noise, "noise", x.device)
+    if noise.shape != x.shape:
+        raise ValueError("noise must have the shape of x")
+    N, K = x.shape
+    ws, ws_host, mode = _scale(scale, N, x.device)
+    dq = torch.empty((N, K), dtype=torch.int8, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(lib().i8f_sr_quant_delta(_ptr(x), _ptr(ws), ws_host, mode, _ptr(noise), N, K, _ptr(dq), _stream(x)),
+               "i8f_sr_quant_delta")
+    return dq
+
+
+def lora_merge_sr(w, w_scale, noise, delta=None, up=None, down=None, lora_scale=1.0, out=None):
+    """w' = sat8(w + SR(delta / w_scale)); delta given, or rebuilt from up [N,r] / down [r,K] (times lora_scale)."""
+    w = _i8_matrix(w, "w")
+    N, K = w.shape
+    noise = _f32_matrix(noise, "noise", w.device)
+    if noise.shape != w.shape:
+        raise ValueError("noise must have the shape of w")
+    rank = 0
+    if delta is not None:
+        delta = _f32_matrix(delta, "delta", w.device)
+        if delta.shape != w.shape:
+            raise ValueError("delta must have the shape of w")
+    else:
+        if up is None or down is None:
+            raise ValueError("give either delta or both up and down")
+        up = _f32_matrix(up, "up", w.device)
+        down = _f32_matrix(down, "down", w.device)
+        rank = up.shape[1]
+        if up.shape[0] != N or down.shape != (rank, K):
+            raise ValueError(f"up must be [{N},r] and down [r,{K}]")
+    ws, ws_host, mode = _scale(w_scale, N, w.device)
+    if out is None:
+        out = torch.empty_like(w)
+    elif out.shape != w.shape or out.dtype != torch.int8 or not out.is_contiguous():
+        raise ValueError("out must be a contiguous int8 tensor like w")
+    with torch.cuda.device(w.device):
+        _check(lib().i8f_lora_merge_sr(_ptr(w), _ptr(ws), ws_host, mode, _ptr(delta), _ptr(up), _ptr(down), rank,
+                                       float(lora_scale), _ptr(noise), N, K, _ptr(out), _stream(w)), "i8f_lora_merge_sr")
+    return out
+
+
+def version() -> int:
+    return int(lib().i8f_version())

@@ -1,0 +1,111 @@
+// Shared device helpers of the gfx950 INT8 linear engine.
+//
+// All floating-point code in this library is compiled with -ffp-contract=off:
+// a multiply followed by an add is two rounded operations unless the source
+// says fmaf().  The bit-exact contracts of the quantiser, the epilogue and the
+// LoRA merge depend on it.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/i8f.h"
+
+namespace i8f {
+
+// thread-local record of the last HIP error, read by i8f_last_hip_error()
+int &last_hip_error_slot();
+
+inline int check_launch() {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        last_hip_error_slot() = (int)e;
+        return I8F_ERR_HIP;
+    }
+    return I8F_OK;
+}
+
+// I8F_OK if the current device is a gfx950, I8F_ERR_DEVICE otherwise (cached per device).
+int check_device();
+
+struct bf16_t {
+    uint16_t bits;
+};
+struct f16_t {
+    uint16_t bits;
+};
+
+// ---- widen -----------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+
+// ---- round to nearest even ---------------------------------------------------
+// bfloat16: the hardware conversion of gfx950 (v_cvt_pk_bf16_f32) rounds to
+// nearest even and quiets NaNs, the same as torch's float -> bfloat16 cast.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float v) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v);
+}
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    f2 in = {lo, hi};
+    bf2 o = __builtin_convertvector(in, bf2);
+    return __builtin_bit_cast(uint32_t, o);
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float v) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v);
+}
+__device__ __forceinline__ uint32_t f32x2_to_f16x2_bits(float lo, float hi) {
+    return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+}
+
+// value rounded to the storage dtype and widened again
+template <int DT>
+__device__ __forceinline__ float round_to_dtype(float v) {
+    if constexpr (DT == I8F_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+    else if constexpr (DT == I8F_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
+    else return v;
+}
+
+template <int DT>
+__device__ __forceinline__ float load_as_f32(const void *p, int64_t i) {
+    if constexpr (DT == I8F_BF16) return bf16_bits_to_f32(((const uint16_t *)p)[i]);
+    else if constexpr (DT == I8F_F16) return f16_bits_to_f32(((const uint16_t *)p)[i]);
+    else return ((const float *)p)[i];
+}
+
+template <int DT>
+__device__ __forceinline__ void store_from_f32(void *p, int64_t i, float v) {
+    if constexpr (DT == I8F_BF16) ((uint16_t *)p)[i] = (uint16_t)f32_to_bf16_bits(v);
+    else if constexpr (DT == I8F_F16) ((uint16_t *)p)[i] = (uint16_t)f32_to_f16_bits(v);
+    else ((float *)p)[i] = v;
+}
+
+// The entry of the normalised 128-point Hadamard matrix in each dtype:
+// 1/sqrt(128) rounded to that dtype (0x3DB504F3 in binary32; 181/2048 in
+// bfloat16 and binary16), as quarot.py:35-36 of the reference builds it.
+template <int DT>
+__device__ __forceinline__ float hadamard_entry() {
+    if constexpr (DT == I8F_F32) return __uint_as_float(0x3DB504F3u);
+    else return 0.08837890625f;
+}
+
+// round-to-nearest-even float -> int8 with saturation
+__device__ __forceinline__ int quant_i8(float v) {
+    float r = __builtin_rintf(v);
+    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return (int)r;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+inline size_t dtype_size(int dt) { return dt == I8F_F32 ? 4 : 2; }
+inline bool valid_dtype(int dt) { return dt == I8F_BF16 || dt == I8F_F16 || dt == I8F_F32; }
+
+}  // namespace i8f

@@ -1,0 +1,385 @@
+// Fused (block-Hadamard rotation +) per-row absmax int8 quantiser for gfx950.
+//
+// One pass over HBM: a row is read once with 16-byte loads, kept in registers,
+// optionally rotated, reduced to its absolute maximum, scaled, rounded and
+// written as int8 with its float scale.  The reference does this in two
+// (quantise, int8_fused_kernel.py:10-73) or three (rotate first, quarot.py:99-102)
+// separate passes.
+//
+// Arithmetic contract (bit-exact with the torch path int8_quant.py:20-31 on CPU):
+//   amax  = max |v|                    v = x, or the rotated row rounded to x's dtype
+//   scale = max(amax / 127.0f, 1e-30f) correctly rounded division
+//   inv   = 1.0f / scale               correctly rounded division
+//   q     = sat8(rint(v * inv))        ties to even
+//
+// Rotation: every aligned block of 128 elements is multiplied by the normalised
+// Sylvester-Hadamard matrix of x's dtype.  It is evaluated as a 7-stage
+// radix-2 butterfly in binary32 with strides 1,2,...,64, each pair (lo,hi)
+// becoming (lo+hi, lo-hi), then one multiply by the matrix entry and one
+// rounding to x's dtype.  Strides smaller than the per-lane chunk are done in
+// registers, the rest across lanes; the order of operations does not depend on
+// how the block is spread over lanes.
+#include "i8f_common.hpp"
+
+namespace i8f {
+namespace {
+
+template <int DT>
+struct Elem {
+    static constexpr int EPC = (DT == I8F_F32) ? 4 : 8;  // elements per 16-byte chunk
+    static constexpr int LPB = 128 / EPC;                // lanes that share one 128-block
+};
+
+template <int DT>
+__device__ __forceinline__ void load_chunk(const void *p, float (&v)[Elem<DT>::EPC]) {
+    const uint4 u = *(const uint4 *)p;
+    if constexpr (DT == I8F_F32) {
+        v[0] = __uint_as_float(u.x);
+        v[1] = __uint_as_float(u.y);
+        v[2] = __uint_as_float(u.z);
+        v[3] = __uint_as_float(u.w);
+    } else if constexpr (DT == I8F_BF16) {
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = __uint_as_float(w[j] << 16);
+            v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        }
+    } else {
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = f16_bits_to_f32(w[j] & 0xffffu);
+            v[2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+        }
+    }
+}
+
+// Rotate the chunk held by this lane; the LPB lanes of an aligned group hold one
+// 128-block, lane g of the group holding elements [g*EPC, (g+1)*EPC).
+template <int DT>
+__device__ __forceinline__ void rotate_chunk(float (&v)[Elem<DT>::EPC], int lane) {
+    constexpr int EPC = Elem<DT>::EPC;
+    constexpr int LPB = Elem<DT>::LPB;
+#pragma unroll
+    for (int s = 1; s < EPC; s <<= 1) {
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) {
+            if ((j & s) == 0) {
+                const float lo = v[j], hi = v[j + s];
+                v[j] = lo + hi;
+                v[j + s] = lo - hi;
+            }
+        }
+    }
+#pragma unroll
+    for (int b = 1; b < LPB; b <<= 1) {
+        const bool upper = (lane & b) != 0;
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) {
+            const float other = __shfl_xor(v[j], b, 64);
+            v[j] = upper ? (other - v[j]) : (v[j] + other);
+        }
+    }
+    const float h = hadamard_entry<DT>();
+#pragma unroll
+    for (int j = 0; j < EPC; ++j) v[j] = round_to_dtype<DT>(v[j] * h);
+}
+
+// TPR threads share a row (64, 256 or 1024); each holds NCH chunks of it.
+template <int DT, bool ROT, int TPR, int NCH>
+__global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void quant_rows_kernel(
+    const char *__restrict__ x, int64_t M, int64_t K, int64_t ldx_bytes, int8_t *__restrict__ q,
+    float *__restrict__ scale) {
+    constexpr int EPC = Elem<DT>::EPC;
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int ROWS = BLOCK / TPR;
+    constexpr int WPR = TPR / 64;  // waves per row
+    const int t = threadIdx.x % TPR;
+    const int rb = threadIdx.x / TPR;
+    const int64_t m = (int64_t)blockIdx.x * ROWS + rb;
+    const bool row_ok = m < M;
+    const int nchunks = (int)(K / EPC);
+    const char *xrow = x + (row_ok ? m : 0) * ldx_bytes;
+
+    float v[NCH][EPC];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = i * TPR + t;
+        if (row_ok && c < nchunks) {
+            load_chunk<DT>(xrow + (int64_t)c * 16, v[i]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPC; ++j) v[i][j] = 0.0f;
+        }
+    }
+
+    if constexpr (ROT) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) rotate_chunk<DT>(v[i], t);
+    }
+
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+    amax = wave_max(amax);
+    if constexpr (WPR > 1) {
+        __shared__ float red[ROWS][WPR];
+        const int wv = t / 64;
+        if ((t & 63) == 0) red[rb][wv] = amax;
+        __syncthreads();
+        amax = red[rb][0];
+#pragma unroll
+        for (int w = 1; w < WPR; ++w) amax = fmaxf(amax, red[rb][w]);
+    }
+
+    float s = amax / 127.0f;
+    s = s < 1e-30f ? 1e-30f : s;
+    const float inv = 1.0f / s;
+
+    if (!row_ok) return;
+    int8_t *qrow = q + m * K;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = i * TPR + t;
+        if (c < nchunks) {
+            uint32_t packed[EPC / 4];
+#pragma unroll
+            for (int j = 0; j < EPC / 4; ++j) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    w |= ((uint32_t)quant_i8(v[i][4 * j + b] * inv) & 0xffu) << (8 * b);
+                packed[j] = w;
+            }
+            if constexpr (EPC == 8) {
+                *(uint2 *)(qrow + (int64_t)c * 8) = make_uint2(packed[0], packed[1]);
+            } else {
+                *(uint32_t *)(qrow + (int64_t)c * 4) = packed[0];
+            }
+        }
+    }
+    if (t == 0) scale[m] = s;
+}
+
+// ---- generic kernel: any K, any alignment; one 256-thread block per row, the row
+// is read twice (the second time from cache) --------------------------------------
+template <int DT>
+__device__ __forceinline__ void rotate128_wave(float &e0, float &e1, int lane) {
+    // the wave holds one 128-block: lane l has elements l (e0) and l + 64 (e1)
+#pragma unroll
+    for (int b = 1; b < 64; b <<= 1) {
+        const bool upper = (lane & b) != 0;
+        const float o0 = __shfl_xor(e0, b, 64);
+        const float o1 = __shfl_xor(e1, b, 64);
+        e0 = upper ? (o0 - e0) : (e0 + o0);
+        e1 = upper ? (o1 - e1) : (e1 + o1);
+    }
+    const float lo = e0, hi = e1;
+    e0 = lo + hi;
+    e1 = lo - hi;
+    const float h = hadamard_entry<DT>();
+    e0 = round_to_dtype<DT>(e0 * h);
+    e1 = round_to_dtype<DT>(e1 * h);
+}
+
+template <int DT, bool ROT>
+__global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__restrict__ x, int64_t M,
+                                                                  int64_t K, int64_t ldx,
+                                                                  int8_t *__restrict__ q,
+                                                                  float *__restrict__ scale) {
+    const int64_t m = blockIdx.x;
+    if (m >= M) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wv = tid >> 6;
+    const int64_t base = m * ldx;
+    __shared__ float red[4];
+
+    float amax = 0.0f;
+    if constexpr (ROT) {
+        for (int64_t blk = wv; blk < K / 128; blk += 4) {
+            float e0 = load_as_f32<DT>(x, base + blk * 128 + lane);
+            float e1 = load_as_f32<DT>(x, base + blk * 128 + 64 + lane);
+            rotate128_wave<DT>(e0, e1, lane);
+            amax = fmaxf(amax, fmaxf(fabsf(e0), fabsf(e1)));
+        }
+    } else {
+        for (int64_t k = tid; k < K; k += 256) amax = fmaxf(amax, fabsf(load_as_f32<DT>(x, base + k)));
+    }
+    amax = wave_max(amax);
+    if (lane == 0) red[wv] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+
+    float s = amax / 127.0f;
+    s = s < 1e-30f ? 1e-30f : s;
+    const float inv = 1.0f / s;
+    int8_t *qrow = q + m * K;
+    if constexpr (ROT) {
+        for (int64_t blk = wv; blk < K / 128; blk += 4) {
+            float e0 = load_as_f32<DT>(x, base + blk * 128 + lane);
+            float e1 = load_as_f32<DT>(x, base + blk * 128 + 64 + lane);
+            rotate128_wave<DT>(e0, e1, lane);
+            qrow[blk * 128 + lane] = (int8_t)quant_i8(e0 * inv);
+            qrow[blk * 128 + 64 + lane] = (int8_t)quant_i8(e1 * inv);
+        }
+    } else {
+        for (int64_t k = tid; k < K; k += 256)
+            qrow[k] = (int8_t)quant_i8(load_as_f32<DT>(x, base + k) * inv);
+    }
+    if (tid == 0) scale[m] = s;
+}
+
+// ---- rotation alone -------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ void store_chunk(void *p, const float (&v)[Elem<DT>::EPC]) {
+    if constexpr (DT == I8F_F32) {
+        *(float4 *)p = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (DT == I8F_BF16) w[j] = f32x2_to_bf16x2_bits(v[2 * j], v[2 * j + 1]);
+            else w[j] = f32x2_to_f16x2_bits(v[2 * j], v[2 * j + 1]);
+        }
+        *(uint4 *)p = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+// one thread per 16-byte chunk; an aligned group of LPB lanes holds one 128-block
+template <int DT>
+__global__ __launch_bounds__(256) void rotate_kernel(const char *x, int64_t M, int64_t K,
+                                                      int64_t ldx_bytes, char *out) {
+    constexpr int EPC = Elem<DT>::EPC;
+    const int64_t nchunks = K / EPC;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool ok = idx < M * nchunks;
+    const int64_t m = ok ? idx / nchunks : 0, c = ok ? idx % nchunks : 0;
+    float v[EPC];
+    if (ok) {
+        load_chunk<DT>(x + m * ldx_bytes + c * 16, v);
+    } else {
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) v[j] = 0.0f;
+    }
+    rotate_chunk<DT>(v, threadIdx.x);
+    if (ok) store_chunk<DT>(out + (m * nchunks + c) * 16, v);
+}
+
+// any alignment: one wavefront per 128-block
+template <int DT>
+__global__ __launch_bounds__(256) void rotate_generic_kernel(const void *x, int64_t M, int64_t K,
+                                                              int64_t ldx, void *out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t per_row = K / 128;
+    if (blk >= M * per_row) return;
+    const int64_t m = blk / per_row, b = blk % per_row;
+    float e0 = load_as_f32<DT>(x, m * ldx + b * 128 + lane);
+    float e1 = load_as_f32<DT>(x, m * ldx + b * 128 + 64 + lane);
+    rotate128_wave<DT>(e0, e1, lane);
+    store_from_f32<DT>(out, m * K + b * 128 + lane, e0);
+    store_from_f32<DT>(out, m * K + b * 128 + 64 + lane, e1);
+}
+
+template <int DT>
+int launch_rotate(const void *x, int64_t M, int64_t K, int64_t ldx, void *out, hipStream_t st) {
+    constexpr int EPC = Elem<DT>::EPC;
+    const size_t es = dtype_size(DT);
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && ((uintptr_t)out % 16 == 0);
+    if (aligned) {
+        const int64_t total = M * (K / EPC);
+        hipLaunchKernelGGL((rotate_kernel<DT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                           (const char *)x, M, K, ldx * (int64_t)es, (char *)out);
+    } else {
+        const int64_t blocks = M * (K / 128);
+        hipLaunchKernelGGL((rotate_generic_kernel<DT>), dim3((unsigned)((blocks + 3) / 4)), dim3(256), 0, st, x, M,
+                           K, ldx, out);
+    }
+    return check_launch();
+}
+
+template <int DT, bool ROT, int TPR, int NCH>
+int launch_fast(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale,
+                hipStream_t st) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int ROWS = BLOCK / TPR;
+    const int64_t blocks = (M + ROWS - 1) / ROWS;
+    hipLaunchKernelGGL((quant_rows_kernel<DT, ROT, TPR, NCH>), dim3((unsigned)blocks), dim3(BLOCK), 0, st,
+                       (const char *)x, M, K, ldx * (int64_t)dtype_size(DT), q, scale);
+    return check_launch();
+}
+
+template <int DT, bool ROT, int TPR>
+int pick_nch(int per_thread, const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale,
+             hipStream_t st) {
+    if (per_thread <= 1) return launch_fast<DT, ROT, TPR, 1>(x, M, K, ldx, q, scale, st);
+    if (per_thread <= 2) return launch_fast<DT, ROT, TPR, 2>(x, M, K, ldx, q, scale, st);
+    if (per_thread <= 4) return launch_fast<DT, ROT, TPR, 4>(x, M, K, ldx, q, scale, st);
+    if (per_thread <= 6) return launch_fast<DT, ROT, TPR, 6>(x, M, K, ldx, q, scale, st);
+    return launch_fast<DT, ROT, TPR, 8>(x, M, K, ldx, q, scale, st);
+}
+
+template <int DT, bool ROT>
+int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st) {
+    constexpr int EPC = Elem<DT>::EPC;
+    const size_t es = dtype_size(DT);
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) &&
+                         ((uintptr_t)q % 8 == 0);
+    const int64_t nchunks = K / EPC;
+    if (aligned && nchunks <= 1024 * 8) {
+        if (nchunks <= 64 * 8) return pick_nch<DT, ROT, 64>((int)((nchunks + 63) / 64), x, M, K, ldx, q, scale, st);
+        if (nchunks <= 256 * 8) return pick_nch<DT, ROT, 256>((int)((nchunks + 255) / 256), x, M, K, ldx, q, scale, st);
+        return pick_nch<DT, ROT, 1024>((int)((nchunks + 1023) / 1024), x, M, K, ldx, q, scale, st);
+    }
+    hipLaunchKernelGGL((quant_rows_generic_kernel<DT, ROT>), dim3((unsigned)M), dim3(256), 0, st, x, M, K, ldx,
+                       q, scale);
+    return check_launch();
+}
+
+template <int DT>
+int dispatch_rot(bool rot, const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale,
+                 hipStream_t st) {
+    return rot ? dispatch<DT, true>(x, M, K, ldx, q, scale, st) : dispatch<DT, false>(x, M, K, ldx, q, scale, st);
+}
+
+}  // namespace
+}  // namespace i8f
+
+extern "C" int i8f_quant_rowwise(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                 int rotate_block, int8_t *q, float *scale, void *stream) {
+    using namespace i8f;
+    if (M < 0 || K < 0 || !valid_dtype(x_dtype)) return I8F_ERR_INVALID;
+    if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
+    if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
+    if (M == 0) return I8F_OK;
+    if (!scale || ldx < K) return I8F_ERR_INVALID;
+    if (K > 0 && (!x || !q)) return I8F_ERR_INVALID;
+    if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
+    if (int rc = check_device()) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const bool rot = rotate_block != 0;
+    switch (x_dtype) {
+    case I8F_BF16: return dispatch_rot<I8F_BF16>(rot, x, M, K, ldx, q, scale, st);
+    case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st);
+    default: return dispatch_rot<I8F_F32>(rot, x, M, K, ldx, q, scale, st);
+    }
+}
+
+extern "C" int i8f_rotate128(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, void *out, void *stream) {
+    using namespace i8f;
+    if (M < 0 || K < 0 || !valid_dtype(dtype) || K % 128) return I8F_ERR_INVALID;
+    if (M == 0 || K == 0) return I8F_OK;
+    if (!x || !out || ldx < K) return I8F_ERR_INVALID;
+    if (x == out && ldx != K) return I8F_ERR_INVALID;
+    if (M * (K / 4) / 256 > 0x7fffffffll) return I8F_ERR_UNSUPPORTED;
+    if (int rc = check_device()) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+    case I8F_BF16: return launch_rotate<I8F_BF16>(x, M, K, ldx, out, st);
+    case I8F_F16: return launch_rotate<I8F_F16>(x, M, K, ldx, out, st);
+    default: return launch_rotate<I8F_F32>(x, M, K, ldx, out, st);
+    }
+}

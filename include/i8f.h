@@ -1,0 +1,185 @@
+/*
+ * i8f.h -- C ABI of the MI355X (gfx950) INT8 linear-layer engine.
+ *
+ * One shared library, libi8f_gfx950.so, built by hipcc for gfx950 only.  It is
+ * the drop-in replacement for the device side of ComfyUI-INT8-Fast's W8A8
+ * linear path: the three Triton kernels of int8_fused_kernel.py, the online
+ * QuaRot rotation of quarot.py and the elementwise torch chain that merges a
+ * LoRA into int8 weights.  The reference has no foreign-function interface of
+ * its own (it launches Triton from Python); each entry point therefore names
+ * the Python function whose device work it replaces.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer owned by the caller.  The library never
+ *     allocates, frees or keeps device memory.
+ *   - Matrices are row-major.  Weights are int8 [N,K] with K contiguous and are
+ *     consumed transposed ("NT" product), exactly the reference's layout
+ *     (int8_fused_kernel.py:211-214,228).  Activation scales are [M] float
+ *     (the reference's [M,1]); per-row weight scales are [N] float ([N,1]).
+ *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.
+ *     Work is enqueued asynchronously; no entry point synchronises.
+ *   - Return value: I8F_OK (0) or a negative i8f_status.  No C++ exception
+ *     crosses this boundary.  Arguments are validated on the host BEFORE any
+ *     launch; a failing call launches nothing.
+ *   - The library keeps no mutable global state: calls are re-entrant and may
+ *     be issued from several host threads on different streams.
+ *   - Non-finite inputs (NaN/Inf) give unspecified int8 values, as in the
+ *     reference (a float NaN cast to int8 is undefined there too).
+ */
+#ifndef I8F_H
+#define I8F_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define I8F_VERSION 100 /* major*10000 + minor*100 + patch */
+
+typedef enum i8f_status {
+    I8F_OK = 0,
+    I8F_ERR_INVALID = -1,     /* NULL pointer, negative size, bad enum, misaligned or aliased argument */
+    I8F_ERR_UNSUPPORTED = -2, /* a shape this build has no kernel for (documented per entry point) */
+    I8F_ERR_HIP = -3,         /* the HIP runtime refused the launch; see i8f_last_hip_error() */
+    I8F_ERR_DEVICE = -4       /* the current device is not gfx950 */
+} i8f_status;
+
+typedef enum i8f_dtype { I8F_BF16 = 0, I8F_F16 = 1, I8F_F32 = 2 } i8f_dtype;
+
+/* one weight scale for the whole matrix, or one per output row (weight row) */
+typedef enum i8f_scale_mode { I8F_SCALE_TENSOR = 0, I8F_SCALE_ROW = 1 } i8f_scale_mode;
+
+/*
+ * Order of the floating-point operations of the dequantisation epilogue.
+ *   I8F_EPI_TORCH  the reference's torch path (int8_quant.py:84-87, 115-118):
+ *                  round the scaled accumulator to the output dtype, then add
+ *                  the bias (itself rounded to the output dtype) and round again.
+ *                  Bit-identical to that path on the CPU.  The default of the
+ *                  Python host layer.
+ *   I8F_EPI_FUSED  the reference's fused kernels (int8_fused_kernel.py:156-173,
+ *                  310-324): acc * (xs * ws) + bias in binary32, one rounding.
+ */
+typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
+
+/* Library version (I8F_VERSION of the build). */
+int i8f_version(void);
+
+/* Static, human-readable text for a status code. */
+const char *i8f_status_string(int status);
+
+/* hipError_t of the most recent I8F_ERR_HIP on the calling thread (0 if none). */
+int i8f_last_hip_error(void);
+
+/*
+ * Fused (optional block rotation +) dynamic per-row absmax int8 quantisation.
+ * Replaces triton_quantize_rowwise / _quantize_rowwise_kernel
+ * (int8_fused_kernel.py:10-73), with the arithmetic of the torch path
+ * quantize_int8_axiswise (int8_quant.py:28-31, 20-21), and, when
+ * rotate_block == 128, the preceding rotate_activation (quarot.py:73-102 called
+ * at int8_quant.py:741-744) or rotate_weight (quarot.py:42-70 called at
+ * int8_quant.py:602-607) in the same pass over memory.
+ *
+ *   x        [M,K] of x_dtype, row stride ldx elements (ldx >= K)
+ *   rotate_block   0 (no rotation) or 128 (K must then be a multiple of 128)
+ *   q        [M,K] int8, contiguous            scale   [M] float
+ *
+ * Any M >= 0 and K >= 0.  I8F_ERR_UNSUPPORTED for another rotate_block.
+ */
+int i8f_quant_rowwise(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                      int rotate_block, int8_t *q, float *scale, void *stream);
+
+/*
+ * Block rotation alone (no quantisation): every aligned block of 128 elements of
+ * each row is multiplied by the normalised Hadamard matrix, result in x's dtype.
+ * Replaces rotate_weight / rotate_activation (quarot.py:42-102) where the rotated
+ * tensor itself is wanted: the LoRA delta of a rotated layer
+ * (int8_quant.py:300-306, 387-393).  Same butterfly as i8f_quant_rowwise.
+ *   x [M,K] of dtype (row stride ldx), out [M,K] contiguous, K % 128 == 0.
+ *   out may equal x when ldx == K.
+ */
+int i8f_rotate128(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, void *out,
+                  void *stream);
+
+/*
+ * int8 x int8 -> int32 product, acc[m,n] = sum_k a[m,k] * w[n,k].
+ * Replaces torch._int_mm(x8, weight.T) (int8_quant.py:80,110); it is the
+ * accumulator of the fused kernels (int8_fused_kernel.py:132-144) made visible,
+ * so that parity of the integer part can be checked bit for bit.
+ *   a [M,K] int8   w [N,K] int8   acc [M,N] int32, all contiguous.
+ */
+int i8f_gemm_i32(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K,
+                 int32_t *acc, void *stream);
+
+/*
+ * INT8 GEMM with the dequantisation epilogue fused in registers.
+ * Replaces _int8_matmul_dequant_kernel and _int8_matmul_dequant_per_row_kernel
+ * (int8_fused_kernel.py:91-173, 253-324) and the torch epilogue
+ * (int8_quant.py:84-87, 115-118):
+ *   out[m,n] = epilogue( sum_k a[m,k]*w[n,k], a_scale[m], w_scale[n or 0], bias[n] )
+ *
+ *   a [M,K] int8, a_scale [M] float          (outputs of i8f_quant_rowwise)
+ *   w [N,K] int8
+ *   w_scale   device pointer to 1 (TENSOR) or N (ROW) floats; with TENSOR it may
+ *             be NULL, and then the host value w_scale_host is used
+ *   bias      NULL or [N] of bias_dtype
+ *   out       [M,N] of out_dtype (I8F_BF16 or I8F_F16; I8F_F32 for debugging)
+ *   order     i8f_epilogue
+ */
+int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                    float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                    void *out, int out_dtype, int64_t M, int64_t N, int64_t K, int order,
+                    void *stream);
+
+/*
+ * Small-batch W8A16 path, M <= 16: activations stay in their dtype, the int8
+ * weight is dequantised on the fly.  Replaces the "small batch fallback" of
+ * Linear.forward (int8_quant.py:756-760):
+ *   out = F.linear(x, (float(w) * w_scale).to(x.dtype), bias.to(x.dtype))
+ * without materialising the dequantised weight.  Products are accumulated in
+ * binary32; the result is within the tolerance the tests state of the
+ * reference, whose BLAS summation order is unspecified.
+ *   x [M,K] of x_dtype (row stride ldx), out [M,N] of x_dtype.
+ * I8F_ERR_UNSUPPORTED for M > 16.
+ */
+int i8f_linear_w8a16_small_m(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                             const int8_t *w, const float *w_scale, float w_scale_host,
+                             int scale_mode, const void *bias, int bias_dtype, void *out,
+                             int64_t N, void *stream);
+
+/*
+ * Stochastic rounding of a float delta to int8 with SUPPLIED uniform noise.
+ * Replaces stochastic_round_int8_delta (int8_quant.py:36-62); the reference
+ * draws the noise from a device generator (:41,55), which no other device can
+ * reproduce, so the caller passes the [N,K] float noise in [0,1).
+ *   dq[n,k] = int8(clamp(noise < frac(x/scale) ? floor(x/scale)+1 : floor(x/scale)))
+ *   x, noise [N,K] float; scale as w_scale above; dq [N,K] int8.
+ */
+int i8f_sr_quant_delta(const float *x, const float *scale, float scale_host, int scale_mode,
+                       const float *noise, int64_t N, int64_t K, int8_t *dq, void *stream);
+
+/*
+ * LoRA merge in int8 space.  Replaces the int8 branch of
+ * INT8LoRAPatchAdapter.calculate_weight / INT8MergedLoRAPatchAdapter
+ * (int8_quant.py:293-318, 382-404): stochastic rounding of the scaled delta with
+ * the layer's weight scale, saturating int8 add, in ONE pass over memory.
+ *
+ *   w_out[n,k] = sat8( w[n,k] + SR(delta_f[n,k] / w_scale[n or 0], noise[n,k]) )
+ *
+ * delta_f is either supplied (delta != NULL: [N,K] float, already multiplied by
+ * the LoRA scale; up/down/rank ignored) or rebuilt in the kernel from the
+ * low-rank factors (delta == NULL): up [N,rank], down [rank,K] float,
+ *   delta_f[n,k] = (sum_j up[n,j]*down[j,k]) * lora_scale
+ * with the sum taken as a chain of fused multiply-adds in increasing j
+ * (reconstruct_lora_diff case 1, int8_quant.py:143-157, and :295).
+ * w_out may equal w (in-place).  rank <= 256 for the fused form.
+ */
+int i8f_lora_merge_sr(const int8_t *w, const float *w_scale, float w_scale_host, int scale_mode,
+                      const float *delta, const float *up, const float *down, int64_t rank,
+                      float lora_scale, const float *noise, int64_t N, int64_t K, int8_t *w_out,
+                      void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* I8F_H */
