@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the INT8 linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
+
+One "step" is one pass of BASELINE config 1, the Flux-style MLP in W8A8 rowwise:
+    quantise x [4608,3072] -> GEMM with W_up [12288,3072] (+bias)
+    quantise h [4608,12288] (synthetic half-normal) -> GEMM with W_dn [3072,12288] (+bias)
+with every input already resident in HBM.  The headline `value` is the int8 GEMM work of
+the step (2*M*N*K per GEMM) divided by the wall time of the WHOLE step, quantisers
+included, in TOP/s.  The JSON line also carries
+    roofline      the dominant kernel (the MFMA GEMM) against the dense int8 peak, from HIP
+                  events recorded around its launches inside the timed region
+    cpu_baseline  the reference's torch CPU path (oracle/torch_path.py) on a bounded sample
+    extras        the north-star target shape, the fused rotate+quant kernel against HBM
+                  bandwidth, the LoRA merge, and ms per Flux-style DiT block (config 3)
+Synthetic data, random-init weights; see make_config() for the seeded recipes.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+
+
+# --------------------------------------------------------------------------- workloads
+def _acts(g, M, K, frac, mul):
+    x = torch.randn(M, K, generator=g)
+    idx = torch.randperm(K, generator=g)[: int(K * frac)]
+    x[:, idx] *= mul
+    return x.bfloat16()
+
+
+def make_config(i: int, rows: int | None = None) -> dict:
+    """Seeded CPU tensors of BASELINE config i (0..4).  `rows` truncates the token dimension
+    (the same leading rows) for CPU-sized checks; weights always have their full shape."""
+    g = torch.Generator().manual_seed(1000 + i)
+    if i == 0:   # single W8A8 linear, one weight scale, no bias
+        x = _acts(g, 4096, 3072, 0.01, 20.0)
+        w = (torch.randn(3072, 3072, generator=g) * 0.02).bfloat16()
+        return {"x": x[:rows] if rows else x, "w": w, "scale_mode": "tensor", "bias": None}
+    if i == 1:   # Flux MLP: up projection on N(0,1) activations, down projection on half-normal ones
+        x = _acts(g, 4608, 3072, 0.01, 20.0)
+        w_up = torch.randn(12288, 3072, generator=g) * 0.02
+        b_up = (torch.randn(12288, generator=g) * 0.01).bfloat16()
+        h = torch.randn(4608 if rows is None else rows, 12288, generator=g).abs_().bfloat16()
+        w_dn = torch.randn(3072, 12288, generator=g) * 0.02
+        b_dn = (torch.randn(3072, generator=g) * 0.01).bfloat16()
+        return {"x": x[:rows] if rows else x, "w_up": w_up, "b_up": b_up, "h": h, "w_dn": w_dn, "b_dn": b_dn}
+    if i == 2:   # QuaRot: heavy outliers, 128-block rotation, width 3840
+        x = _acts(g, 4096, 3840, 0.02, 50.0)
+        w = torch.randn(3840, 3840, generator=g) * 0.02
+        return {"x": x[:rows] if rows else x, "w": w, "rotate": True}
+    if i == 3:   # one double-stream DiT block, width 3072: shapes only (weights are drawn on the device)
+        return {"hidden": 3072, "heads": 24, "img": 4096, "txt": 512,
+                "linears": {"qkv": (9216, 3072), "proj": (3072, 3072), "up": (12288, 3072), "down": (3072, 12288),
+                            "adaln": (18432, 3072)}}
+    if i == 4:   # stochastic LoRA merge, then a skinny GEMM
+        w = torch.randn(12288, 3072, generator=g) * 0.02
+        down = torch.randn(32, 3072, generator=g) * 0.01
+        up = torch.randn(12288, 32, generator=g) * 0.01
+        noise = torch.rand(12288, 3072, generator=g)
+        x = _acts(g, 256, 3072, 0.01, 20.0)
+        return {"w": w, "up": up, "down": down, "alpha": 32.0, "noise": noise, "x": x}
+    raise ValueError(i)
+
+
+# --------------------------------------------------------------------------- timing helpers
+def _events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_kernel(fn, iters=50, warmup=5, sets=1):
+    """Median / min / mean device time of fn(set_index) in microseconds, from HIP events on the
+    launch stream.  `sets` distinct argument sets are cycled so that a bandwidth kernel does not
+    find its operands in the 256 MB memory-side cache."""
+    for i in range(warmup):
+        fn(i % sets)
+    torch.cuda.synchronize()
+    starts, stops = _events(iters), _events(iters)
+    for i in range(iters):
+        starts[i].record()
+        fn(i % sets)
+        stops[i].record()
+    torch.cuda.synchronize()
+    us = [s.elapsed_time(e) * 1e3 for s, e in zip(starts, stops)]
+    return {"median_us": statistics.median(us), "min_us": min(us), "mean_us": statistics.fmean(us)}
+
+
+# --------------------------------------------------------------------------- the step
+class MlpStep:
+    """Config 1 resident on the device."""
+
+    def __init__(self, L, dev):
+        c = make_config(1)
+        self.L = L
+        self.x = c["x"].to(dev)
+        self.h = c["h"].to(dev)
+        self.wq_up, self.ws_up = L.quant_rowwise(c["w_up"].to(dev))
+        self.wq_dn, self.ws_dn = L.quant_rowwise(c["w_dn"].to(dev))
+        self.b_up, self.b_dn = c["b_up"].to(dev), c["b_dn"].to(dev)
+        M = self.x.shape[0]
+        self.y_up = torch.empty(M, 12288, dtype=torch.bfloat16, device=dev)
+        self.y_dn = torch.empty(M, 3072, dtype=torch.bfloat16, device=dev)
+        self.gemm_ops = 2 * M * 12288 * 3072   # per GEMM launch; both GEMMs of the step have this many
+        self.quant_bytes = M * 3072 * 3 + 4 * M + M * 12288 * 3 + 4 * M
+
+    def run(self, ev=None):
+        L = self.L
+        q, s = L.quant_rowwise(self.x)
+        if ev:
+            ev[0].record()
+        L.linear_w8a8(q, s, self.wq_up, self.ws_up, self.b_up, torch.bfloat16, L.EPI_TORCH, self.y_up)
+        if ev:
+            ev[1].record()
+        q2, s2 = L.quant_rowwise(self.h)
+        if ev:
+            ev[2].record()
+        L.linear_w8a8(q2, s2, self.wq_dn, self.ws_dn, self.b_dn, torch.bfloat16, L.EPI_TORCH, self.y_dn)
+        if ev:
+            ev[3].record()
+
+
+# --------------------------------------------------------------------------- extras
+def extras(L, dev, quick=False):
+    out = {}
+    iters = 20 if quick else 100
+    g = torch.Generator().manual_seed(99)
+
+    # north-star target shape: M=4608, K=N=3072, W8A8 rowwise
+    M, N, K = 4608, 3072, 3072
+    x = _acts(g, M, K, 0.01, 20.0).to(dev)
+    wq, ws = L.quant_rowwise((torch.randn(N, K, generator=g) * 0.02).to(dev))
+    q, s = L.quant_rowwise(x)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    t = time_kernel(lambda i: L.linear_w8a8(q, s, wq, ws, None, torch.bfloat16, L.EPI_TORCH, y), iters)
+    tops = 2 * M * N * K / t["median_us"] / 1e6
+    out["target_gemm_4608x3072x3072"] = {"median_us": round(t["median_us"], 2), "min_us": round(t["min_us"], 2),
+                                          "tops": round(tops, 1), "frac_of_int8_peak": round(tops / PEAK_INT8_TOPS, 4)}
+
+    # fused rotate + quant at the same shape, cycling 8 buffer sets (> 256 MB in total)
+    sets = 8
+    xs = [x] + [_acts(g, M, K, 0.01, 20.0).to(dev) for _ in range(sets - 1)]
+    qs = [torch.empty(M, K, dtype=torch.int8, device=dev) for _ in range(sets)]
+    ss = [torch.empty(M, 1, dtype=torch.float32, device=dev) for _ in range(sets)]
+    lib, ptr, stream = L.lib(), L._ptr, L._stream(x)
+    qbytes = M * K * 3 + 4 * M
+    for name, rb in (("quant_4608x3072", 0), ("rotate_quant_4608x3072", 128)):
+        def call(i, rb=rb):
+            rc = lib.i8f_quant_rowwise(ptr(xs[i]), L.BF16, M, K, K, rb, ptr(qs[i]), ptr(ss[i]), stream)
+            assert rc == 0, rc
+        t = time_kernel(call, iters, sets=sets)
+        gbs = qbytes / t["median_us"] / 1e3
+        out[name] = {"median_us": round(t["median_us"], 2), "min_us": round(t["min_us"], 2), "gbs": round(gbs, 1),
+                     "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4), "bytes": qbytes, "buffer_sets": sets}
+    del xs, qs, ss
+
+    # config 4: stochastic LoRA merge (rank 32 rebuilt in the kernel, float noise) and the skinny GEMM
+    c = make_config(4)
+    w4q, w4s = L.quant_rowwise(c["w"].to(dev))
+    up, down = c["up"].to(dev), c["down"].to(dev)
+    Nw, Kw, r = 12288, 3072, 32
+    noises = [c["noise"].to(dev)] + [torch.rand(Nw, Kw, device=dev) for _ in range(2)]
+    outs = [torch.empty_like(w4q) for _ in range(3)]
+    mbytes = Nw * Kw * 6 + 4 * Nw + 4 * r * (Nw + Kw)
+    t = time_kernel(lambda i: L.lora_merge_sr(w4q, w4s, noises[i], up=up, down=down, lora_scale=1.0, out=outs[i]),
+                    max(10, iters // 4), sets=3)
+    gbs = mbytes / t["median_us"] / 1e3
+    out["lora_merge_fused_12288x3072_r32"] = {"median_us": round(t["median_us"], 2), "gbs": round(gbs, 1),
+                                              "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4), "bytes": mbytes}
+    x4 = c["x"].to(dev)
+    q4, s4 = L.quant_rowwise(x4)
+    y4 = torch.empty(256, Nw, dtype=torch.bfloat16, device=dev)
+    t = time_kernel(lambda i: L.linear_w8a8(q4, s4, outs[0], w4s, None, torch.bfloat16, L.EPI_TORCH, y4), iters)
+    out["skinny_gemm_256x12288x3072"] = {"median_us": round(t["median_us"], 2),
+                                         "tops": round(2 * 256 * Nw * Kw / t["median_us"] / 1e6, 1)}
+    del noises, outs
+
+    # config 3: the linears of one double-stream DiT block (attention stays bf16 and is not counted)
+    c3 = make_config(3)
+    lin = {}
+    for name, (n_out, k_in) in c3["linears"].items():
+        wq_, ws_ = L.quant_rowwise(torch.randn(n_out, k_in, device=dev) * 0.02)
+        lin[name] = (wq_, ws_, (torch.randn(n_out, device=dev) * 0.01).bfloat16())
+    acts = {m: {k: torch.randn(m, k, device=dev).bfloat16() for k in (3072, 12288)} for m in (4096, 512)}
+    vec = torch.randn(1, 3072, device=dev).bfloat16()
+    bufs = {(m, n): torch.empty(m, n, dtype=torch.bfloat16, device=dev) for m in (4096, 512) for n in (9216, 3072, 12288)}
+
+    def block(_i):
+        for m in (4096, 512):   # image stream, text stream
+            L.linear_w8a16_small_m(vec, lin["adaln"][0], lin["adaln"][1], lin["adaln"][2])
+            for name, k in (("qkv", 3072), ("proj", 3072), ("up", 3072), ("down", 12288)):
+                wq_, ws_, b_ = lin[name]
+                q_, s_ = L.quant_rowwise(acts[m][k])
+                L.linear_w8a8(q_, s_, wq_, ws_, b_, torch.bfloat16, L.EPI_TORCH, bufs[(m, wq_.shape[0])])
+
+    t = time_kernel(block, max(10, iters // 4))
+    ops = sum(2 * m * n * k for m in (4096, 512) for (n, k) in [c3["linears"][x] for x in ("qkv", "proj", "up", "down")])
+    out["dit_block_linears"] = {"ms": round(t["median_us"] / 1e3, 4), "gemm_gop": round(ops / 1e9, 1),
+                                "tops": round(ops / t["median_us"] / 1e6, 1),
+                                "note": "8 W8A8 linears (quantise + GEMM) and 2 adaLN W8A16 linears at M=1; attention not included"}
+    return out
+
+
+# --------------------------------------------------------------------------- CPU baseline
+def cpu_baseline(reps=3):
+    """The reference's torch CPU path on config 1.  A 512-row probe sizes the sample: the whole
+    workload (4608 rows) if that takes under about 10 s per run on this host, else the probe itself."""
+    from oracle import torch_path as T
+
+    def run(c, wq_up, ws_up, wq_dn, ws_dn):
+        t0 = time.perf_counter()
+        T.linear_w8a8(c["x"], wq_up, ws_up, c["b_up"], torch.bfloat16)
+        T.linear_w8a8(c["h"], wq_dn, ws_dn, c["b_dn"], torch.bfloat16)
+        return time.perf_counter() - t0
+
+    full = make_config(1)
+    wq_up, ws_up = T.quant_rowwise(full["w_up"])
+    wq_dn, ws_dn = T.quant_rowwise(full["w_dn"])
+    probe = {"x": full["x"][:512], "h": full["h"][:512], "b_up": full["b_up"], "b_dn": full["b_dn"]}
+    run(probe, wq_up, ws_up, wq_dn, ws_dn)
+    t_probe = run(probe, wq_up, ws_up, wq_dn, ws_dn)
+    rows, c = (4608, full) if t_probe * 9 < 10.0 else (512, probe)
+    t = statistics.median(run(c, wq_up, ws_up, wq_dn, ws_dn) for _ in range(reps))
+    ops = 2 * 2 * rows * 12288 * 3072
+    what = "all 4608 token rows" if rows == 4608 else "first 512 of 4608 token rows"
+    return {"value": round(ops / t / 1e12, 4), "unit": "TOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{what} of config 1 (quantise + int8 matmul + dequant for both projections, full K and N), "
+                      f"torch CPU restatement of the reference's slow path, median of {reps} runs, {t:.3f} s per run"}
+
+
+# --------------------------------------------------------------------------- main
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--quick", action="store_true", help="fewer iterations in the extra measurements")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one GPU: the INT8 linear path has no multi-GPU part (run with --gpus 1)")
+
+    import __graft_entry__ as ge
+
+    pkg = ge.load_package()
+    L = pkg._lib
+    L.lib()   # fails loudly if the HIP library is not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    step = MlpStep(L, dev)
+    for _ in range(a.warmup):
+        step.run()
+    torch.cuda.synchronize()
+    evs = [_events(4) for _ in range(a.steps)]
+    t0 = time.perf_counter()
+    for k in range(a.steps):
+        step.run(evs[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    gemm_us = [e[0].elapsed_time(e[1]) * 1e3 for e in evs] + [e[2].elapsed_time(e[3]) * 1e3 for e in evs]
+    avg_gemm_us = statistics.fmean(gemm_us)
+    achieved = step.gemm_ops / avg_gemm_us / 1e6
+    ms_per_step = wall / a.steps * 1e3
+    value = 2 * step.gemm_ops / (ms_per_step * 1e-3) / 1e12
+
+    line = {
+        "metric": "INT8 GEMM TOPS (% of int8 MFMA peak) + ms per Flux-style DiT block, 1 GPU",
+        "value": round(value, 1),
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 1: Flux MLP W8A8 rowwise, M=4608, 3072->12288->3072, bf16 in/out, bias; "
+                               "quantise + GEMM for both projections, inputs resident in HBM"},
+        "pct_of_int8_peak": round(100 * value / PEAK_INT8_TOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": None,
+                     "kernel": "gemm_i8_kernel (int8 MFMA GEMM + dequant epilogue)",
+                     "ops_per_launch": step.gemm_ops, "avg_launch_us": round(avg_gemm_us, 2),
+                     "launches_timed": len(gemm_us)},
+    }
+    if not a.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    if not a.no_extras:
+        line["extras"] = extras(L, dev, quick=a.quick)
+        if "dit_block_linears" in line["extras"]:
+            line["dit_block_ms"] = line["extras"]["dit_block_linears"]["ms"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,59 @@
+"""Fused W8A8 linear pipeline on the HIP library.
+
+Same entry points as the reference's int8_fused_kernel.py, which launches Triton
+kernels; here each call goes through the C ABI of libi8f_gfx950.so:
+
+    hip_quantize_rowwise      <- triton_quantize_rowwise      (int8_fused_kernel.py:55-73)
+    hip_int8_linear           <- triton_int8_linear           (int8_fused_kernel.py:179-235)
+    hip_int8_linear_per_row   <- triton_int8_linear_per_row   (int8_fused_kernel.py:330-372)
+
+The triton_* names are kept as aliases so that callers written against the
+reference keep working.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import EPI_FUSED, EPI_TORCH  # noqa: F401  (re-exported)
+
+# Order of the epilogue's float operations used by the wrappers below.  EPI_TORCH
+# reproduces the reference's torch path bit for bit; EPI_FUSED is the single-rounding
+# order of the reference's Triton kernels.
+DEFAULT_EPILOGUE = EPI_TORCH
+
+
+def hip_quantize_rowwise(x: torch.Tensor, rotate: bool = False):
+    """[rows, cols] float -> (int8 [rows, cols], float32 [rows, 1]) per-row absmax quantisation;
+    rotate=True applies the online QuaRot rotation in the same pass."""
+    if x.dim() != 2:
+        raise ValueError(f"expected a 2-D tensor, got shape {tuple(x.shape)}")
+    return _lib.quant_rowwise(x, rotate=rotate)
+
+
+def _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order):
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    q, s = _lib.quant_rowwise(x2, rotate=rotate)
+    y = _lib.linear_w8a8(q, s, weight, weight_scale, bias, compute_dtype, DEFAULT_EPILOGUE if order is None else order)
+    return y.reshape(*lead, weight.shape[0])
+
+
+def hip_int8_linear(x, weight, weight_scale, bias=None, compute_dtype=torch.float16, rotate=False, order=None):
+    """W8A8 linear with ONE weight scale (Python float or 1-element tensor)."""
+    if isinstance(weight_scale, torch.Tensor) and weight_scale.numel() != 1:
+        # the reference's kernel reads element 0 only (int8_fused_kernel.py:153)
+        weight_scale = weight_scale.reshape(-1)[:1]
+    return _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order)
+
+
+def hip_int8_linear_per_row(x, weight, weight_scale, bias=None, compute_dtype=torch.float16, rotate=False, order=None):
+    """W8A8 linear with one weight scale per output row ([N,1] or [N] float32 tensor)."""
+    if not isinstance(weight_scale, torch.Tensor) or weight_scale.numel() != weight.shape[0]:
+        raise ValueError("per-row weight scale must be a tensor with one element per weight row")
+    return _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order)
+
+
+triton_quantize_rowwise = hip_quantize_rowwise
+triton_int8_linear = hip_int8_linear
+triton_int8_linear_per_row = hip_int8_linear_per_row

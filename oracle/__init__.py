@@ -167,7 +167,7 @@ def rotate(x, dtype_code, block=128):
     M, K = x.shape
     if K % block:
         raise ValueError("K must be a multiple of the block")
-    v = np.ascontiguousarray(to_f32(x, dtype_code))
+    v = np.array(to_f32(x, dtype_code), dtype=np.float32, order="C", copy=True)
     for m in range(M):
         row = v[m]
         lib().orc_rotate_row(_p(row), K, dtype_code, block)

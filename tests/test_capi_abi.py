@@ -1,0 +1,95 @@
+"""The C ABI: the library loads, exports everything include/i8f.h declares, and rejects bad
+arguments on the host before anything is launched (so these run without a GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "i8f.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(i8f_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points(L):
+    names = declared_functions()
+    assert set(names) == set(L.EXPORTS)
+    assert len(names) == 10
+
+
+def test_library_exports_every_declared_symbol(L):
+    lib = L.lib()
+    for name in declared_functions():
+        assert getattr(lib, name) is not None
+
+
+def test_version_and_status_strings(L):
+    lib = L.lib()
+    header = open(os.path.join(ROOT, "include", "i8f.h")).read()
+    assert lib.i8f_version() == int(re.search(r"#define I8F_VERSION (\d+)", header).group(1))
+    assert lib.i8f_status_string(0) == b"ok"
+    for code in (-1, -2, -3, -4):
+        assert lib.i8f_status_string(code) not in (b"ok", b"unknown status")
+    assert lib.i8f_status_string(-99) == b"unknown status"
+    assert lib.i8f_last_hip_error() == 0
+
+
+def test_bad_arguments_are_rejected_before_any_launch(L):
+    lib = L.lib()
+    null = ctypes.c_void_p(None)
+    one = ctypes.c_void_p(16)   # never dereferenced: validation fails first
+    INVALID, UNSUPPORTED = -1, -2
+    # negative sizes, bad dtype, bad rotate block, rotation with K not a multiple of 128
+    assert lib.i8f_quant_rowwise(one, L.BF16, -1, 8, 8, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise(one, 7, 4, 8, 8, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise(one, L.BF16, 4, 256, 256, 64, one, one, null) == UNSUPPORTED
+    assert lib.i8f_quant_rowwise(one, L.BF16, 4, 200, 200, 128, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise(one, L.BF16, 4, 256, 128, 0, one, one, null) == INVALID     # ldx < K
+    assert lib.i8f_quant_rowwise(null, L.BF16, 4, 256, 256, 0, one, one, null) == INVALID    # NULL input
+    assert lib.i8f_quant_rowwise(null, L.BF16, 0, 256, 256, 0, null, null, null) == 0        # empty: nothing to do
+    assert lib.i8f_rotate128(one, L.F32, 4, 100, 100, one, null) == INVALID
+    assert lib.i8f_gemm_i32(one, one, -1, 4, 4, one, null) == INVALID
+    assert lib.i8f_gemm_i32(null, one, 4, 4, 4, one, null) == INVALID
+    assert lib.i8f_gemm_i32(null, null, 0, 4, 4, null, null) == 0
+    assert lib.i8f_linear_w8a8(one, one, one, null, 1.0, L.SCALE_ROW, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID  # row scales missing
+    assert lib.i8f_linear_w8a8(one, one, one, one, 1.0, 5, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID             # bad scale mode
+    assert lib.i8f_linear_w8a8(one, one, one, one, 1.0, 0, null, 0, one, L.BF16, 4, 4, 4, 9, null) == INVALID             # bad epilogue order
+    assert lib.i8f_linear_w8a8(one, null, one, one, 1.0, 0, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID            # activation scales missing
+    assert lib.i8f_linear_w8a16_small_m(one, L.BF16, 17, 8, 8, one, one, 1.0, 0, null, 0, one, 4, null) == UNSUPPORTED    # M > 16
+    assert lib.i8f_sr_quant_delta(null, one, 1.0, 0, one, 4, 4, one, null) == INVALID
+    assert lib.i8f_lora_merge_sr(one, one, 1.0, 0, null, null, null, 8, 1.0, one, 4, 4, one, null) == INVALID             # neither delta nor factors
+    assert lib.i8f_lora_merge_sr(one, one, 1.0, 0, null, one, one, 300, 1.0, one, 4, 4, one, null) == UNSUPPORTED         # rank > 256
+
+
+def test_missing_library_is_a_loud_error(pkg, monkeypatch, tmp_path):
+    monkeypatch.setattr(pkg._lib, "_lib", None)
+    monkeypatch.setattr(pkg._lib, "LIB_PATH", str(tmp_path / "libi8f_gfx950.so"))
+    with pytest.raises(RuntimeError, match="is missing"):
+        pkg._lib.lib()
+
+
+def test_cpu_tensors_are_refused_not_emulated(pkg):
+    import torch
+
+    x = torch.randn(32, 128).bfloat16()
+    w = torch.zeros(16, 128, dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        pkg.hip_quantize_rowwise(x)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        pkg.int8_forward_dynamic(x, w, 0.01, None, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        pkg._lib.gemm_i32(w, w)
+
+
+def test_product_code_never_imports_the_oracle():
+    pkg_dir = os.path.join(ROOT, "comfyui-int8-fast_amd")
+    for dirpath, _, files in os.walk(pkg_dir):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+                assert "_int_mm(" not in text, f"{f} calls torch._int_mm"

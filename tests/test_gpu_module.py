@@ -1,0 +1,169 @@
+"""The ComfyUI-facing layer on the GPU: Int8TensorwiseOps.Linear and the INT8 LoRA adapters
+produce what the oracle computes from the same inputs."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+G = torch.Generator().manual_seed(777)
+
+
+@pytest.fixture(autouse=True)
+def reset_flags(pkg):
+    ops = pkg.Int8TensorwiseOps
+    saved = (list(ops.excluded_names), ops.dynamic_quantize, ops.enable_quarot)
+    yield
+    ops.excluded_names, ops.dynamic_quantize, ops.enable_quarot = saved
+
+
+def load(layer, sd, prefix="l."):
+    layer._load_from_state_dict(dict(sd), prefix, {}, True, [], [], [])
+    return layer
+
+
+def bits(t):
+    return O.from_torch(t.cpu())[0]
+
+
+@pytest.mark.parametrize("quarot", [False, True])
+def test_on_the_fly_quantised_linear_forward(pkg, dev, quarot):
+    ops = pkg.Int8TensorwiseOps
+    ops.dynamic_quantize, ops.enable_quarot = True, quarot
+    w = (torch.randn(384, 512, generator=G) * 0.02).bfloat16()
+    b = (torch.randn(384, generator=G) * 0.01).bfloat16()
+    lin = load(ops.Linear(512, 384, bias=True), {"l.weight": w, "l.bias": b})
+    rb = 128 if quarot else 0
+    wq, ws = O.quant_rowwise(w.float().numpy(), O.F32, rb)          # the loader widens to float32 first
+    assert lin._is_quantized and lin._is_per_row and lin._use_quarot == quarot
+    assert lin.weight.device.type == "cpu" and np.array_equal(lin.weight.numpy(), wq) and np.array_equal(lin.weight_scale.numpy(), ws)
+
+    x = torch.randn(2, 40, 512, generator=G)
+    x[..., 5] *= 30
+    x = x.bfloat16()
+    y = lin(x.to(dev))
+    assert y.shape == (2, 40, 384) and y.dtype == torch.bfloat16
+    xa, code = O.from_torch(x.reshape(80, 512))
+    want = O.linear_w8a8(xa, code, wq, ws, O.from_torch(b)[0], O.BF16, O.BF16, rb)
+    assert np.array_equal(bits(y.reshape(80, 384)), want)
+
+    # fp32 activations are computed and returned in bf16; fp16 activations in fp16
+    y32 = lin(x.float().to(dev))
+    assert y32.dtype == torch.bfloat16
+    xa32, _ = O.from_torch(x.float().reshape(80, 512))
+    assert np.array_equal(bits(y32.reshape(80, 384)), O.linear_w8a8(xa32, O.F32, wq, ws, O.from_torch(b)[0], O.BF16, O.BF16, rb))
+    y16 = lin(x.half().to(dev))
+    assert y16.dtype == torch.float16
+
+    # 16 rows or fewer: W8A16 path, output in x's dtype, within the small-batch tolerance
+    xs = x[0, :9]
+    ys = lin(xs.to(dev))
+    xin = O.rotate(O.from_torch(xs)[0], O.BF16) if quarot else O.from_torch(xs)[0]
+    ref = O.to_f32(O.linear_w8a16(xin, O.BF16, wq, ws, O.from_torch(b)[0], O.BF16), O.BF16)
+    got = ys.float().cpu().numpy()
+    assert ys.shape == (9, 384) and (np.abs(got - ref) <= 2.0**-7 * np.abs(ref) + 2.0**-8 * np.abs(ref).max()).all()
+
+
+def test_prequantised_tensorwise_linear_forward(pkg, dev):
+    wf = torch.randn(256, 384, generator=G) * 0.02
+    wq, ws = O.quant_tensorwise(wf.numpy(), O.F32)
+    lin = load(pkg.Int8TensorwiseOps.Linear(384, 256, bias=False),
+               {"l.weight": torch.from_numpy(wq), "l.weight_scale": torch.tensor(float(ws[0]))})
+    x = torch.randn(33, 384, generator=G).bfloat16()
+    y = lin.to(dev)(x.to(dev))
+    xa, code = O.from_torch(x)
+    assert np.array_equal(bits(y), O.linear_w8a8(xa, code, wq, ws))
+
+
+def test_dynamic_lora_side_branch(pkg, dev):
+    wq = torch.randint(-128, 128, (64, 128), dtype=torch.int8, generator=G)
+    lin = load(pkg.Int8TensorwiseOps.Linear(128, 64, bias=False), {"l.weight": wq, "l.weight_scale": torch.rand(64, 1) * 0.01}).to(dev)
+    x = torch.randn(20, 128, generator=G).bfloat16().to(dev)
+    base = lin(x)
+    lin.lora_A, lin.lora_B = torch.randn(4, 128, generator=G).bfloat16(), torch.randn(64, 4, generator=G).bfloat16()
+    withl = lin(x)
+    side = torch.nn.functional.linear(torch.nn.functional.linear(x, lin.lora_A.to(dev)), lin.lora_B.to(dev))
+    assert torch.equal(withl, base + side.to(base.dtype))
+
+
+def test_set_weight_requantises_a_float_patch_with_the_layers_scale(pkg, dev):
+    wq = torch.randint(-100, 100, (32, 64), dtype=torch.int8, generator=G)
+    ws = torch.rand(32, 1, generator=G) * 0.01 + 0.001
+    lin = load(pkg.Int8TensorwiseOps.Linear(64, 32, bias=False), {"l.weight": wq, "l.weight_scale": ws})
+    patched = wq.float() * ws + 0.0004                                 # what a float fallback would hand over
+    noise = torch.rand(32, 64, generator=G)
+    want = O.sr_delta(patched.numpy(), ws.numpy(), noise.numpy())
+    got = pkg.stochastic_round_int8_delta(patched.to(dev), ws, noise=noise)
+    assert np.array_equal(got.cpu().numpy(), want)
+    out = lin.set_weight(patched, seed=3, return_weight=True)           # device-drawn noise: check the bracket only
+    assert out.dtype == torch.int8 and out.device.type == "cpu"
+    xs = patched / ws
+    assert ((out.float() - torch.floor(xs)).abs() <= 1).all()
+
+
+@pytest.mark.parametrize("quarot", [False, True])
+@pytest.mark.parametrize("fused", [True, False])
+def test_lora_patch_adapter_merges_like_the_oracle(pkg, dev, quarot, fused):
+    ops = pkg.Int8TensorwiseOps
+    ops.enable_quarot = quarot
+    N, K, r = 192, 256, 8
+    wq = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=G)
+    ws = torch.rand(N, 1, generator=G) * 0.002 + 0.0005
+    up, down = torch.randn(N, r, generator=G) * 0.05, torch.randn(r, K, generator=G) * 0.05
+    ad = pkg.INT8LoRAPatchAdapter({"k"}, (up, down, 4.0, None, None, None), ws, seed=318008)
+    ad.fuse_low_rank = fused
+    out = ad.calculate_weight(wq, "k", 0.8, 1.0, None, None)
+    assert out.dtype == torch.int8 and out.device == wq.device and out.shape == wq.shape
+    noise = pkg.int8_quant._draw_noise((N, K), 318008, dev).cpu()      # the adapter's own draw
+    mult = (4.0 / r) * 0.8
+    if fused:
+        dn = O.rotate(down.numpy(), O.F32) if quarot else down.numpy()
+        want = O.lora_merge_sr(wq.numpy(), ws.numpy(), noise.numpy(), up=up.numpy(), down=dn, lora_scale=mult)
+        assert np.array_equal(out.numpy(), want)
+    else:   # delta comes from a device BLAS product: compare against the oracle fed with that very delta
+        delta = (torch.mm(up.to(dev), down.to(dev)) * mult).cpu()
+        if quarot:
+            delta = torch.from_numpy(O.rotate(delta.numpy(), O.F32))
+        want = O.lora_merge_sr(wq.numpy(), ws.numpy(), noise.numpy(), delta=delta.numpy())
+        assert np.array_equal(out.numpy(), want)
+    # narrowed weight (fused QKV): ComfyUI hands over the slice and its LoRA, the scale is still the full tensor
+    sl = slice(64, 128)
+    ad_q = pkg.INT8LoRAPatchAdapter({"k"}, (up[sl], down, 4.0, None, None, None), ws, seed=318008)
+    ad_ref = pkg.INT8LoRAPatchAdapter({"k"}, (up[sl], down, 4.0, None, None, None), ws[sl], seed=318008)
+    ad_q.fuse_low_rank = ad_ref.fuse_low_rank = fused
+    part = ad_q.calculate_weight(wq[sl].contiguous(), "k", 0.8, 1.0, (0, 64, 64), None)
+    assert torch.equal(part, ad_ref.calculate_weight(wq[sl].contiguous(), "k", 0.8, 1.0, None, None))
+    assert not torch.equal(part, wq[sl])
+
+
+def test_merged_adapter_sums_deltas_then_rounds_once(pkg, dev):
+    N, K = 96, 128
+    wq = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=G)
+    ws = torch.rand(N, 1, generator=G) * 0.002 + 0.0005
+    mk = lambda r: (torch.randn(N, r, generator=G) * 0.05, torch.randn(r, K, generator=G) * 0.05, float(r), None, None, None)
+    a1, a2 = pkg.INT8LoRAPatchAdapter({"a"}, mk(4), ws), pkg.INT8LoRAPatchAdapter({"b"}, mk(8), ws)
+    merged = pkg.INT8MergedLoRAPatchAdapter([(a1, 0.5), (a2, -0.25)], ws, seed=11)
+    out = merged.calculate_weight(wq, "k", 1.0, 1.0, None, None)
+    total = (torch.mm(a1.weights[0].to(dev), a1.weights[1].to(dev)) * 0.5)
+    total += torch.mm(a2.weights[0].to(dev), a2.weights[1].to(dev)) * -0.25
+    noise = pkg.int8_quant._draw_noise((N, K), 11, dev).cpu()
+    want = O.lora_merge_sr(wq.numpy(), ws.numpy(), noise.numpy(), delta=total.cpu().numpy())
+    assert np.array_equal(out.numpy(), want)
+    # float weights take the float branch
+    wf = torch.randn(N, K, generator=G)
+    outf = merged.calculate_weight(wf, "k", 1.0, 1.0, None, None)
+    assert outf.dtype == torch.float32 and not torch.equal(outf, wf)
+
+
+def test_quantize_helpers_on_device(pkg, dev):
+    x = (torch.randn(40, 96, generator=G) * 0.02).bfloat16()
+    q, s = pkg.quantize_int8_tensorwise(x.to(dev))
+    qo, so = O.quant_tensorwise(O.from_torch(x)[0], O.BF16)
+    assert s.dim() == 0 and np.array_equal(q.cpu().numpy(), qo) and float(s) == float(so[0])
+    x3 = torch.randn(3, 5, 64, generator=G).to(dev)
+    q3, s3 = pkg.quantize_int8_axiswise(x3, dim=-1)
+    qo3, so3 = O.quant_rowwise(x3.cpu().reshape(15, 64).numpy(), O.F32)
+    assert s3.shape == (3, 5, 1) and np.array_equal(q3.cpu().numpy().reshape(15, 64), qo3)
+    r = pkg.quarot.rotate_activation(x3[..., :128].contiguous() if x3.shape[-1] >= 128 else torch.randn(2, 3, 128, device=dev))
+    assert r.shape[-1] == 128

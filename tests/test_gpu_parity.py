@@ -1,0 +1,300 @@
+"""Parity of the HIP library with the CPU oracle on identical seeded inputs, through the C ABI.
+
+Bars: int8 activations, their scales, int32 accumulators and merged int8 weights are
+bit-exact; bf16/fp16 outputs of the W8A8 linear are bit-exact as well, in BOTH epilogue
+orders (the oracle restates each order operation for operation); the small-batch W8A16
+path, whose reference is a BLAS product of unspecified order, is held to
+|y - y_ref| <= 2^-7 |y_ref| + 2^-8 max|y_ref| for bf16 (2^-10 / 2^-11 for fp16, 1e-5 relative for fp32).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from bench import make_config
+
+pytestmark = pytest.mark.gpu
+
+G = torch.Generator().manual_seed(4321)
+
+
+def acts(M, K, dt=torch.bfloat16, frac=0.01, mul=20.0):
+    x = torch.randn(M, K, generator=G)
+    if K > 8:
+        x[:, torch.randperm(K, generator=G)[: max(1, int(K * frac))]] *= mul
+    return x.to(dt)
+
+
+def i8(*shape):
+    return torch.randint(-128, 128, shape, dtype=torch.int8, generator=G)
+
+
+def bits(t):
+    return O.from_torch(t.cpu())[0]
+
+
+# ------------------------------------------------------------------ quantiser (a1, a3, a4)
+QUANT_CASES = [
+    # M, K, dtype, rotate
+    (64, 3072, torch.bfloat16, False), (64, 3072, torch.bfloat16, True), (33, 3840, torch.bfloat16, True),
+    (17, 12288, torch.bfloat16, False), (9, 12288, torch.bfloat16, True), (5, 18432, torch.bfloat16, False),
+    (16, 1000, torch.bfloat16, False), (7, 1001, torch.bfloat16, False), (3, 77, torch.float16, False), (4, 1, torch.float32, False),
+    (8, 3072, torch.float32, True), (8, 3072, torch.float16, True), (5, 24576, torch.float32, True),
+    (6, 40960, torch.float32, True), (2, 70000, torch.bfloat16, False), (3, 66048, torch.bfloat16, True),
+    (4, 384, torch.bfloat16, True), (1, 128, torch.float32, True), (257, 512, torch.float16, False), (1, 8, torch.bfloat16, False),
+]
+
+
+@pytest.mark.parametrize("M,K,dt,rot", QUANT_CASES)
+def test_quant_rowwise_bit_exact(L, dev, M, K, dt, rot):
+    x = acts(M, K, dt)
+    if M > 2:
+        x[1] = 0                                   # an all-zero row: scale clamps to 1e-30
+    xa, code = O.from_torch(x)
+    qo, so = O.quant_rowwise(xa, code, 128 if rot else 0)
+    q, s = L.quant_rowwise(x.to(dev), rotate=rot)
+    assert np.array_equal(q.cpu().numpy(), qo)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
+def test_quant_rowwise_strided_and_misaligned_views(L, dev):
+    big = acts(40, 1100).to(dev)
+    for view in (big[:, :1024], big[:, 3:1027], big[::2, 8:520], big[5:6, 1:130]):
+        xa, code = O.from_torch(view.cpu())
+        for rot in (False, True) if view.shape[1] % 128 == 0 else (False,):
+            qo, so = O.quant_rowwise(xa, code, 128 if rot else 0)
+            q, s = L.quant_rowwise(view, rotate=rot)
+            assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(s.cpu().numpy(), so)
+
+
+def test_quant_rowwise_empty(L, dev):
+    q, s = L.quant_rowwise(torch.empty(0, 256, dtype=torch.bfloat16, device=dev))
+    assert q.shape == (0, 256) and s.shape == (0, 1)
+    q, s = L.quant_rowwise(torch.empty(5, 0, dtype=torch.bfloat16, device=dev))
+    assert q.shape == (5, 0) and (s.cpu() == 1e-30).all()
+
+
+def test_quant_extreme_magnitudes(L, dev):
+    x = torch.tensor([[1e-38, -2e-38, 0.0, 5e-39], [3e38, -1e38, 1.0, 0.0], [1e-45, 0, 0, 0], [6e4, -6.5e4, 1e-3, 7.0]],
+                     dtype=torch.float32).repeat(1, 32)
+    for dt in (torch.float32, torch.bfloat16):
+        xa, code = O.from_torch(x.to(dt))
+        qo, so = O.quant_rowwise(xa, code)
+        q, s = L.quant_rowwise(x.to(dt).to(dev))
+        assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(s.cpu().numpy(), so)
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+def test_rotate128_bit_exact_and_in_place(L, dev, dt):
+    x = acts(19, 640, dt, 0.02, 50.0)
+    xa, code = O.from_torch(x)
+    want = O.rotate(xa, code)
+    xd = x.to(dev)
+    assert np.array_equal(bits(L.rotate128(xd)), want)
+    assert np.array_equal(bits(L.rotate128(xd[:, 128:512])), O.rotate(np.ascontiguousarray(xa[:, 128:512]), code))
+    L.rotate128(xd, out=xd)
+    assert np.array_equal(bits(xd), want)
+
+
+def test_weight_prep_matches_oracle_for_rotated_rowwise_weights(L, dev):
+    w = torch.randn(96, 3840, generator=G) * 0.02
+    qo, so = O.quant_rowwise(w.numpy(), O.F32, 128)
+    q, s = L.quant_rowwise(w.to(dev), rotate=True)
+    assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(s.cpu().numpy(), so)
+
+
+# ------------------------------------------------------------------ integer product (a5)
+GEMM_CASES = [(256, 256, 64), (256, 256, 3072), (300, 520, 1040), (128, 128, 128), (100, 72, 48), (64, 64, 50),
+              (1, 8, 16), (17, 3072, 3072), (1024, 768, 12288), (513, 1032, 80), (40, 24, 16), (31, 33, 35), (512, 512, 0)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_CASES)
+def test_gemm_i32_bit_exact(L, dev, M, N, K):
+    a, w = i8(M, K), i8(N, K)
+    acc = L.gemm_i32(a.to(dev), w.to(dev))
+    assert np.array_equal(acc.cpu().numpy(), O.gemm_i32(a.numpy(), w.numpy()))
+
+
+def test_gemm_i32_saturating_inputs_at_largest_k(L, dev):
+    K = 12288
+    a = torch.full((64, K), -128, dtype=torch.int8)
+    w = torch.cat([torch.full((32, K), -128, dtype=torch.int8), torch.full((32, K), 127, dtype=torch.int8)])
+    acc = L.gemm_i32(a.to(dev), w.to(dev)).cpu()
+    assert (acc[:, :32] == K * 16384).all() and (acc[:, 32:] == -K * 16256).all()
+
+
+def test_gemm_i32_misaligned_operands_use_the_generic_kernel(L, dev):
+    a, w = i8(70, 161), i8(90, 161)
+    a_d, w_d = a.to(dev), w.to(dev)
+    flat = torch.empty(70 * 160 + 1, dtype=torch.int8, device=dev)
+    a_off = flat[1:].view(70, 160)
+    a_off.copy_(a_d[:, :160])
+    acc = L.gemm_i32(a_off, w_d[:, :160].contiguous())
+    assert np.array_equal(acc.cpu().numpy(), O.gemm_i32(np.ascontiguousarray(a.numpy()[:, :160]), np.ascontiguousarray(w.numpy()[:, :160])))
+
+
+# ------------------------------------------------------------------ fused linear (a6, a7)
+LIN_CASES = [
+    # M, N, K, row, bias dtype or None, out dtype, order
+    (256, 256, 512, True, torch.bfloat16, torch.bfloat16, 0), (300, 520, 1040, False, None, torch.bfloat16, 0),
+    (512, 768, 3072, True, torch.float16, torch.float16, 0), (512, 768, 3072, True, torch.bfloat16, torch.bfloat16, 1),
+    (256, 256, 512, False, torch.bfloat16, torch.float32, 0), (100, 72, 48, True, torch.float32, torch.bfloat16, 0),
+    (17, 3072, 3072, True, torch.bfloat16, torch.bfloat16, 0), (64, 50, 50, True, torch.bfloat16, torch.bfloat16, 0),
+    (1030, 264, 272, False, torch.float32, torch.float16, 1), (40, 24, 16, False, None, torch.float16, 1),
+]
+
+
+@pytest.mark.parametrize("M,N,K,row,bdt,odt,order", LIN_CASES)
+def test_linear_w8a8_bit_exact(L, dev, M, N, K, row, bdt, odt, order):
+    x = acts(M, K)
+    wf = torch.randn(N, K, generator=G) * 0.02
+    wq, ws = O.quant_rowwise(wf.numpy(), O.F32) if row else O.quant_tensorwise(wf.numpy(), O.F32)
+    bias = None if bdt is None else (torch.randn(N, generator=G) * 0.01).to(bdt)
+    xa, code = O.from_torch(x)
+    ocode = {torch.bfloat16: O.BF16, torch.float16: O.F16, torch.float32: O.F32}[odt]
+    ba, bcode = (None, O.BF16) if bias is None else O.from_torch(bias)
+    want = O.linear_w8a8(xa, code, wq, ws, ba, bcode, ocode, 0, order)
+    q, s = L.quant_rowwise(x.to(dev))
+    ws_arg = torch.from_numpy(ws).to(dev) if row else float(ws[0])
+    got = L.linear_w8a8(q, s, torch.from_numpy(wq).to(dev), ws_arg, None if bias is None else bias.to(dev), odt, order)
+    assert np.array_equal(bits(got), want)
+    if not row:   # the scale may also arrive as a one-element device tensor
+        got2 = L.linear_w8a8(q, s, torch.from_numpy(wq).to(dev), torch.from_numpy(ws).to(dev), None if bias is None else bias.to(dev), odt, order)
+        assert np.array_equal(bits(got2), want)
+
+
+def test_linear_accumulator_beyond_2_pow_24_rounds_like_the_oracle(L, dev):
+    K = 4096
+    a = torch.full((32, K), 127, dtype=torch.int8)
+    a[:, ::3] = 126
+    w = torch.full((16, K), 127, dtype=torch.int8)
+    w[:, ::5] = -128
+    xs = np.full(32, 1e-3, dtype=np.float32)
+    ws = np.linspace(1e-4, 2e-4, 16, dtype=np.float32)
+    acc = O.gemm_i32(a.numpy(), w.numpy())
+    assert np.abs(acc).max() > 2**24
+    want = O.epilogue(acc, xs, ws, None, O.BF16, O.F32, O.EPI_TORCH)
+    got = L.linear_w8a8(a.to(dev), torch.from_numpy(xs).to(dev), w.to(dev), torch.from_numpy(ws).to(dev), None, torch.float32, 0)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+# ------------------------------------------------------------------ BASELINE configs at full size
+def _check_rows(L, dev, x, wq_d, ws_d, bias, rows, rotate=False, scalar=None):
+    """Full-size launch, oracle on a row sample (bit-exact), integer checksum over everything."""
+    xd = x.to(dev)
+    q, s = L.quant_rowwise(xd, rotate=rotate)
+    xa, code = O.from_torch(x[rows])
+    qo, so = O.quant_rowwise(xa, code, 128 if rotate else 0)
+    assert np.array_equal(q[rows].cpu().numpy(), qo) and np.array_equal(s[rows].cpu().numpy(), so)
+    acc = L.gemm_i32(q, wq_d)
+    wq = wq_d.cpu().numpy()
+    assert np.array_equal(acc[rows].cpu().numpy(), O.gemm_i32(qo, wq))
+    # checksum of checksums: sum_n acc[m,n] == q[m,:] . sum_n w[n,:]   for EVERY row, in int64
+    col = wq.astype(np.int64).sum(axis=0)
+    assert np.array_equal(acc.sum(dim=1, dtype=torch.int64).cpu().numpy(), q.cpu().numpy().astype(np.int64) @ col)
+    ws_arg = ws_d if scalar is None else scalar
+    y = L.linear_w8a8(q, s, wq_d, ws_arg, None if bias is None else bias.to(dev), torch.bfloat16, 0)
+    ws_np = ws_d.cpu().numpy() if scalar is None else np.float32(scalar)
+    want = O.epilogue(O.gemm_i32(qo, wq), so, ws_np, None if bias is None else O.from_torch(bias)[0], O.BF16, O.BF16)
+    assert np.array_equal(bits(y[rows]), want)
+    return y
+
+
+def test_config0_tensorwise_full_size(L, dev):
+    c = make_config(0)
+    wq, ws = O.quant_tensorwise(O.from_torch(c["w"])[0], O.BF16)
+    rows = torch.randperm(4096, generator=G)[:48].sort().values
+    _check_rows(L, dev, c["x"], torch.from_numpy(wq).to(dev), None, None, rows, scalar=float(ws[0]))
+
+
+def test_config1_flux_mlp_full_size(L, dev):
+    c = make_config(1)
+    rows = torch.randperm(4608, generator=G)[:32].sort().values
+    wq, ws = L.quant_rowwise(c["w_up"].to(dev))
+    qo, so = O.quant_rowwise(c["w_up"][:64].numpy(), O.F32)
+    assert np.array_equal(wq[:64].cpu().numpy(), qo) and np.array_equal(ws[:64].cpu().numpy(), so)
+    _check_rows(L, dev, c["x"], wq, ws, c["b_up"], rows)
+    wq, ws = L.quant_rowwise(c["w_dn"].to(dev))
+    _check_rows(L, dev, c["h"], wq, ws, c["b_dn"], rows[:16])
+
+
+def test_config2_quarot_full_size_and_error_vs_bf16(L, dev):
+    c = make_config(2)
+    x, w = c["x"], c["w"]
+    rows = torch.randperm(4096, generator=G)[:32].sort().values
+    wq_r, ws_r = L.quant_rowwise(w.to(dev), rotate=True)
+    y_rot = _check_rows(L, dev, x, wq_r, ws_r, None, rows, rotate=True).float()
+    wq_p, ws_p = L.quant_rowwise(w.to(dev))
+    q, s = L.quant_rowwise(x.to(dev))
+    y_plain = L.linear_w8a8(q, s, wq_p, ws_p, None, torch.bfloat16, 0).float()
+    ref = (x.to(dev).float() @ w.to(dev).bfloat16().float().T)
+    err_rot = ((y_rot - ref).norm() / ref.norm()).item()
+    err_plain = ((y_plain - ref).norm() / ref.norm()).item()
+    assert err_rot < 0.5 * err_plain and err_rot < 0.03       # the rotation is what makes the outliers quantisable
+
+
+def test_config4_merge_full_size_then_skinny_gemm(L, dev):
+    c = make_config(4)
+    wq, ws = L.quant_rowwise(c["w"].to(dev))
+    noise, up, down = c["noise"], c["up"], c["down"]
+    merged = L.lora_merge_sr(wq, ws, noise.to(dev), up=up.to(dev), down=down.to(dev), lora_scale=c["alpha"] / 32)
+    rows = torch.randperm(12288, generator=G)[:96].sort().values
+    want = O.lora_merge_sr(wq[rows].cpu().numpy(), ws[rows].cpu().numpy(), noise[rows].numpy(),
+                           up=up[rows].numpy(), down=down.numpy(), lora_scale=1.0)
+    assert np.array_equal(merged[rows].cpu().numpy(), want)
+    changed = (merged != wq).float().mean().item()
+    assert 0.05 < changed < 0.95
+    # in place gives the same bytes
+    w2 = wq.clone()
+    L.lora_merge_sr(w2, ws, noise.to(dev), up=up.to(dev), down=down.to(dev), lora_scale=1.0, out=w2)
+    assert torch.equal(w2, merged)
+    # skinny GEMM on the merged weight, M = 256
+    x = c["x"]
+    q, s = L.quant_rowwise(x.to(dev))
+    y = L.linear_w8a8(q, s, merged, ws, None, torch.bfloat16, 0)
+    xa, code = O.from_torch(x)
+    want_y = O.linear_w8a8(xa, code, merged.cpu().numpy(), ws.cpu().numpy())
+    assert np.array_equal(bits(y), want_y)
+
+
+# ------------------------------------------------------------------ small batch W8A16 (a8)
+@pytest.mark.parametrize("M,N,K,dt,rel,absf", [
+    (1, 18432, 3072, torch.bfloat16, 2.0**-7, 2.0**-8), (16, 260, 1024, torch.bfloat16, 2.0**-7, 2.0**-8),
+    (3, 100, 77, torch.float16, 2.0**-10, 2.0**-11), (2, 64, 256, torch.float32, 1e-5, 1e-6), (7, 33, 4096, torch.float16, 2.0**-10, 2.0**-11),
+])
+def test_small_m_w8a16_within_tolerance(L, dev, M, N, K, dt, rel, absf):
+    x = torch.randn(M, K, generator=G).to(dt)
+    wq = i8(N, K)
+    ws = torch.rand(N, generator=G) * 0.01 + 0.001
+    bias = (torch.randn(N, generator=G) * 0.1).to(dt)
+    xa, code = O.from_torch(x)
+    ref = O.to_f32(O.linear_w8a16(xa, code, wq.numpy(), ws.numpy(), O.from_torch(bias)[0], code), code)
+    got = L.linear_w8a16_small_m(x.to(dev), wq.to(dev), ws.to(dev), bias.to(dev)).float().cpu().numpy()
+    assert (np.abs(got - ref) <= rel * np.abs(ref) + absf * np.abs(ref).max()).all()
+    got_t = L.linear_w8a16_small_m(x.to(dev), wq.to(dev), 0.004, None).float().cpu().numpy()
+    ref_t = O.to_f32(O.linear_w8a16(xa, code, wq.numpy(), np.float32(0.004)), code)
+    assert (np.abs(got_t - ref_t) <= rel * np.abs(ref_t) + absf * np.abs(ref_t).max()).all()
+
+
+# ------------------------------------------------------------------ stochastic merge (a9, a10, a11)
+@pytest.mark.parametrize("N,K,r,row", [(256, 1024, 32, True), (100, 77, 8, False), (512, 3072, 32, True), (3, 5, 1, True), (64, 130, 256, False)])
+def test_lora_merge_bit_exact(L, dev, N, K, r, row):
+    w = i8(N, K)
+    ws = torch.rand(N if row else 1, generator=G) * 0.002 + 0.0005
+    up, down = torch.randn(N, r, generator=G) * 0.05, torch.randn(r, K, generator=G) * 0.05
+    noise = torch.rand(N, K, generator=G)
+    delta = O.lora_delta(up.numpy(), down.numpy(), 0.7)
+    ws_arg = ws.to(dev) if row else float(ws[0])
+    fused = L.lora_merge_sr(w.to(dev), ws_arg, noise.to(dev), up=up.to(dev), down=down.to(dev), lora_scale=0.7)
+    given = L.lora_merge_sr(w.to(dev), ws_arg, noise.to(dev), delta=torch.from_numpy(delta).to(dev))
+    dq = L.sr_quant_delta(torch.from_numpy(delta).to(dev), ws_arg, noise.to(dev))
+    assert np.array_equal(fused.cpu().numpy(), O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), up=up.numpy(), down=down.numpy(), lora_scale=0.7))
+    assert np.array_equal(given.cpu().numpy(), O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), delta=delta))
+    assert np.array_equal(dq.cpu().numpy(), O.sr_delta(delta, ws.numpy(), noise.numpy()))
+
+
+def test_sr_special_noise_values(L, dev):
+    x = torch.tensor([[0.5, 0.3, -0.3, 0.26, -0.26, 0.0, 40.0, -40.0]])
+    for noise in (torch.zeros(1, 8), torch.full((1, 8), 1 - 2.0**-24), torch.tensor([[0.0, 0.2, 0.8, 0.04, 0.96, 0.5, 0.5, 0.5]])):
+        got = L.sr_quant_delta(x.to(dev), 0.25, noise.to(dev)).cpu().numpy()
+        assert np.array_equal(got, O.sr_delta(x.numpy(), np.float32(0.25), noise.numpy()))

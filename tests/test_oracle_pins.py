@@ -1,0 +1,400 @@
+"""Pins the CPU oracle (oracle/i8f_oracle.c) before anything is compared with it.
+
+Each oracle function is checked against something that does not share its code:
+the torch CPU routines the reference itself calls (oracle/torch_path.py), exact
+rational arithmetic on tiny inputs, closed forms and invariants of the maths.
+A wrong sign, index, rounding mode or operand order fails at least one of them.
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from oracle import torch_path as T
+
+G = torch.Generator().manual_seed(1234)
+
+
+def randn(*shape, scale=1.0):
+    return torch.randn(*shape, generator=G) * scale
+
+
+def rn_f32(fr: Fraction) -> Fraction:
+    """Correctly rounded (nearest, ties to even) binary32 value of a rational, as a Fraction; normal range only."""
+    if fr == 0:
+        return Fraction(0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    e = 0
+    while a >= 2:
+        a /= 2
+        e += 1
+    while a < 1:
+        a *= 2
+        e -= 1
+    scaled = a * (1 << 23)
+    fl = scaled.numerator // scaled.denominator
+    rem = scaled - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return sign * Fraction(fl, 1 << 23) * (Fraction(2) ** e)
+
+
+def rne_int(fr: Fraction) -> int:
+    fl = fr.numerator // fr.denominator
+    rem = fr - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return fl
+
+
+# ------------------------------------------------------------------ storage conversions
+def test_bf16_widening_all_patterns():
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    want = torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16).float().numpy()
+    got = np.array([O.lib().orc_bf16_to_f32(int(b)) for b in bits[::7]], dtype=np.float32)
+    ok = ~np.isnan(want[::7])   # a signalling NaN is quieted on its way back through the C float return
+    assert np.array_equal(got.view(np.uint32)[ok], want[::7].view(np.uint32)[ok]) and np.isnan(got[~ok]).all()
+    assert np.array_equal(O.to_f32(bits, O.BF16).view(np.uint32), want.view(np.uint32))
+
+
+def test_f16_widening_all_patterns():
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([O.lib().orc_f16_to_f32(int(b)) for b in bits[::5]], dtype=np.float32)
+    ok = ~np.isnan(want[::5])
+    assert np.array_equal(got.view(np.uint32)[ok], want[::5].view(np.uint32)[ok]) and np.isnan(got[~ok]).all()
+
+
+@pytest.mark.parametrize("code,tdt", [(O.BF16, torch.bfloat16), (O.F16, torch.float16)])
+def test_narrowing_matches_torch_cast(code, tdt):
+    v = torch.cat([
+        randn(4000), randn(2000, scale=1e-6), randn(2000, scale=3e4), randn(500, scale=1e-8),
+        torch.tensor([0.0, -0.0, 1.0, 65504.0, 65519.9, 65520.0, 1e38, -1e38, 2.0**-24, 2.0**-25, 3 * 2.0**-25,
+                      float("inf"), -float("inf"), 1.00390625, 1.01171875, 1.005859375]),
+    ])
+    # exact ties of both formats
+    base = randn(500).bfloat16().float() if code == O.BF16 else randn(500).half().float()
+    ulp = (base.abs() * 2.0**-8) if code == O.BF16 else (base.abs() * 2.0**-11)
+    v = torch.cat([v, base + ulp])
+    want = v.to(tdt).view(torch.int16).numpy().view(np.uint16)
+    fn = O.lib().orc_f32_to_bf16 if code == O.BF16 else O.lib().orc_f32_to_f16
+    got = np.array([fn(float(t)) for t in v.numpy()], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    assert np.array_equal(O.round_to(v.numpy(), code), want)
+
+
+# ------------------------------------------------------------------ a1: row quantiser
+@pytest.mark.parametrize("tdt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(37, 512), (5, 3072), (3, 77), (1, 1)])
+def test_quant_rowwise_equals_torch_ops(tdt, shape):
+    x = randn(*shape)
+    x[:, :: max(1, shape[1] // 7)] *= 20
+    x = x.to(tdt)
+    xa, code = O.from_torch(x)
+    q, s = O.quant_rowwise(xa, code)
+    qt, st = T.quant_rowwise(x)
+    assert np.array_equal(q, qt.numpy())
+    assert np.array_equal(s.view(np.uint32), st.numpy().view(np.uint32))
+
+
+def test_quant_rowwise_exact_rational_bruteforce():
+    x = randn(6, 9).bfloat16()
+    xa, code = O.from_torch(x)
+    q, s = O.quant_rowwise(xa, code)
+    for m in range(6):
+        vals = [Fraction(float(v)) for v in x[m].float()]
+        amax = max(abs(v) for v in vals)
+        sc = rn_f32(amax / 127)
+        inv = rn_f32(1 / sc)
+        assert Fraction(float(s[m, 0])) == sc
+        for k, v in enumerate(vals):
+            assert int(q[m, k]) == max(-128, min(127, rne_int(rn_f32(v * inv))))
+
+
+def test_quant_rowwise_properties():
+    x = randn(64, 256).bfloat16()
+    x[3] = 0
+    x[5, :] = 0
+    x[5, 17] = -3.0
+    xa, code = O.from_torch(x)
+    q, s = O.quant_rowwise(xa, code)
+    assert s[3, 0] == np.float32(1e-30) and not q[3].any()           # zero row: clamp on the scale
+    nz = [m for m in range(64) if m != 3]
+    assert (np.abs(q[nz].astype(np.int32)).max(axis=1) == 127).all()  # the absmax element lands on +-127
+    assert q[5, 17] == -127 and np.count_nonzero(q[5]) == 1
+    err = np.abs(x.float().numpy() - q.astype(np.float32) * s)
+    assert (err <= s * 0.5 + np.abs(x.float().numpy()) * 1e-6).all()  # half a quantisation step
+    # ties go to even: x = (n + 0.5) * scale exactly
+    row = torch.tensor([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5]])
+    q2, s2 = O.quant_rowwise(row.numpy(), O.F32)
+    assert s2[0, 0] == 1.0 and q2.tolist() == [[127, 0, 2, 2, 0, -2, -2, 4]]
+    # idempotence: quantising the dequantised grid returns the same integers
+    deq = (q.astype(np.float32) * s).astype(np.float32)
+    q3, s3 = O.quant_rowwise(deq, O.F32)
+    assert np.array_equal(q3[nz], q[nz])
+
+
+def test_quant_tensorwise_equals_torch_ops():
+    w = (randn(96, 160) * 0.02).bfloat16()
+    wa, code = O.from_torch(w)
+    q, s = O.quant_tensorwise(wa, code)
+    qt, st = T.quant_tensorwise(w)
+    assert np.array_equal(q, qt.numpy()) and s[0] == st.item()
+
+
+# ------------------------------------------------------------------ a3/a4: rotation
+def test_hadamard_entry_constants():
+    for code, tdt in [(O.BF16, torch.bfloat16), (O.F16, torch.float16), (O.F32, torch.float32)]:
+        H = T.hadamard(128, tdt)
+        assert float(H[0, 0].float()) == O.lib().orc_hadamard_entry(code)
+        assert torch.equal(H.abs(), torch.full_like(H, H[0, 0].item()))
+
+
+@pytest.mark.parametrize("n", [2, 8, 128])
+def test_fwht_is_sylvester_hadamard_exactly_on_integers(n):
+    from scipy.linalg import hadamard
+
+    # small integers: every butterfly sum is exact in binary32, so any order gives the dense product exactly
+    v = torch.randint(-512, 513, (n,), generator=G).float().numpy()
+    want = v.astype(np.float64) @ hadamard(n).astype(np.float64)
+    assert np.array_equal(O.fwht(v).astype(np.float64), want)
+    assert np.array_equal(O.fwht(O.fwht(v)), v * n)                  # H H = n I
+    e = np.zeros(n, dtype=np.float32)
+    e[5 % n] = 1
+    assert np.array_equal(O.fwht(e), hadamard(n)[5 % n].astype(np.float32))  # one row of H: fixes the sign pattern
+
+
+def test_fwht_stage_order_is_the_documented_one():
+    # the rounding of binary32 sums depends on the order: restate the butterfly in numpy float32
+    v = (randn(128) * torch.logspace(-3, 3, 128)).numpy().astype(np.float32)
+    w = v.copy()
+    stride = 1
+    while stride < 128:
+        w = w.reshape(-1, 2, stride)
+        lo, hi = w[:, 0, :].copy(), w[:, 1, :].copy()
+        w[:, 0, :], w[:, 1, :] = lo + hi, lo - hi
+        w = w.reshape(-1)
+        stride *= 2
+    assert np.array_equal(O.fwht(v).view(np.uint32), w.view(np.uint32))
+
+
+@pytest.mark.parametrize("code,tdt,tol_ulp", [(O.BF16, torch.bfloat16, 2.0**-8), (O.F16, torch.float16, 2.0**-11),
+                                              (O.F32, torch.float32, 2.0**-22)])
+def test_rotate_close_to_dense_matmul(code, tdt, tol_ulp):
+    x = randn(24, 512)
+    x[:, ::37] *= 50
+    x = x.to(tdt)
+    xa, _ = O.from_torch(x)
+    got = O.to_f32(O.rotate(xa, code), code).astype(np.float64)
+    H = T.hadamard(128, tdt).double().numpy()
+    dense = (x.double().numpy().reshape(24, 4, 128) @ H).reshape(24, 512)   # exact product, float64
+    # error budget: one rounding of the result to the dtype, plus binary32 accumulation error, which is
+    # relative to the sum of the magnitudes (8 adds deep), not to the possibly cancelled result
+    mags = (np.abs(x.double().numpy()).reshape(24, 4, 128) @ np.abs(H)).reshape(24, 512)
+    budget = tol_ulp * np.abs(dense) * 1.01 + 8 * 2.0**-24 * mags
+    assert (np.abs(got - dense) <= budget).all()
+    # and against the library product the reference actually runs (its summation order is BLAS's)
+    lib = T.rotate(x).double().numpy()
+    assert (np.abs(got - lib) <= 2 * tol_ulp * np.abs(dense) * 1.01 + 64 * 2.0**-24 * mags).all()
+
+
+def test_rotated_quantisation_agrees_with_torch_path_statistically():
+    x = randn(64, 3840)
+    x[:, torch.randperm(3840, generator=G)[:77]] *= 50
+    x = x.bfloat16()
+    xa, code = O.from_torch(x)
+    q, s = O.quant_rowwise(xa, code, 128)
+    qt, st = T.quant_rowwise(T.rotate(x))
+    diff = np.abs(q.astype(np.int32) - qt.numpy().astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3              # only summation-order ties differ
+    assert np.allclose(s, st.numpy(), rtol=2.0**-7)                   # scales within one bf16 ulp
+
+
+def test_rotation_is_orthogonal_and_cancels_in_the_product():
+    x, w = randn(16, 256).numpy(), randn(24, 256, scale=0.02).numpy()
+    xr, wr = O.rotate(x, O.F32), O.rotate(w, O.F32)
+    assert np.allclose((xr**2).sum(1), (x**2).sum(1), rtol=1e-5)
+    assert np.allclose(xr @ wr.T, x @ w.T, rtol=1e-4, atol=1e-5)
+    assert np.allclose(O.rotate(xr, O.F32), x, rtol=1e-5, atol=1e-6)  # H is an involution
+
+
+def test_rotation_spreads_outliers():
+    x = randn(32, 1024)
+    x[:, 100] = 50.0
+    xa, code = O.from_torch(x.bfloat16())
+    _, s_plain = O.quant_rowwise(xa, code)
+    _, s_rot = O.quant_rowwise(xa, code, 128)
+    assert (s_rot < s_plain * 0.5).all()
+
+
+# ------------------------------------------------------------------ a5: integer product
+@pytest.mark.parametrize("M,N,K", [(32, 24, 64), (17, 40, 3072), (33, 8, 8), (64, 16, 1000)])
+def test_gemm_i32_equals_int_mm_and_int64(M, N, K):
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=G)
+    w = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=G)
+    acc = O.gemm_i32(a.numpy(), w.numpy())
+    assert np.array_equal(acc, a.numpy().astype(np.int64) @ w.numpy().astype(np.int64).T)
+    if M > 16 and K % 8 == 0 and N % 8 == 0:
+        assert np.array_equal(acc, torch._int_mm(a, w.T).numpy())
+
+
+def test_gemm_i32_extremes_do_not_overflow():
+    K = 12288
+    a = np.full((2, K), -128, dtype=np.int8)
+    w = np.stack([np.full(K, -128, dtype=np.int8), np.full(K, 127, dtype=np.int8)])
+    acc = O.gemm_i32(a, w)
+    assert acc.tolist() == [[K * 16384, -K * 16256]] * 2
+    ident = np.eye(64, dtype=np.int8)
+    b = np.random.default_rng(0).integers(-128, 128, (9, 64), dtype=np.int8)
+    assert np.array_equal(O.gemm_i32(b, ident), b.astype(np.int32))   # a @ I.T = a: operands are not swapped
+    assert O.gemm_i32(np.zeros((3, 0), np.int8), np.zeros((5, 0), np.int8)).tolist() == [[0] * 5] * 3
+
+
+# ------------------------------------------------------------------ a6/a7: epilogue
+def _epi_inputs(M=40, N=56):
+    acc = torch.randint(-2_000_000, 2_000_000, (M, N), dtype=torch.int32, generator=G)
+    acc[0, 0], acc[0, 1] = 2**27 + 5, -(2**27) - 3                    # beyond 2^24: int -> float rounds
+    xs = (torch.rand(M, 1, generator=G) * 0.05 + 1e-3)
+    ws_row = (torch.rand(N, 1, generator=G) * 2e-3 + 1e-4)
+    bias = randn(N, scale=0.3)
+    return acc, xs, ws_row, bias
+
+
+@pytest.mark.parametrize("tdt,code", [(torch.bfloat16, O.BF16), (torch.float16, O.F16)])
+@pytest.mark.parametrize("row", [False, True])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_epilogue_torch_order_equals_torch_ops(tdt, code, row, with_bias):
+    acc, xs, ws_row, bias = _epi_inputs()
+    b = bias.to(tdt) if with_bias else None
+    if row:
+        want = acc.float().mul_(xs).mul_(ws_row.T).to(tdt)
+        ws = ws_row
+    else:
+        ws = 0.00123
+        want = acc.float().mul_(ws * xs).to(tdt)
+    if with_bias:
+        want = want + b.to(tdt)
+    got = O.epilogue(acc.numpy(), xs.numpy(), ws_row.numpy() if row else np.float32(ws),
+                     None if b is None else O.from_torch(b)[0], code, code, O.EPI_TORCH)
+    assert np.array_equal(got, O.from_torch(want)[0])
+
+
+def test_epilogue_float32_bias_is_rounded_to_output_dtype_first():
+    acc, xs, ws_row, bias = _epi_inputs()
+    want = acc.float().mul_(xs).mul_(ws_row.T).to(torch.bfloat16) + bias.to(torch.bfloat16)
+    got = O.epilogue(acc.numpy(), xs.numpy(), ws_row.numpy(), bias.numpy(), O.F32, O.BF16, O.EPI_TORCH)
+    assert np.array_equal(got, O.from_torch(want)[0])
+
+
+@pytest.mark.parametrize("row", [False, True])
+def test_epilogue_fused_order_closed_form(row):
+    acc, xs, ws_row, bias = _epi_inputs()
+    ws = ws_row if row else torch.tensor([[0.00123]])
+    got32 = O.epilogue(acc.numpy(), xs.numpy(), ws.numpy(), bias.numpy(), O.F32, O.F32, O.EPI_FUSED)
+    sc = (xs * ws.T).float()                                          # one rounded product of the scales
+    want32 = (acc.float() * sc + bias).numpy()                        # torch: separate multiply and add
+    assert np.array_equal(got32.view(np.uint32), want32.view(np.uint32))
+    exact = acc.double() * xs.double() * ws.T.double() + bias.double()
+    mag = (acc.double() * xs.double() * ws.T.double()).abs() + bias.double().abs()
+    assert ((torch.from_numpy(got32).double() - exact).abs() <= 4 * 2.0**-24 * mag).all()
+    got16 = O.epilogue(acc.numpy(), xs.numpy(), ws.numpy(), O.from_torch(bias.bfloat16())[0], O.BF16, O.BF16, O.EPI_FUSED)
+    want16 = (acc.float() * sc + bias.bfloat16().float()).bfloat16()
+    assert np.array_equal(got16, O.from_torch(want16)[0])
+
+
+@pytest.mark.parametrize("row", [False, True])
+@pytest.mark.parametrize("rot", [0, 128])
+def test_linear_w8a8_equals_torch_path(row, rot):
+    x = randn(48, 256)
+    x[:, 7] *= 20
+    x = x.bfloat16()
+    wf = randn(40, 256, scale=0.02)
+    wq, ws = (T.quant_rowwise(wf) if row else T.quant_tensorwise(wf))
+    bias = randn(40, scale=0.01).bfloat16()
+    xa, code = O.from_torch(x)
+    got = O.linear_w8a8(xa, code, wq.numpy(), ws.numpy(), O.from_torch(bias)[0], O.BF16, O.BF16, rot)
+    if rot:   # the torch path rotates with a BLAS product: compare from the oracle's own rotated activations on
+        xr = O.to_torch(O.rotate(xa, code), code)
+        want = T.linear_w8a8(xr, wq, ws if row else ws.item(), bias, torch.bfloat16)
+    else:
+        want = T.linear_w8a8(x, wq, ws if row else ws.item(), bias, torch.bfloat16)
+    assert np.array_equal(got, O.from_torch(want)[0])
+
+
+# ------------------------------------------------------------------ a8: small batch W8A16
+@pytest.mark.parametrize("tdt,tol", [(torch.bfloat16, 2.0**-7), (torch.float16, 2.0**-10), (torch.float32, 1e-5)])
+def test_linear_w8a16_within_tolerance_of_f_linear(tdt, tol):
+    x = randn(5, 384).to(tdt)
+    wq = torch.randint(-128, 128, (72, 384), dtype=torch.int8, generator=G)
+    ws = torch.rand(72, 1, generator=G) * 1e-2 + 1e-3
+    bias = randn(72, scale=0.1).to(tdt)
+    want = T.linear_w8a16(x, wq, ws, bias).float().numpy()
+    xa, code = O.from_torch(x)
+    got = O.to_f32(O.linear_w8a16(xa, code, wq.numpy(), ws.numpy(), O.from_torch(bias)[0], code), code)
+    assert (np.abs(got - want) <= tol * np.abs(want) + tol * 0.05).all()
+
+
+# ------------------------------------------------------------------ a9/a10/a11: stochastic merge
+@pytest.mark.parametrize("row", [False, True])
+def test_sr_delta_equals_torch_ops(row):
+    x = randn(64, 96, scale=0.01)
+    x[0, :4] = torch.tensor([1.0, -1.0, 0.5, 3.0])                    # saturation on both sides
+    scale = (torch.rand(64, 1, generator=G) * 1e-3 + 1e-4) if row else 0.00037
+    noise = torch.rand(64, 96, generator=G)
+    want = T.sr_delta(x, scale, noise)
+    got = O.sr_delta(x.numpy(), scale.numpy() if row else np.float32(scale), noise.numpy())
+    assert np.array_equal(got, want.numpy())
+    assert got.min() == -128 and got.max() == 127
+
+
+def test_sr_delta_special_cases():
+    scale = np.float32(0.25)
+    x = np.array([[0.5, 0.3, -0.3, 0.26, -0.26, 0.0, 40.0, -40.0]], dtype=np.float32)   # x/scale = 2, 1.2, -1.2, 1.04, ...
+    zeros, almost1 = np.zeros_like(x), np.full_like(x, 1 - 2.0**-24)
+    assert O.sr_delta(x, scale, zeros).tolist() == [[2, 2, -1, 2, -1, 0, 127, -128]]     # noise 0: up whenever frac > 0, never when frac == 0
+    assert O.sr_delta(x, scale, almost1).tolist() == [[2, 1, -2, 1, -2, 0, 127, -128]]   # noise -> 1: floor
+    # strict compare: noise == frac rounds down
+    assert O.sr_delta(np.array([[0.375]], np.float32), scale, np.array([[0.5]], np.float32)).tolist() == [[1]]
+    # unbiased: the mean over many draws approaches x / scale
+    xs = np.full((1, 200000), 0.3, dtype=np.float32)
+    noise = torch.rand(1, 200000, generator=G).numpy()
+    assert abs(O.sr_delta(xs, scale, noise).astype(np.float64).mean() - 1.2) < 5e-3
+
+
+def test_merge_i8_all_pairs():
+    a = np.arange(-128, 128, dtype=np.int8)
+    w, dq = np.meshgrid(a, a, indexing="ij")
+    got = O.merge_i8(np.ascontiguousarray(w), np.ascontiguousarray(dq))
+    assert np.array_equal(got, np.clip(w.astype(np.int32) + dq.astype(np.int32), -128, 127).astype(np.int8))
+    assert np.array_equal(got, T.merge_i8(torch.from_numpy(np.ascontiguousarray(w)), torch.from_numpy(np.ascontiguousarray(dq))).numpy())
+
+
+def test_lora_delta_fma_chain_exact_and_close_to_mm():
+    up, down = randn(6, 4, scale=0.1), randn(4, 5, scale=0.1)
+    got = O.lora_delta(up.numpy(), down.numpy(), 0.7)
+    s32 = Fraction(float(np.float32(0.7)))
+    for n in range(6):
+        for k in range(5):
+            acc = Fraction(0)
+            for j in range(4):   # fma: one rounding of the exact a*b + c
+                acc = rn_f32(Fraction(float(up[n, j])) * Fraction(float(down[j, k])) + acc)
+            assert Fraction(float(got[n, k])) == rn_f32(acc * s32)
+    up, down = randn(128, 32, scale=0.01), randn(32, 96, scale=0.01)
+    got = O.lora_delta(up.numpy(), down.numpy(), 1.0)
+    assert np.allclose(got, torch.mm(up, down).numpy(), rtol=1e-4, atol=1e-9)
+
+
+def test_lora_merge_composes_the_three_steps():
+    N, K, r = 48, 64, 8
+    w = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=G)
+    ws = torch.rand(N, 1, generator=G) * 1e-3 + 2e-4
+    up, down = randn(N, r, scale=0.05), randn(r, K, scale=0.05)
+    noise = torch.rand(N, K, generator=G)
+    delta = O.lora_delta(up.numpy(), down.numpy(), 0.5)
+    want = T.merge_i8(w, T.sr_delta(torch.from_numpy(delta), ws, noise)).numpy()
+    assert np.array_equal(O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), delta=delta), want)
+    assert np.array_equal(O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), up=up.numpy(), down=down.numpy(), lora_scale=0.5), want)
+    assert (want != w.numpy()).mean() > 0.5
