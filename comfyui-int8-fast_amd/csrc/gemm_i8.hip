@@ -22,7 +22,12 @@
 //     round-robin), so ids are first regrouped per XCD and then walked in
 //     GROUP_M-row panels, which keeps the X and W panels a single XCD touches
 //     small enough for its own L2.
+#include <type_traits>
+
 #include "i8f_common.hpp"
+#ifdef I8F_TRACE
+#include <cstdlib>
+#endif
 
 namespace i8f {
 namespace {
@@ -45,6 +50,9 @@ struct GemmArgs {
     int order;
     void *out;
     int tiles_m, tiles_n;
+#ifdef I8F_TRACE
+    long long *trace;  // [blocks][4] wall-clock stamps: start, first tile landed, loop done, end
+#endif
 };
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_>
@@ -63,14 +71,14 @@ struct Cfg {
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(X_BYTES % (1024 * NW) == 0 && W_BYTES % (1024 * NW) == 0, "tile must split into whole wave loads");
     static_assert(BK == 64 || BK == 128, "BK");
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+    static_assert(LDS_BYTES + 4 * (BM + 2 * BN) <= 160 * 1024, "LDS");
 };
 
 // chunk swizzle: a function of the low 5 bits of the row only
 template <int CPR>
 __device__ __forceinline__ int swz(int r) {
     if constexpr (CPR == 4) return ((r >> 1) & 3) ^ ((r >> 3) & 1);
-    else return (r ^ (r >> 3)) & 7;
+    else return (r ^ ((r >> 3) & 3)) & 7;
 }
 
 __device__ __forceinline__ constexpr int waitcnt_vm(int n) {
@@ -85,16 +93,59 @@ struct OutElem {
     static constexpr int BYTES = (OUT == OUT_BF16 || OUT == OUT_F16) ? 2 : 4;
 };
 
-template <class C, int OUT>
+// One 4-element group of the epilogue, with the operation order, the scale mode and the bias
+// fixed at compile time (a run-time test per value costs more than the arithmetic).
+template <int OUT, int ORDER, bool ROW, bool BIAS>
+__device__ __forceinline__ void epilogue_quad(const int (&a4)[4], float xs, const float4 w4, const float4 b4,
+                                              char *dst) {
+    constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : (OUT == OUT_F16 ? I8F_F16 : I8F_F32);
+    const float wsv[4] = {w4.x, w4.y, w4.z, w4.w};
+    const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
+    float y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float a = (float)a4[e];
+        float t;
+        if constexpr (ORDER == I8F_EPI_TORCH) {
+            if constexpr (ROW) {
+                t = a * xs;
+                t = t * wsv[e];
+            } else {
+                const float sc = wsv[e] * xs;
+                t = a * sc;
+            }
+            t = round_to_dtype<DT>(t);
+            if constexpr (BIAS) t = t + round_to_dtype<DT>(bv[e]);
+        } else {
+            const float sc = xs * wsv[e];
+            t = a * sc;
+            if constexpr (BIAS) t = t + bv[e];
+        }
+        y[e] = t;
+    }
+    if constexpr (OUT == OUT_BF16) {
+        *(uint2 *)dst = make_uint2(f32x2_to_bf16x2_bits(y[0], y[1]), f32x2_to_bf16x2_bits(y[2], y[3]));
+    } else if constexpr (OUT == OUT_F16) {
+        *(uint2 *)dst = make_uint2(f32x2_to_f16x2_bits(y[0], y[1]), f32x2_to_f16x2_bits(y[2], y[3]));
+    } else {
+        *(float4 *)dst = make_float4(y[0], y[1], y[2], y[3]);
+    }
+}
+
+// KTAIL: K is not a multiple of BK (the last tile is ragged); the common case is the other kernel.
+template <class C, int OUT, bool KTAIL>
 __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NI = C::NI, CPR = C::CPR;
     constexpr int S = C::STAGES;
     constexpr int OB = OutElem<OUT>::BYTES;
+    constexpr int KS = BK / 32;  // MFMA k-steps per tile
+    static_assert(KS % 2 == 0, "fragment double-buffering alternates over an even number of k-steps");
     __shared__ __attribute__((aligned(1024))) char smem[C::LDS_BYTES];
+    __shared__ float s_xs[BM], s_ws[BN], s_bias[BN];  // epilogue operands of this tile
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: lets LDS bases live in SGPRs
     const int wm = wave / C::WN, wn = wave % C::WN;
     const int l32 = lane & 31, lhalf = lane >> 5;
 
@@ -116,12 +167,39 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         tile_n = r / gsz;
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+#ifdef I8F_TRACE
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 0] = wall_clock64();
+#endif
+
+    // ---- epilogue operands: fetched once, long before they are needed ----------------------
+    if constexpr (OUT != OUT_I32) {
+        const float ws_one = g.ws ? (g.row_scale ? 0.0f : g.ws[0]) : g.ws_host;
+        for (int t = tid; t < BM; t += C::NT) s_xs[t] = (m0 + t < g.M) ? g.xs[m0 + t] : 0.0f;
+        for (int t = tid; t < BN; t += C::NT) {
+            const int n = n0 + t;
+            float wsv = ws_one, bv = 0.0f;
+            if (n < g.N) {
+                if (g.row_scale) wsv = g.ws[n];
+                if (g.bias) {
+                    if (g.bias_dtype == I8F_F32) bv = ((const float *)g.bias)[n];
+                    else if (g.bias_dtype == I8F_BF16) bv = bf16_bits_to_f32(((const uint16_t *)g.bias)[n]);
+                    else bv = f16_bits_to_f32(((const uint16_t *)g.bias)[n]);
+                }
+            }
+            s_ws[t] = wsv;
+            s_bias[t] = bv;
+        }
+    }
 
     // ---- global -> LDS plan ------------------------------------------------------------
+    // One wave load moves 64 x 16 bytes into 1 KB of LDS (lane l lands at offset 16*l).  The lane
+    // decides WHICH global chunk it fetches, which is where the swizzle is applied.  The byte
+    // offset of the K-tile travels in the scalar offset of the buffer instruction, so issuing a
+    // load costs no vector arithmetic; rows beyond the matrix carry an out-of-range vector offset
+    // and are zero-filled by the buffer bounds check (which looks at the vector offset only).
     const int K = g.K;
     __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)((int64_t)g.M * K), 0x00020000);
     __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)g.w, 0, (int)((int64_t)g.N * K), 0x00020000);
-    const bool k_tail = (K % BK) != 0;
     const uint32_t OOB = 0x7ffffff0u;
 
     uint32_t xoff[C::X_LOADS], woff[C::W_LOADS];  // byte offset of this lane's chunk at k-tile 0
@@ -143,30 +221,41 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         woff[t] = grow < g.N ? (uint32_t)(grow * K + wck[t]) : OOB;
     }
 
-    auto issue = [&](int kt) {
-        char *st = smem + (kt % S) * C::STAGE_BYTES;
+    const int KT = (K + BK - 1) / BK;
+
+    // `live` false (a tile index past the end, at the tail of the loop) turns every lane's offset
+    // out of range: the instruction is still issued, which keeps the loop body free of branches,
+    // but moves no data.
+    auto issue = [&](int kt, bool live) {
+        char *st = smem + (kt % S) * C::STAGE_BYTES + wave * 1024;
         const int kb = kt * BK;
 #pragma unroll
         for (int t = 0; t < C::X_LOADS; ++t) {
-            uint32_t vo = xoff[t] + (uint32_t)kb;
-            if (k_tail && kb + xck[t] >= K) vo = OOB;
-            if (xoff[t] == OOB) vo = OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(st + (t * NW + wave) * 1024), 16, vo, 0, 0, 0);
+            uint32_t vo = live ? xoff[t] : OOB;
+            int so = kb;
+            if constexpr (KTAIL) {  // chunks past K are forced out of range per lane
+                vo = (kb + xck[t] < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
+                so = 0;
+            }
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(st + t * NW * 1024), 16, vo, so, 0, 0);
         }
 #pragma unroll
         for (int t = 0; t < C::W_LOADS; ++t) {
-            uint32_t vo = woff[t] + (uint32_t)kb;
-            if (k_tail && kb + wck[t] >= K) vo = OOB;
-            if (woff[t] == OOB) vo = OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(st + C::X_BYTES + (t * NW + wave) * 1024), 16, vo, 0, 0, 0);
+            uint32_t vo = live ? woff[t] : OOB;
+            int so = kb;
+            if constexpr (KTAIL) {
+                vo = (kb + wck[t] < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
+                so = 0;
+            }
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(st + C::X_BYTES + t * NW * 1024), 16, vo, so, 0, 0);
         }
     };
 
     // ---- LDS -> register plan ----------------------------------------------------------
     const int sw = swz<CPR>(l32);
-    int koff[BK / 32];
+    int koff[KS];
 #pragma unroll
-    for (int ks = 0; ks < BK / 32; ++ks) koff[ks] = ((ks * 2 + lhalf) ^ sw) * 16;
+    for (int ks = 0; ks < KS; ++ks) koff[ks] = ((ks * 2 + lhalf) ^ sw) * 16;
     const int xrow_off = (wm * C::WTM + l32) * BK;
     const int wrow_off = C::X_BYTES + (wn * C::WTN + l32) * BK;
 
@@ -178,124 +267,146 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    const int KT = (K + BK - 1) / BK;
-
-    // ---- prologue: S-1 tiles in flight ---------------------------------------------------
+    auto load_frags = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI]) {
+#ifdef I8F_ABLATE_LDSREAD  // development probe
+        return;
+#endif
 #pragma unroll
-    for (int s = 0; s < S - 1; ++s)
-        if (s < KT) issue(s);
+        for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
+#pragma unroll
+        for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ks]);
+    };
+    auto mma = [&](const v4i (&xf)[MI], const v4i (&wf)[NI]) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#ifndef I8F_ABLATE_MFMA
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+#else
+                acc[i][j][0] += xf[i][0] ^ wf[j][0];
+#endif
+    };
+
+    // ---- prologue: S tiles in flight, fragments of the first k-step in registers --------------
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+        if (s < KT) issue(s, true);
+    if (KT >= S) __builtin_amdgcn_s_waitcnt(waitcnt_vm((S - 1) * C::LOADS));  // tiles 1..S-1 may be in flight
+    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __syncthreads();  // tile 0 and the staged epilogue operands are visible to everyone
+#ifdef I8F_TRACE
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 1] = wall_clock64();
+#endif
+
+    // Fragments are double-buffered in registers: the LDS reads of k-step s+1 are issued before
+    // the MFMAs of k-step s, so the matrix pipe does not wait for LDS.  There is one barrier per
+    // K-tile, in front of its last MFMA group: by then every wave has finished reading tile kt
+    // (its last fragments are in registers), so the stage of tile kt is refilled with tile kt+S
+    // right away, and tile kt+1 is known to have landed, so its first fragments can be fetched.
+    v4i xa[MI] = {}, wa[NI] = {}, xb[MI] = {}, wb[NI] = {};
+    if (KT > 0) load_frags(smem, 0, xa, wa);
+    // Drain scalar loads (kernel arguments) here: a scalar load still pending at the loop header
+    // would turn every LDS wait inside the loop into a full lgkmcnt(0).
+    __builtin_amdgcn_s_waitcnt(0xC07F);
 
     for (int kt = 0; kt < KT; ++kt) {
-        // tile kt must have landed; tiles kt+1 .. kt+S-2 may still be in flight
-        if (kt + S - 2 < KT) __builtin_amdgcn_s_waitcnt(waitcnt_vm((S - 2) * C::LOADS));
-        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-        // A bare barrier: __syncthreads() would add a fence that waits for ALL loads in flight.
-        __builtin_amdgcn_s_barrier();  // everyone's part of tile kt is in LDS; everyone is done reading tile kt-1
-        if (kt + S - 1 < KT) issue(kt + S - 1);  // overwrites the stage tile kt-1 was in
-
         const char *st = smem + (kt % S) * C::STAGE_BYTES;
+        const char *nx = smem + ((kt + 1) % S) * C::STAGE_BYTES;
 #pragma unroll
-        for (int ks = 0; ks < BK / 32; ++ks) {
-            v4i xf[MI], wf[NI];
+        for (int ks = 0; ks < KS; ++ks) {
+            const bool last = ks == KS - 1;
+            if (last) {
+                // my part of tile kt+1 has landed (tiles kt+2 .. kt+S-1 may still be in flight) and
+                // my LDS reads of tile kt have returned
+                if (kt + S - 1 < KT) __builtin_amdgcn_s_waitcnt(waitcnt_vm((S - 2) * C::LOADS) & 0xF0FF);
+                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0) & 0xF0FF);
+                __builtin_amdgcn_s_barrier();
+            }
+            v4i(&xc)[MI] = (ks & 1) ? xb : xa;
+            v4i(&wc)[NI] = (ks & 1) ? wb : wa;
+            v4i(&xn)[MI] = (ks & 1) ? xa : xb;
+            v4i(&wn_)[NI] = (ks & 1) ? wa : wb;
+            // past the last tile the next-fragment reads fetch stale LDS that nobody uses
+            if (!last) load_frags(st, ks + 1, xn, wn_);
+            else load_frags(nx, 0, xn, wn_);
+#ifndef I8F_ABLATE_DMA
+            if (last) issue(kt + S, kt + S < KT);  // refills the stage tile kt was in
+#endif
+            mma(xc, wc);
+            // Issue order inside the phase: all LDS reads of the NEXT k-step first, so that they
+            // complete under this phase's MFMAs; in the last phase the global loads of tile kt+S
+            // are spread between the MFMAs.
+            __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
+            if (last) {
 #pragma unroll
-            for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
-#pragma unroll
-            for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ks]);
-#pragma unroll
-            for (int i = 0; i < MI; ++i)
-#pragma unroll
-                for (int j = 0; j < NI; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+                for (int r = 0; r < C::LOADS; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                }
+                if (MI * NI > C::LOADS) __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - C::LOADS, 0);
+            } else {
+                __builtin_amdgcn_sched_group_barrier(0x008, MI * NI, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
     // ---- epilogue ----------------------------------------------------------------------
     __syncthreads();  // the stages are dead; reuse them as per-wave transpose buffers
+#ifdef I8F_TRACE
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 2] = wall_clock64();
+#endif
     constexpr int ROW_BYTES = C::WTN * OB;
     constexpr int PITCH = ROW_BYTES + (OB == 2 ? 8 : 16);
     constexpr int WAVE_BYTES = 32 * PITCH;
     static_assert(WAVE_BYTES * NW <= C::LDS_BYTES, "epilogue buffer");
     char *ebuf = smem + wave * WAVE_BYTES;
 
-    const bool has_bias = g.bias != nullptr;
-    const float ws_one = g.ws ? (g.row_scale ? 0.0f : g.ws[0]) : g.ws_host;
-
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-        const int m = m0 + wm * C::WTM + i * 32 + l32;
-        float xs = 0.0f;
-        if (OUT != OUT_I32 && m < g.M) xs = g.xs[m];
+    // scale, bias, round: the flags are wave-uniform, so the variant is chosen once
+    auto convert_strip = [&](int i, auto ORDER, auto ROW, auto BIAS) {
+        const float xs = s_xs[wm * C::WTM + i * 32 + l32];
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
                 const int nl = j * 32 + qd * 8 + lhalf * 4;  // first of 4 consecutive n held by this lane
-                const int n = n0 + wn * C::WTN + nl;
-                if constexpr (OUT == OUT_I32) {
+                const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
+                float4 w4, b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                w4 = *(const float4 *)&s_ws[wn * C::WTN + nl];
+                if constexpr (decltype(BIAS)::value) b4 = *(const float4 *)&s_bias[wn * C::WTN + nl];
+                epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value>(
+                    a4, xs, w4, b4, ebuf + l32 * PITCH + nl * OB);
+            }
+        }
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    using O0 = std::integral_constant<int, I8F_EPI_TORCH>;
+    using O1 = std::integral_constant<int, I8F_EPI_FUSED>;
+    const int variant = (g.order == I8F_EPI_FUSED ? 4 : 0) | (g.row_scale ? 2 : 0) | (g.bias ? 1 : 0);
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        if constexpr (OUT == OUT_I32) {
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    const int nl = j * 32 + qd * 8 + lhalf * 4;
                     v4i o = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
                     *(v4i *)(ebuf + l32 * PITCH + nl * 4) = o;
-                } else {
-                    float wsv[4], bv[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        wsv[e] = ws_one;
-                        bv[e] = 0.0f;
-                    }
-                    if (n < g.N) {  // N is a multiple of 8 here: the four n are all inside or all outside
-                        if (g.row_scale) {
-                            const float4 t = *(const float4 *)(g.ws + n);
-                            wsv[0] = t.x, wsv[1] = t.y, wsv[2] = t.z, wsv[3] = t.w;
-                        }
-                        if (has_bias) {
-                            if (g.bias_dtype == I8F_F32) {
-                                const float4 t = *(const float4 *)((const float *)g.bias + n);
-                                bv[0] = t.x, bv[1] = t.y, bv[2] = t.z, bv[3] = t.w;
-                            } else {
-                                const uint2 t = *(const uint2 *)((const uint16_t *)g.bias + n);
-                                if (g.bias_dtype == I8F_BF16) {
-                                    bv[0] = bf16_bits_to_f32(t.x & 0xffffu), bv[1] = bf16_bits_to_f32(t.x >> 16);
-                                    bv[2] = bf16_bits_to_f32(t.y & 0xffffu), bv[3] = bf16_bits_to_f32(t.y >> 16);
-                                } else {
-                                    bv[0] = f16_bits_to_f32(t.x & 0xffffu), bv[1] = f16_bits_to_f32(t.x >> 16);
-                                    bv[2] = f16_bits_to_f32(t.y & 0xffffu), bv[3] = f16_bits_to_f32(t.y >> 16);
-                                }
-                            }
-                        }
-                    }
-                    float y[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float a = (float)acc[i][j][4 * qd + e];
-                        constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : (OUT == OUT_F16 ? I8F_F16 : I8F_F32);
-                        if (g.order == I8F_EPI_TORCH) {
-                            float t;
-                            if (g.row_scale) {
-                                t = a * xs;
-                                t = t * wsv[e];
-                            } else {
-                                const float sc = wsv[e] * xs;
-                                t = a * sc;
-                            }
-                            t = round_to_dtype<DT>(t);
-                            if (has_bias) t = t + round_to_dtype<DT>(bv[e]);
-                            y[e] = t;
-                        } else {
-                            const float sc = xs * wsv[e];
-                            float t = a * sc;
-                            if (has_bias) t = t + bv[e];
-                            y[e] = t;
-                        }
-                    }
-                    if constexpr (OUT == OUT_BF16) {
-                        *(uint2 *)(ebuf + l32 * PITCH + nl * 2) =
-                            make_uint2(f32x2_to_bf16x2_bits(y[0], y[1]), f32x2_to_bf16x2_bits(y[2], y[3]));
-                    } else if constexpr (OUT == OUT_F16) {
-                        *(uint2 *)(ebuf + l32 * PITCH + nl * 2) =
-                            make_uint2(f32x2_to_f16x2_bits(y[0], y[1]), f32x2_to_f16x2_bits(y[2], y[3]));
-                    } else {
-                        *(float4 *)(ebuf + l32 * PITCH + nl * 4) = make_float4(y[0], y[1], y[2], y[3]);
-                    }
                 }
+        } else {
+            switch (variant) {
+            case 0: convert_strip(i, O0{}, F_{}, F_{}); break;
+            case 1: convert_strip(i, O0{}, F_{}, T_{}); break;
+            case 2: convert_strip(i, O0{}, T_{}, F_{}); break;
+            case 3: convert_strip(i, O0{}, T_{}, T_{}); break;
+            case 4: convert_strip(i, O1{}, F_{}, F_{}); break;
+            case 5: convert_strip(i, O1{}, F_{}, T_{}); break;
+            case 6: convert_strip(i, O1{}, T_{}, F_{}); break;
+            default: convert_strip(i, O1{}, T_{}, T_{}); break;
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -310,10 +421,19 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
             const uint4 val = *(const uint4 *)(ebuf + row * PITCH + cc * 16);
             const int mm = m0 + wm * C::WTM + i * 32 + row;
             const int nn = n0 + wn * C::WTN + cc * EPCO;
-            if (mm < g.M && nn < g.N) *(uint4 *)((char *)g.out + ((int64_t)mm * g.N + nn) * OB) = val;
+#ifdef I8F_ABLATE_STORE  // development probe: the store is kept in the code but never taken
+            if (mm < g.M && nn < g.N && val.x == 0x12345678u && val.y == 0x9abcdef0u)
+#else
+            if (mm < g.M && nn < g.N)
+#endif
+                *(uint4 *)((char *)g.out + ((int64_t)mm * g.N + nn) * OB) = val;
         }
         __builtin_amdgcn_wave_barrier();
     }
+#ifdef I8F_TRACE
+    __syncthreads();
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 3] = wall_clock64();
+#endif
 }
 
 // ---- slow but shape-agnostic kernel: one thread per output -----------------------------
@@ -360,15 +480,19 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 }
 
 // tile configurations
-using CfgBig = Cfg<256, 256, 64, 2, 4, 4, 6>;    // 8 waves, 128 KB LDS, one workgroup per CU
-using CfgMid = Cfg<128, 128, 64, 2, 2, 4, 8>;    // 4 waves, 64 KB LDS, two workgroups per CU
+using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6>;   // 8 waves, 2 x 64 KB stages, one workgroup per CU
+using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
 
 template <class C, int OUT>
 int launch_cfg(GemmArgs &g, hipStream_t st) {
     g.tiles_m = (g.M + C::BM - 1) / C::BM;
     g.tiles_n = (g.N + C::BN - 1) / C::BN;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    hipLaunchKernelGGL((gemm_i8_kernel<C, OUT>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g);
+#ifdef I8F_TRACE
+    g.trace = (long long *)(getenv("I8F_TRACE_PTR") ? strtoull(getenv("I8F_TRACE_PTR"), nullptr, 0) : 0ull);
+#endif
+    if (g.K % C::BK) hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g);
+    else hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g);
     return check_launch();
 }
 

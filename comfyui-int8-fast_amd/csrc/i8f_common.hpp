@@ -54,7 +54,11 @@ __device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
     bf2 o = __builtin_convertvector(in, bf2);
     return __builtin_bit_cast(uint32_t, o);
 }
+// The empty asm keeps the value opaque on its way into the conversion: without it the compiler
+// folds a preceding binary32 multiply into v_fma_mixlo_f16, which rounds the exact product once
+// to binary16 instead of first to binary32 and then to binary16, and the results differ on ties.
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float v) {
+    asm("" : "+v"(v));
     return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v);
 }
 __device__ __forceinline__ uint32_t f32x2_to_f16x2_bits(float lo, float hi) {
