@@ -51,7 +51,7 @@ struct GemmArgs {
     void *out;
     int tiles_m, tiles_n;
 #ifdef I8F_TRACE
-    long long *trace;  // [blocks][4] wall-clock stamps: start, first tile landed, loop done, end
+    long long *trace;  // [blocks][8] wall-clock stamps: start, first tile landed, loop done, end, + epilogue detail
 #endif
 };
 
@@ -71,7 +71,6 @@ struct Cfg {
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(X_BYTES % (1024 * NW) == 0 && W_BYTES % (1024 * NW) == 0, "tile must split into whole wave loads");
     static_assert(BK == 64 || BK == 128, "BK");
-    static_assert(LDS_BYTES + 4 * (BM + 2 * BN) <= 160 * 1024, "LDS");
 };
 
 // chunk swizzle: a function of the low 5 bits of the row only
@@ -140,7 +139,15 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     constexpr int OB = OutElem<OUT>::BYTES;
     constexpr int KS = BK / 32;  // MFMA k-steps per tile
     static_assert(KS % 2 == 0, "fragment double-buffering alternates over an even number of k-steps");
-    __shared__ __attribute__((aligned(1024))) char smem[C::LDS_BYTES];
+    // The epilogue stages EPI_STRIPS 32-row strips of a wave's tile at once (all of it for 2-byte
+    // outputs), padded so that the transposing writes do not collide on banks.
+    constexpr int ROW_BYTES = C::WTN * OB;
+    constexpr int PITCH = ROW_BYTES + (OB == 2 ? 8 : 16);
+    constexpr int EPI_STRIPS = (OB == 2 || MI == 1) ? MI : MI / 2;
+    constexpr int WAVE_BYTES = EPI_STRIPS * 32 * PITCH;
+    constexpr int SMEM_BYTES = C::LDS_BYTES > WAVE_BYTES * NW ? C::LDS_BYTES : WAVE_BYTES * NW;
+    static_assert(SMEM_BYTES + 4 * (BM + 2 * BN) <= 160 * 1024, "LDS");
+    __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
     __shared__ float s_xs[BM], s_ws[BN], s_bias[BN];  // epilogue operands of this tile
 
     const int tid = threadIdx.x;
@@ -168,7 +175,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 #ifdef I8F_TRACE
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 0] = wall_clock64();
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 0] = wall_clock64();
 #endif
 
     // ---- epilogue operands: fetched once, long before they are needed ----------------------
@@ -267,14 +274,14 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    auto load_frags = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI]) {
-#ifdef I8F_ABLATE_LDSREAD  // development probe
-        return;
+    auto load_frags = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI], bool force = false) {
+#ifdef I8F_ABLATE_LDSREAD  // development probe: fragments are read once, before the loop
+        if (!force) return;
 #endif
 #pragma unroll
-        for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
-#pragma unroll
         for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ks]);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
     };
     auto mma = [&](const v4i (&xf)[MI], const v4i (&wf)[NI]) {
 #pragma unroll
@@ -296,7 +303,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();  // tile 0 and the staged epilogue operands are visible to everyone
 #ifdef I8F_TRACE
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 1] = wall_clock64();
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 1] = wall_clock64();
 #endif
 
     // Fragments are double-buffered in registers: the LDS reads of k-step s+1 are issued before
@@ -305,7 +312,10 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // (its last fragments are in registers), so the stage of tile kt is refilled with tile kt+S
     // right away, and tile kt+1 is known to have landed, so its first fragments can be fetched.
     v4i xa[MI] = {}, wa[NI] = {}, xb[MI] = {}, wb[NI] = {};
-    if (KT > 0) load_frags(smem, 0, xa, wa);
+    if (KT > 0) load_frags(smem, 0, xa, wa, true);
+#ifdef I8F_ABLATE_LDSREAD
+    load_frags(smem, 1, xb, wb, true);
+#endif
     // Drain scalar loads (kernel arguments) here: a scalar load still pending at the loop header
     // would turn every LDS wait inside the loop into a full lgkmcnt(0).
     __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -337,16 +347,28 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
             // Issue order inside the phase: all LDS reads of the NEXT k-step first, so that they
             // complete under this phase's MFMAs; in the last phase the global loads of tile kt+S
             // are spread between the MFMAs.
-            __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-            if (last) {
+#ifndef I8F_SCHED
+#define I8F_SCHED 0
+#endif
+            if constexpr (I8F_SCHED == 0) {  // all LDS reads first
+                __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
+                if (last) {
 #pragma unroll
-                for (int r = 0; r < C::LOADS; ++r) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    for (int r = 0; r < C::LOADS; ++r) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    }
+                    if (MI * NI > C::LOADS) __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - C::LOADS, 0);
+                } else {
+                    __builtin_amdgcn_sched_group_barrier(0x008, MI * NI, 0);
                 }
-                if (MI * NI > C::LOADS) __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - C::LOADS, 0);
-            } else {
-                __builtin_amdgcn_sched_group_barrier(0x008, MI * NI, 0);
+            } else {  // one LDS read after each of the first MFMAs (and one global load in the last phase)
+#pragma unroll
+                for (int r = 0; r < MI * NI; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (r < MI + NI) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if (last && r < C::LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -355,16 +377,16 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // ---- epilogue ----------------------------------------------------------------------
     __syncthreads();  // the stages are dead; reuse them as per-wave transpose buffers
 #ifdef I8F_TRACE
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 2] = wall_clock64();
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 2] = wall_clock64();
 #endif
-    constexpr int ROW_BYTES = C::WTN * OB;
-    constexpr int PITCH = ROW_BYTES + (OB == 2 ? 8 : 16);
-    constexpr int WAVE_BYTES = 32 * PITCH;
-    static_assert(WAVE_BYTES * NW <= C::LDS_BYTES, "epilogue buffer");
     char *ebuf = smem + wave * WAVE_BYTES;
 
     // scale, bias, round: the flags are wave-uniform, so the variant is chosen once
-    auto convert_strip = [&](int i, auto ORDER, auto ROW, auto BIAS) {
+    // scale, bias, round.  The per-column operands (4 consecutive n per lane and MFMA block) are
+    // fetched from LDS into registers once, in front of the strips: fetched inside, every group of
+    // four values would wait for an LDS round trip.
+    auto convert_strip = [&](int i, char *dst_rows, const float4 (&wr)[NI][4], const float4 (&br)[NI][4], auto ORDER,
+                             auto ROW, auto BIAS) {
         const float xs = s_xs[wm * C::WTM + i * 32 + l32];
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
@@ -372,11 +394,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
             for (int qd = 0; qd < 4; ++qd) {
                 const int nl = j * 32 + qd * 8 + lhalf * 4;  // first of 4 consecutive n held by this lane
                 const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-                float4 w4, b4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                w4 = *(const float4 *)&s_ws[wn * C::WTN + nl];
-                if constexpr (decltype(BIAS)::value) b4 = *(const float4 *)&s_bias[wn * C::WTN + nl];
                 epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value>(
-                    a4, xs, w4, b4, ebuf + l32 * PITCH + nl * OB);
+                    a4, xs, wr[j][qd], br[j][qd], dst_rows + l32 * PITCH + nl * OB);
             }
         }
     };
@@ -386,53 +405,91 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     using O1 = std::integral_constant<int, I8F_EPI_FUSED>;
     const int variant = (g.order == I8F_EPI_FUSED ? 4 : 0) | (g.row_scale ? 2 : 0) | (g.bias ? 1 : 0);
 
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-        if constexpr (OUT == OUT_I32) {
+    // The whole epilogue is instantiated once per variant and the variant is chosen ONCE, so that
+    // the instructions a wave executes are contiguous in memory (the epilogue runs once per wave,
+    // straight from a cold instruction cache).
+    auto run_epilogue = [&](auto ORDER, auto ROW, auto BIAS) {
+        float4 wr[NI][4], br[NI][4];
+        if constexpr (OUT != OUT_I32) {
 #pragma unroll
             for (int j = 0; j < NI; ++j)
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd) {
-                    const int nl = j * 32 + qd * 8 + lhalf * 4;
-                    v4i o = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-                    *(v4i *)(ebuf + l32 * PITCH + nl * 4) = o;
+                    const int nl = wn * C::WTN + j * 32 + qd * 8 + lhalf * 4;
+                    if constexpr (decltype(ROW)::value) wr[j][qd] = *(const float4 *)&s_ws[nl];
+                    else wr[j][qd] = make_float4(s_ws[0], s_ws[0], s_ws[0], s_ws[0]);
+                    if constexpr (decltype(BIAS)::value) br[j][qd] = *(const float4 *)&s_bias[nl];
+                    else br[j][qd] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
-        } else {
-            switch (variant) {
-            case 0: convert_strip(i, O0{}, F_{}, F_{}); break;
-            case 1: convert_strip(i, O0{}, F_{}, T_{}); break;
-            case 2: convert_strip(i, O0{}, T_{}, F_{}); break;
-            case 3: convert_strip(i, O0{}, T_{}, T_{}); break;
-            case 4: convert_strip(i, O1{}, F_{}, F_{}); break;
-            case 5: convert_strip(i, O1{}, F_{}, T_{}); break;
-            case 6: convert_strip(i, O1{}, T_{}, F_{}); break;
-            default: convert_strip(i, O1{}, T_{}, T_{}); break;
-            }
         }
-        __builtin_amdgcn_wave_barrier();
-        // read the 32 x WTN strip back row-contiguously and store 16 bytes per lane
-        constexpr int CPO = ROW_BYTES / 16;      // chunks per output row of the strip
-        constexpr int EPCO = 16 / OB;            // output elements per chunk
-        constexpr int PASSES = 32 * CPO / 64;
-#pragma unroll
-        for (int p = 0; p < PASSES; ++p) {
-            const int id = p * 64 + lane;
-            const int row = id / CPO, cc = id % CPO;
-            const uint4 val = *(const uint4 *)(ebuf + row * PITCH + cc * 16);
-            const int mm = m0 + wm * C::WTM + i * 32 + row;
-            const int nn = n0 + wn * C::WTN + cc * EPCO;
-#ifdef I8F_ABLATE_STORE  // development probe: the store is kept in the code but never taken
-            if (mm < g.M && nn < g.N && val.x == 0x12345678u && val.y == 0x9abcdef0u)
-#else
-            if (mm < g.M && nn < g.N)
+#ifdef I8F_TRACE
+        if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 4] = wall_clock64();
 #endif
-                *(uint4 *)((char *)g.out + ((int64_t)mm * g.N + nn) * OB) = val;
+#pragma unroll
+        for (int i0 = 0; i0 < MI; i0 += EPI_STRIPS) {
+#pragma unroll
+            for (int is = 0; is < EPI_STRIPS; ++is) {
+                const int i = i0 + is;
+                char *rows = ebuf + is * 32 * PITCH;
+                if constexpr (OUT == OUT_I32) {
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+#pragma unroll
+                        for (int qd = 0; qd < 4; ++qd) {
+                            const int nl = j * 32 + qd * 8 + lhalf * 4;
+                            v4i o = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
+                            *(v4i *)(rows + l32 * PITCH + nl * 4) = o;
+                        }
+                } else {
+                    convert_strip(i, rows, wr, br, ORDER, ROW, BIAS);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+#ifdef I8F_TRACE
+            if (tid == 0 && g.trace && i0 == 0) g.trace[blockIdx.x * 8 + 5] = wall_clock64();
+#endif
+            // read the staged rows back row-contiguously and store 16 bytes per lane
+            constexpr int CPO = ROW_BYTES / 16;      // chunks per output row
+            constexpr int EPCO = 16 / OB;            // output elements per chunk
+            constexpr int PASSES = EPI_STRIPS * 32 * CPO / 64;
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int id = p * 64 + lane;
+                const int row = id / CPO, cc = id % CPO;
+                const uint4 val = *(const uint4 *)(ebuf + row * PITCH + cc * 16);
+                const int mm = m0 + wm * C::WTM + i0 * 32 + row;
+                const int nn = n0 + wn * C::WTN + cc * EPCO;
+#ifdef I8F_ABLATE_STORE  // development probe: the store is kept in the code but never taken
+                if (mm < g.M && nn < g.N && val.x == 0x12345678u && val.y == 0x9abcdef0u)
+#else
+                if (mm < g.M && nn < g.N)
+#endif
+                    *(uint4 *)((char *)g.out + ((int64_t)mm * g.N + nn) * OB) = val;
+            }
+            __builtin_amdgcn_wave_barrier();
+#ifdef I8F_TRACE
+            if (tid == 0 && g.trace && i0 == 0) g.trace[blockIdx.x * 8 + 6] = wall_clock64();
+#endif
         }
-        __builtin_amdgcn_wave_barrier();
+    };
+    if constexpr (OUT == OUT_I32) {
+        run_epilogue(O0{}, F_{}, F_{});
+    } else {
+        switch (variant) {
+        case 0: run_epilogue(O0{}, F_{}, F_{}); break;
+        case 1: run_epilogue(O0{}, F_{}, T_{}); break;
+        case 2: run_epilogue(O0{}, T_{}, F_{}); break;
+        case 3: run_epilogue(O0{}, T_{}, T_{}); break;
+        case 4: run_epilogue(O1{}, F_{}, F_{}); break;
+        case 5: run_epilogue(O1{}, F_{}, T_{}); break;
+        case 6: run_epilogue(O1{}, T_{}, F_{}); break;
+        default: run_epilogue(O1{}, T_{}, T_{}); break;
+        }
     }
 #ifdef I8F_TRACE
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 7] = wall_clock64();
     __syncthreads();
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 4 + 3] = wall_clock64();
+    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 3] = wall_clock64();
 #endif
 }
 
