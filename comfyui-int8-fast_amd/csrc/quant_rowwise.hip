@@ -19,6 +19,8 @@
 // rounding to x's dtype.  Strides smaller than the per-lane chunk are done in
 // registers, the rest across lanes; the order of operations does not depend on
 // how the block is spread over lanes.
+#include <cstdlib>
+
 #include "i8f_common.hpp"
 
 namespace i8f {
@@ -162,6 +164,237 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void quant_rows_kernel(
         }
     }
     if (t == 0) scale[m] = s;
+}
+
+// ---- 16-bit inputs, the hot case -------------------------------------------------------
+// A lane owns runs of 16 consecutive elements (32 bytes in, 16 bytes out): the int8 store is
+// one fully coalesced 16-byte store per lane and run.  With the rotation a 128-block is 8 runs,
+// held by an aligned group of 8 lanes: strides 1..8 of the butterfly stay inside a lane, strides
+// 16, 32, 64 pair lanes through DPP (quad permutes and the 8-lane mirror).  The mirror flips all
+// three low lane bits, so lanes 4..7 of a group hold runs 7,6,5,4: then "mirror" pairs exactly
+// the runs that differ in bit 2.  The arithmetic is the same fixed-order butterfly as everywhere
+// else; only the assignment of elements to lanes differs.
+//
+// Rounding to int8 uses the 1.5*2^23 trick: p + 12582912.0f is exact round-half-to-even of p for
+// |p| < 2^22 and leaves the two's-complement integer in the low mantissa bits.  No clamp is
+// needed: |v * inv| <= 127 * (1 + 2^-22) because inv = 1/fl(amax/127) and |v| <= amax.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+template <int DT>
+__device__ __forceinline__ void expand16(const uint4 &a, const uint4 &b, float (&v)[16]) {
+    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if constexpr (DT == I8F_BF16) {
+            v[2 * j] = __uint_as_float(w[j] << 16);
+            v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        } else {
+            v[2 * j] = f16_bits_to_f32(w[j] & 0xffffu);
+            v[2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+        }
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void rotate_run16(float (&v)[16], float s0, float s1, float s2) {
+#pragma unroll
+    for (int s = 1; s < 16; s <<= 1) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            if ((j & s) == 0) {
+                const float lo = v[j], hi = v[j + s];
+                v[j] = lo + hi;
+                v[j + s] = lo - hi;
+            }
+        }
+    }
+    // lower lane: own + other; upper lane: other - own  ==  other + sign * own (the product is exact)
+    // (all products first, then the DPP adds: a DPP instruction needs two wait states after a VALU
+    // write of any of its sources, which back-to-back pairs would pay as s_nop)
+    float w[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) w[j] = v[j] * s0;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = dpp_f32<0xB1>(v[j]) + w[j];   // quad_perm [1,0,3,2]
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) w[j] = v[j] * s1;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = dpp_f32<0x4E>(v[j]) + w[j];   // quad_perm [2,3,0,1]
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) w[j] = v[j] * s2;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = dpp_f32<0x141>(v[j]) + w[j];  // row_half_mirror
+    __builtin_amdgcn_sched_barrier(0);
+    const float h = hadamard_entry<DT>();
+#pragma unroll
+    for (int j = 0; j < 16; j += 2) {
+        const float a = v[j] * h, b = v[j + 1] * h;
+        if constexpr (DT == I8F_BF16) {  // one packed conversion rounds two values
+            const uint32_t pk = f32x2_to_bf16x2_bits(a, b);
+            v[j] = __uint_as_float(pk << 16);
+            v[j + 1] = __uint_as_float(pk & 0xffff0000u);
+        } else {
+            v[j] = round_to_dtype<DT>(a);
+            v[j + 1] = round_to_dtype<DT>(b);
+        }
+    }
+}
+
+__device__ __forceinline__ float max3_abs(float m, float a, float b) {
+    float r;
+    asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(m), "v"(a), "v"(b));
+    return r;
+}
+
+__device__ __forceinline__ uint32_t quant4_magic(float a, float b, float c, float d, float inv) {
+    const float M = 12582912.0f;
+    const uint32_t ua = __float_as_uint(a * inv + M), ub = __float_as_uint(b * inv + M);
+    const uint32_t uc = __float_as_uint(c * inv + M), ud = __float_as_uint(d * inv + M);
+    // low bytes of the four sums: {ua.b0, ub.b0} and {uc.b0, ud.b0}, then the two halves
+    const uint32_t lo = __builtin_amdgcn_perm(ub, ua, 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm(ud, uc, 0x04000c0cu);
+    return lo | hi;
+}
+
+// WPR waves share a row (1 or 4); each lane holds RUNS runs of 16 elements.  With WPR == 1 a wave
+// walks NROW rows (grid-strided, so that the waves running together touch neighbouring rows) and
+// fetches the next row while it reduces, scales and stores the current one: loads and stores of
+// different rows overlap inside a wave instead of every wave of the grid moving from a read phase
+// to a write phase in step.
+template <int DT, bool ROT, int WPR, int RUNS, int NROW>
+__global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x, int64_t M, int64_t K,
+                                                       int64_t ldx_bytes, int8_t *__restrict__ q,
+                                                       float *__restrict__ scale) {
+    static_assert(WPR == 1 || NROW == 1, "rows are walked only by single-wave rows");
+    constexpr int TPR = 64 * WPR;
+    constexpr int ROWS = 256 / TPR;
+    const int t = threadIdx.x % TPR;
+    const int rb = threadIdx.x / TPR;
+    const int64_t row_stride = (int64_t)gridDim.x * ROWS;
+    const int64_t m_first = (int64_t)blockIdx.x * ROWS + rb;
+    const int nruns = (int)(K / 16);
+    // run held by this lane inside its group of 8: lanes 4..7 take runs 7..4
+    const int p = t ^ (((t >> 2) & 1) * 3);
+    const float s0 = (p & 1) ? -1.0f : 1.0f, s1 = (p & 2) ? -1.0f : 1.0f, s2 = (p & 4) ? -1.0f : 1.0f;
+
+    auto fetch = [&](int64_t m, uint4 (&raw)[RUNS][2]) {
+        const bool ok = m < M;
+        const char *xrow = x + (ok ? m : 0) * ldx_bytes;
+#pragma unroll
+        for (int r = 0; r < RUNS; ++r) {
+            const int R = r * TPR + p;
+            if (ok && R < nruns) {
+                raw[r][0] = *(const uint4 *)(xrow + (int64_t)R * 32);
+                raw[r][1] = *(const uint4 *)(xrow + (int64_t)R * 32 + 16);
+            } else {
+                raw[r][0] = make_uint4(0, 0, 0, 0);
+                raw[r][1] = make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+
+    uint4 raw[2][RUNS][2];
+    fetch(m_first, raw[0]);
+#pragma unroll
+    for (int it = 0; it < NROW; ++it) {
+        const int64_t m = m_first + it * row_stride;
+        if (it + 1 < NROW) fetch(m + row_stride, raw[(it + 1) & 1]);
+
+        float v[RUNS][16];
+        float amax = 0.0f;
+#pragma unroll
+        for (int r = 0; r < RUNS; ++r) {
+            expand16<DT>(raw[it & 1][r][0], raw[it & 1][r][1], v[r]);
+            if constexpr (ROT) rotate_run16<DT>(v[r], s0, s1, s2);
+#pragma unroll
+            for (int j = 0; j < 16; j += 2) amax = max3_abs(amax, v[r][j], v[r][j + 1]);
+        }
+        amax = wave_max(amax);
+        if constexpr (WPR > 1) {
+            __shared__ float red[ROWS][WPR];
+            if ((t & 63) == 0) red[rb][t / 64] = amax;
+            __syncthreads();
+            amax = red[rb][0];
+#pragma unroll
+            for (int w = 1; w < WPR; ++w) amax = fmaxf(amax, red[rb][w]);
+        }
+
+        float s = amax / 127.0f;
+        s = s < 1e-30f ? 1e-30f : s;
+        const float inv = 1.0f / s;
+
+        if (m < M) {
+            int8_t *qrow = q + m * K;
+#pragma unroll
+            for (int r = 0; r < RUNS; ++r) {
+                const int R = r * TPR + p;
+                if (R < nruns) {
+                    uint4 o;
+                    o.x = quant4_magic(v[r][0], v[r][1], v[r][2], v[r][3], inv);
+                    o.y = quant4_magic(v[r][4], v[r][5], v[r][6], v[r][7], inv);
+                    o.z = quant4_magic(v[r][8], v[r][9], v[r][10], v[r][11], inv);
+                    o.w = quant4_magic(v[r][12], v[r][13], v[r][14], v[r][15], inv);
+                    *(uint4 *)(qrow + (int64_t)R * 16) = o;
+                }
+            }
+            if (t == 0) scale[m] = s;
+        }
+    }
+}
+
+// rows a wave walks; development probes may override it through I8F_QUANT_NROW
+static int nrow_for(int64_t M) {
+    static const int forced = [] {
+        const char *e = getenv("I8F_QUANT_NROW");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced >= 1 && forced <= 4) return forced;
+    return 1;
+}
+
+// development probe: dynamic LDS per block, which caps the blocks resident on a CU
+static unsigned lds_probe() {
+    static const unsigned v = [] {
+        const char *e = getenv("I8F_QUANT_LDS");
+        return e ? (unsigned)atoi(e) : 0u;
+    }();
+    return v;
+}
+
+template <int DT, bool ROT, int WPR, int RUNS>
+int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st) {
+    constexpr int ROWS = 256 / (64 * WPR);
+    const int nrow = WPR == 1 ? nrow_for(M) : 1;
+    const int64_t blocks = (M + (int64_t)ROWS * nrow - 1) / ((int64_t)ROWS * nrow);
+    const char *xc = (const char *)x;
+    if constexpr (WPR == 1) {
+        switch (nrow) {
+        case 2: hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 2>), dim3((unsigned)blocks), dim3(256), 0, st, xc, M, K, ldx * 2, q, scale); return check_launch();
+        case 3: hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 3>), dim3((unsigned)blocks), dim3(256), 0, st, xc, M, K, ldx * 2, q, scale); return check_launch();
+        case 4: hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 4>), dim3((unsigned)blocks), dim3(256), 0, st, xc, M, K, ldx * 2, q, scale); return check_launch();
+        default: break;
+        }
+    }
+    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1>), dim3((unsigned)blocks), dim3(256), lds_probe(), st, xc, M, K, ldx * 2, q, scale);
+    return check_launch();
+}
+
+template <int DT, bool ROT, int WPR>
+int pick_runs16(int runs, const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st) {
+    switch (runs) {
+    case 1: return launch16<DT, ROT, WPR, 1>(x, M, K, ldx, q, scale, st);
+    case 2: return launch16<DT, ROT, WPR, 2>(x, M, K, ldx, q, scale, st);
+    case 3: return launch16<DT, ROT, WPR, 3>(x, M, K, ldx, q, scale, st);
+    default: return launch16<DT, ROT, WPR, 4>(x, M, K, ldx, q, scale, st);
+    }
 }
 
 // ---- generic kernel: any K, any alignment; one 256-thread block per row, the row
@@ -329,6 +562,13 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
     const bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) &&
                          ((uintptr_t)q % 8 == 0);
     const int64_t nchunks = K / EPC;
+    if constexpr (DT != I8F_F32) {
+        const int64_t nruns = K / 16;
+        if (aligned && K % 16 == 0 && (uintptr_t)q % 16 == 0 && nruns >= 1 && nruns <= 64 * 4 * 4) {
+            if (nruns <= 64 * 4) return pick_runs16<DT, ROT, 1>((int)((nruns + 63) / 64), x, M, K, ldx, q, scale, st);
+            return pick_runs16<DT, ROT, 4>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st);
+        }
+    }
     if (aligned && nchunks <= 1024 * 8) {
         if (nchunks <= 64 * 8) return pick_nch<DT, ROT, 64>((int)((nchunks + 63) / 64), x, M, K, ldx, q, scale, st);
         if (nchunks <= 256 * 8) return pick_nch<DT, ROT, 256>((int)((nchunks + 255) / 256), x, M, K, ldx, q, scale, st);
