@@ -82,20 +82,25 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def time_kernel(fn, iters=50, warmup=5, sets=1):
-    """Median / min / mean device time of fn(set_index) in microseconds, from HIP events on the
-    launch stream.  `sets` distinct argument sets are cycled so that a bandwidth kernel does not
-    find its operands in the 256 MB memory-side cache."""
+def time_kernel(fn, iters=50, warmup=5, sets=1, burst=1):
+    """Median / min / mean device time of ONE fn(set_index) launch in microseconds, from HIP events on
+    the launch stream.  `sets` distinct argument sets are cycled so that a bandwidth kernel does not
+    find its operands in the 256 MB memory-side cache.  With burst > 1 each event pair brackets that
+    many back-to-back launches and the time is divided by it: for kernels of a few microseconds a
+    pair of events around a single launch mostly measures the gap between dispatches."""
     for i in range(warmup):
         fn(i % sets)
     torch.cuda.synchronize()
     starts, stops = _events(iters), _events(iters)
+    k = 0
     for i in range(iters):
         starts[i].record()
-        fn(i % sets)
+        for _ in range(burst):
+            fn(k % sets)
+            k += 1
         stops[i].record()
     torch.cuda.synchronize()
-    us = [s.elapsed_time(e) * 1e3 for s, e in zip(starts, stops)]
+    us = [s.elapsed_time(e) * 1e3 / burst for s, e in zip(starts, stops)]
     return {"median_us": statistics.median(us), "min_us": min(us), "mean_us": statistics.fmean(us)}
 
 
@@ -150,22 +155,30 @@ def extras(L, dev, quick=False):
     out["target_gemm_4608x3072x3072"] = {"median_us": round(t["median_us"], 2), "min_us": round(t["min_us"], 2),
                                           "tops": round(tops, 1), "frac_of_int8_peak": round(tops / PEAK_INT8_TOPS, 4)}
 
-    # fused rotate + quant at the same shape, cycling 8 buffer sets (> 256 MB in total)
+    # fused rotate + quant at the same shape, cycling 8 buffer sets (> 256 MB in total), bursts of 8
+    # launches per event pair; a plain device copy of the same byte count is the practical ceiling
     sets = 8
     xs = [x] + [_acts(g, M, K, 0.01, 20.0).to(dev) for _ in range(sets - 1)]
     qs = [torch.empty(M, K, dtype=torch.int8, device=dev) for _ in range(sets)]
     ss = [torch.empty(M, 1, dtype=torch.float32, device=dev) for _ in range(sets)]
     lib, ptr, stream = L.lib(), L._ptr, L._stream(x)
     qbytes = M * K * 3 + 4 * M
+    reps = max(5, iters // 8)
     for name, rb in (("quant_4608x3072", 0), ("rotate_quant_4608x3072", 128)):
         def call(i, rb=rb):
             rc = lib.i8f_quant_rowwise(ptr(xs[i]), L.BF16, M, K, K, rb, ptr(qs[i]), ptr(ss[i]), stream)
             assert rc == 0, rc
-        t = time_kernel(call, iters, sets=sets)
+        t = time_kernel(call, reps, sets=sets, burst=sets)
         gbs = qbytes / t["median_us"] / 1e3
         out[name] = {"median_us": round(t["median_us"], 2), "min_us": round(t["min_us"], 2), "gbs": round(gbs, 1),
                      "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4), "bytes": qbytes, "buffer_sets": sets}
-    del xs, qs, ss
+    half = qbytes // 2
+    srcs = [xs[i].view(torch.uint8).reshape(-1)[:half] for i in range(sets)]
+    dsts = [torch.empty(half, dtype=torch.uint8, device=dev) for _ in range(sets)]
+    t = time_kernel(lambda i: dsts[i].copy_(srcs[i]), reps, sets=sets, burst=sets)
+    out["device_copy_same_bytes"] = {"median_us": round(t["median_us"], 2), "gbs": round(2 * half / t["median_us"] / 1e3, 1),
+                                     "note": "torch copy_ of 21.2 MB -> 21.2 MB, same rotation of buffers: the practical HBM ceiling at this size"}
+    del xs, qs, ss, srcs, dsts
 
     # config 4: stochastic LoRA merge (rank 32 rebuilt in the kernel, float noise) and the skinny GEMM
     c = make_config(4)

@@ -108,6 +108,72 @@ __global__ __launch_bounds__(256) void lora_merge_kernel(const MergeArgs a) {
     }
 }
 
+// Fused low-rank form, the fast kernel.  A thread owns 4 consecutive columns and keeps the RANK x 4
+// slice of `down` it needs in registers for the whole kernel; the block then walks a band of rows.
+// Per row and thread that leaves 16 bytes of noise and 4 bytes of weight to read, 4 bytes to write,
+// and the row of `up`, which is the same for every lane and comes through scalar loads.  (Indexing
+// the other way round, every element re-reads its column of `down` from L2: 32 bytes of cache
+// traffic per byte of weight.)  The sum over the rank is the same fma chain in increasing j.
+// One row is fetched ahead; fetching further ahead costs registers, hence resident waves, and is
+// slower: the kernel is bound by the fma chain, not by memory.
+template <int RANK>
+__global__ __launch_bounds__(256) void lora_merge_band_kernel(const MergeArgs a, int rows_per_block) {
+    const int64_t k0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const bool col_ok = k0 < a.K;  // K % 4 == 0 here
+    float4 dn[RANK];
+#pragma unroll
+    for (int j = 0; j < RANK; ++j)
+        dn[j] = col_ok ? *(const float4 *)(a.down + (int64_t)j * a.K + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
+
+    const int64_t n_begin = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t n_end = n_begin + rows_per_block < a.N ? n_begin + rows_per_block : a.N;
+    if (n_begin >= n_end || !col_ok) return;
+
+    float4 nz = *(const float4 *)(a.noise + n_begin * a.K + k0);
+    uint32_t wp = *(const uint32_t *)(a.w + n_begin * a.K + k0);
+    for (int64_t n = n_begin; n < n_end; ++n) {
+        const float4 nz_cur = nz;
+        const uint32_t wp_cur = wp;
+        if (n + 1 < n_end) {  // next row's operands are in flight while this row is computed
+            nz = *(const float4 *)(a.noise + (n + 1) * a.K + k0);
+            wp = *(const uint32_t *)(a.w + (n + 1) * a.K + k0);
+        }
+        const float sc = a.ws ? a.ws[a.row_scale ? n : 0] : a.ws_host;
+        const float *upr = a.up + n * RANK;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < RANK; ++j) {
+            const float u = upr[j];
+            acc[0] = fmaf(u, dn[j].x, acc[0]);
+            acc[1] = fmaf(u, dn[j].y, acc[1]);
+            acc[2] = fmaf(u, dn[j].z, acc[2]);
+            acc[3] = fmaf(u, dn[j].w, acc[3]);
+        }
+        const float nzv[4] = {nz_cur.x, nz_cur.y, nz_cur.z, nz_cur.w};
+        uint32_t o = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int dq = sr_one(acc[e] * a.lora_scale, sc, nzv[e]);
+            const int wv = (int)(int8_t)(wp_cur >> (8 * e));
+            o |= ((uint32_t)sat8(wv + dq) & 0xffu) << (8 * e);
+        }
+        *(uint32_t *)(a.out + n * a.K + k0) = o;
+    }
+}
+
+template <int RANK>
+int launch_band(const MergeArgs &a, hipStream_t st) {
+    const unsigned col_blocks = (unsigned)((a.K + 1023) / 1024);
+    // enough row bands to fill the chip several times over, each long enough to amortise its slice of `down`
+    int64_t bands = (256 * 12 + col_blocks - 1) / col_blocks;
+    int64_t rows = (a.N + bands - 1) / bands;
+    if (rows < 16) rows = 16;
+    bands = (a.N + rows - 1) / rows;
+    if (bands > 65535) return I8F_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((lora_merge_band_kernel<RANK>), dim3(col_blocks, (unsigned)bands), dim3(256), 0, st, a, (int)rows);
+    return check_launch();
+}
+
 int run(MergeArgs &a, hipStream_t st) {
     if (a.N == 0 || a.K == 0) return I8F_OK;
     if (a.N > 65535 * 1024ll) return I8F_ERR_UNSUPPORTED;
@@ -115,6 +181,15 @@ int run(MergeArgs &a, hipStream_t st) {
     auto al = [](const void *p, int n) { return p == nullptr || (uintptr_t)p % n == 0; };
     const bool vec = a.K % 4 == 0 && al(a.w, 4) && al(a.out, 4) && al(a.noise, 16) && al(a.delta, 16) &&
                      (!fused || al(a.down, 16));
+    if (fused && vec && a.w && a.N < (1ll << 31)) {
+        switch (a.rank) {
+        case 4: return launch_band<4>(a, st);
+        case 8: return launch_band<8>(a, st);
+        case 16: return launch_band<16>(a, st);
+        case 32: return launch_band<32>(a, st);
+        default: break;  // other ranks take the per-element kernel below
+        }
+    }
     // grid.y is limited to 65535: fold larger N into several launches
     for (int64_t n0 = 0; n0 < a.N; n0 += 65535) {
         MergeArgs b = a;
