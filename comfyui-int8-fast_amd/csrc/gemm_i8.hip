@@ -538,6 +538,7 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 
 // tile configurations
 using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6>;   // 8 waves, 2 x 64 KB stages, one workgroup per CU
+using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
 
 template <class C, int OUT>
@@ -567,9 +568,18 @@ int launch(GemmArgs &g, hipStream_t st) {
         hipLaunchKernelGGL((gemm_i8_generic_kernel<OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, g);
         return check_launch();
     }
+    // Tile choice: one workgroup per CU at a time, so a launch costs about
+    // ceil(tiles / 256 CUs) rounds of one tile's work (BM * BN).  Small problems take 128 x 128 tiles,
+    // two workgroups per CU.
+    const int64_t CUS = 256;
+    auto rounds_cost = [&](int bm, int bn) {
+        const int64_t tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
+        return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn;
+    };
     const int64_t big_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    if (big_tiles >= 128) return launch_cfg<CfgBig, OUT>(g, st);
-    return launch_cfg<CfgMid, OUT>(g, st);
+    if (big_tiles < 128) return launch_cfg<CfgMid, OUT>(g, st);
+    if (rounds_cost(256, 192) < rounds_cost(256, 256)) return launch_cfg<CfgB192, OUT>(g, st);
+    return launch_cfg<CfgBig, OUT>(g, st);
 }
 
 int validate(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K, const void *out) {
