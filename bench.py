@@ -77,6 +77,14 @@ def make_config(i: int, rows: int | None = None) -> dict:
     raise ValueError(i)
 
 
+# HBM-side bytes per GEMM launch of config 1, from two rocprofv3 --pmc runs of
+# comfyui-int8-fast_amd/profiling/traffic_probe.py (summary in profiles/hbm_traffic_fetch_write_size.txt):
+# FETCH_SIZE 189790 KiB / WRITE_SIZE 110592 KiB for 4608x12288x3072 and 153780 / 27648 KiB for
+# 4608x3072x12288; a 256 MiB device copy reads 131084 / 262144 KiB on the same counters, so fetches
+# scale by 2.00 and writes by 1.00.  The mean of the two launches:
+GEMM_TRAFFIC_BYTES = int(((189790 * 2.0 + 110592) + (153780 * 2.0 + 27648)) / 2 * 1024)
+
+
 # --------------------------------------------------------------------------- timing helpers
 def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -309,7 +317,9 @@ def main():
                                "quantise + GEMM for both projections, inputs resident in HBM"},
         "pct_of_int8_peak": round(100 * value / PEAK_INT8_TOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
+                     "traffic_unit": "bytes per launch beyond L2 (mean of the two GEMM launches; FETCH_SIZE x 2.00 + "
+                                     "WRITE_SIZE x 1.00, the factors a 256 MiB device copy gives)",
                      "kernel": "gemm_i8_kernel (int8 MFMA GEMM + dequant epilogue)",
                      "ops_per_launch": step.gemm_ops, "avg_launch_us": round(avg_gemm_us, 2),
                      "launches_timed": len(gemm_us)},
