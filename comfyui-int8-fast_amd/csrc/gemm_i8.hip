@@ -577,6 +577,11 @@ int launch(GemmArgs &g, hipStream_t st) {
         return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn;
     };
     const int64_t big_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
+#ifdef I8F_FORCE_CFG  // development probe: one fixed configuration
+    if (I8F_FORCE_CFG == 1) return launch_cfg<CfgBig, OUT>(g, st);
+    if (I8F_FORCE_CFG == 2) return launch_cfg<CfgB192, OUT>(g, st);
+    if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
+#endif
     if (big_tiles < 128) return launch_cfg<CfgMid, OUT>(g, st);
     if (rounds_cost(256, 192) < rounds_cost(256, 256)) return launch_cfg<CfgB192, OUT>(g, st);
     return launch_cfg<CfgBig, OUT>(g, st);
