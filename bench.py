@@ -90,7 +90,7 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def time_kernel(fn, iters=50, warmup=5, sets=1, burst=1):
+def time_kernel(fn, iters=50, warmup=5, sets=1, burst=1, ramp_s=0.05):
     """Median / min / mean device time of ONE fn(set_index) launch in microseconds, from HIP events on
     the launch stream.  `sets` distinct argument sets are cycled so that a bandwidth kernel does not
     find its operands in the 256 MB memory-side cache.  With burst > 1 each event pair brackets that
@@ -99,6 +99,12 @@ def time_kernel(fn, iters=50, warmup=5, sets=1, burst=1):
     for i in range(warmup):
         fn(i % sets)
     torch.cuda.synchronize()
+    t_ramp, i = time.perf_counter(), 0
+    while time.perf_counter() - t_ramp < ramp_s:   # keep the GPU at its sustained clocks (see main)
+        for _ in range(20):
+            fn(i % sets)
+            i += 1
+        torch.cuda.synchronize()
     starts, stops = _events(iters), _events(iters)
     k = 0
     for i in range(iters):
@@ -266,8 +272,10 @@ def cpu_baseline(reps=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--clock-ramp-s", type=float, default=0.2,
+                    help="seconds of untimed steps before the warm-up, so that the GPU is at its sustained clocks")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--quick", action="store_true", help="fewer iterations in the extra measurements")
@@ -284,6 +292,13 @@ def main():
     torch.cuda.set_device(dev)
 
     step = MlpStep(L, dev)
+    # Clock ramp: after idling, the GPU needs about 30 ms of load to reach its sustained clocks (the
+    # first steps run up to twice slower).  Untimed steps bring it there before the W warm-up steps.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < a.clock_ramp_s:
+        for _ in range(10):
+            step.run()
+        torch.cuda.synchronize()
     for _ in range(a.warmup):
         step.run()
     torch.cuda.synchronize()
@@ -313,6 +328,7 @@ def main():
         "vs_baseline": None,
         "dtype": "int8",
         "data": "synthetic",
+        "clock_ramp_s": a.clock_ramp_s,
         "config": {"workload": "BASELINE config 1: Flux MLP W8A8 rowwise, M=4608, 3072->12288->3072, bf16 in/out, bias; "
                                "quantise + GEMM for both projections, inputs resident in HBM"},
         "pct_of_int8_peak": round(100 * value / PEAK_INT8_TOPS, 2),
@@ -324,12 +340,13 @@ def main():
                      "ops_per_launch": step.gemm_ops, "avg_launch_us": round(avg_gemm_us, 2),
                      "launches_timed": len(gemm_us)},
     }
+    extra = extras(L, dev, quick=a.quick) if not a.no_extras else None   # before the CPU leg: the GPU is still warm
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
-    if not a.no_extras:
-        line["extras"] = extras(L, dev, quick=a.quick)
-        if "dit_block_linears" in line["extras"]:
-            line["dit_block_ms"] = line["extras"]["dit_block_linears"]["ms"]
+    if extra is not None:
+        line["extras"] = extra
+        if "dit_block_linears" in extra:
+            line["dit_block_ms"] = extra["dit_block_linears"]["ms"]
     print(json.dumps(line))
 
 

@@ -5,6 +5,7 @@ The package replaces the W8A8 linear hot path of ComfyUI-INT8-Fast:
     int8_fused_kernel   quantise + GEMM + dequant pipeline   (HIP, was Triton)
     int8_quant          quantisation helpers, Int8TensorwiseOps, INT8 LoRA adapters
     quarot              128-block Hadamard rotation
+    compile_ops         torch.library operators (namespace i8f) for torch.compile
     _lib                ctypes binding of libi8f_gfx950.so (include/i8f.h)
     build               hipcc build of the library
 
@@ -14,7 +15,7 @@ tests (see `load_package` in __graft_entry__.py).  ComfyUI's graph nodes (loader
 LoRA loader nodes) are host-application glue and are not part of this package;
 `Int8TensorwiseOps` is the object they would pass as `custom_operations`.
 """
-from . import _lib, int8_fused_kernel, int8_quant, quarot  # noqa: F401
+from . import _lib, compile_ops, int8_fused_kernel, int8_quant, quarot  # noqa: F401
 from .int8_fused_kernel import (  # noqa: F401
     hip_int8_linear,
     hip_int8_linear_per_row,

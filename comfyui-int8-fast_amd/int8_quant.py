@@ -12,7 +12,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from . import _lib
+from . import _lib, compile_ops, int8_fused_kernel
 from ._comfy_compat import (
     LoRAAdapter,
     cast_bias_weight,
@@ -429,7 +429,15 @@ class Int8TensorwiseOps(manual_cast):
             x_2d = x.reshape(-1, x.shape[-1])
             rotate = bool(getattr(self, "_use_quarot", False))
 
-            if x_2d.shape[0] > SMALL_BATCH_ROWS:
+            if torch.compiler.is_compiling():
+                # under torch.compile the same two branches go through the registered operators
+                ws_t, ws_v = compile_ops.split_scale(w_scale)
+                if x_2d.shape[0] > SMALL_BATCH_ROWS:
+                    y = torch.ops.i8f.int8_linear(x_2d, weight, ws_t, ws_v, bias, compute_dtype, rotate,
+                                                  int8_fused_kernel.DEFAULT_EPILOGUE)
+                else:
+                    y = torch.ops.i8f.linear_w8a16_small_m(x_2d, weight, ws_t, ws_v, bias, rotate)
+            elif x_2d.shape[0] > SMALL_BATCH_ROWS:
                 fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
                 y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate)
             else:
@@ -442,7 +450,12 @@ class Int8TensorwiseOps(manual_cast):
                 # as in the reference (int8_quant.py:741-744,768)
                 lA = self.lora_A.to(x.device, non_blocking=True)
                 lB = self.lora_B.to(x.device, non_blocking=True)
-                x_side = _lib.rotate128(x_2d) if rotate else x_2d
+                if not rotate:
+                    x_side = x_2d
+                elif torch.compiler.is_compiling():
+                    x_side = torch.ops.i8f.rotate128(x_2d)
+                else:
+                    x_side = _lib.rotate128(x_2d)
                 side = F.linear(F.linear(x_side.to(lA.dtype), lA), lB)
                 if self.lora_alpha is not None:
                     side = side * self.lora_alpha
