@@ -540,6 +540,7 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6>;   // 8 waves, 2 x 64 KB stages, one workgroup per CU
 using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
+using CfgT64 = Cfg<64, 64, 128, 2, 2, 2, 8>;     // 4 waves of 32 x 32, 2 x 16 KB stages: outputs of few tiles still fill the chip
 
 template <class C, int OUT>
 int launch_cfg(GemmArgs &g, hipStream_t st) {
@@ -568,22 +569,28 @@ int launch(GemmArgs &g, hipStream_t st) {
         hipLaunchKernelGGL((gemm_i8_generic_kernel<OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, g);
         return check_launch();
     }
-    // Tile choice: one workgroup per CU at a time, so a launch costs about
-    // ceil(tiles / 256 CUs) rounds of one tile's work (BM * BN).  Small problems take 128 x 128 tiles,
-    // two workgroups per CU.
+    // Tile choice.  With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
+    // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
+    // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA).  Outputs of fewer than 128
+    // such tiles take 128 x 128 tiles if that gives at least one workgroup per CU, else 64 x 64.
     const int64_t CUS = 256;
-    auto rounds_cost = [&](int bm, int bn) {
+    auto rounds_cost = [&](int bm, int bn, int per_op_cost) {
         const int64_t tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
-        return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn;
+        return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn * per_op_cost;
     };
     const int64_t big_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
 #ifdef I8F_FORCE_CFG  // development probe: one fixed configuration
     if (I8F_FORCE_CFG == 1) return launch_cfg<CfgBig, OUT>(g, st);
     if (I8F_FORCE_CFG == 2) return launch_cfg<CfgB192, OUT>(g, st);
     if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
+    if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64, OUT>(g, st);
 #endif
-    if (big_tiles < 128) return launch_cfg<CfgMid, OUT>(g, st);
-    if (rounds_cost(256, 192) < rounds_cost(256, 256)) return launch_cfg<CfgB192, OUT>(g, st);
+    if (big_tiles < 128) {
+        const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+        if (mid_tiles >= CUS) return launch_cfg<CfgMid, OUT>(g, st);
+        return launch_cfg<CfgT64, OUT>(g, st);
+    }
+    if (rounds_cost(256, 192, 108) < rounds_cost(256, 256, 100)) return launch_cfg<CfgB192, OUT>(g, st);
     return launch_cfg<CfgBig, OUT>(g, st);
 }
 

@@ -105,7 +105,9 @@ def test_weight_prep_matches_oracle_for_rotated_rowwise_weights(L, dev):
 
 # ------------------------------------------------------------------ integer product (a5)
 GEMM_CASES = [(256, 256, 64), (256, 256, 3072), (300, 520, 1040), (128, 128, 128), (100, 72, 48), (64, 64, 50),
-              (1, 8, 16), (17, 3072, 3072), (1024, 768, 12288), (513, 1032, 80), (40, 24, 16), (31, 33, 35), (512, 512, 0)]
+              (1, 8, 16), (17, 3072, 3072), (1024, 768, 12288), (513, 1032, 80), (40, 24, 16), (31, 33, 35), (512, 512, 0),
+              # one ragged case per tile configuration of the fast kernel: 128x128, 256x192, 256x256 (K tails included)
+              (2048, 2048, 256), (2000, 2056, 200), (4100, 2056, 144), (3000, 4104, 80), (3000, 4104, 256)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_CASES)
@@ -141,6 +143,8 @@ LIN_CASES = [
     (256, 256, 512, False, torch.bfloat16, torch.float32, 0), (100, 72, 48, True, torch.float32, torch.bfloat16, 0),
     (17, 3072, 3072, True, torch.bfloat16, torch.bfloat16, 0), (64, 50, 50, True, torch.bfloat16, torch.bfloat16, 0),
     (1030, 264, 272, False, torch.float32, torch.float16, 1), (40, 24, 16, False, None, torch.float16, 1),
+    (2000, 2056, 200, True, torch.bfloat16, torch.bfloat16, 0), (4100, 2056, 144, True, torch.float16, torch.float16, 1),
+    (3000, 4104, 80, False, torch.bfloat16, torch.bfloat16, 0), (3000, 4104, 256, True, None, torch.float32, 1),
 ]
 
 
