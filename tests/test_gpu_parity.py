@@ -107,7 +107,9 @@ def test_weight_prep_matches_oracle_for_rotated_rowwise_weights(L, dev):
 GEMM_CASES = [(256, 256, 64), (256, 256, 3072), (300, 520, 1040), (128, 128, 128), (100, 72, 48), (64, 64, 50),
               (1, 8, 16), (17, 3072, 3072), (1024, 768, 12288), (513, 1032, 80), (40, 24, 16), (31, 33, 35), (512, 512, 0),
               # one ragged case per tile configuration of the fast kernel: 128x128, 256x192, 256x256 (K tails included)
-              (2048, 2048, 256), (2000, 2056, 200), (4100, 2056, 144), (3000, 4104, 80), (3000, 4104, 256)]
+              (2048, 2048, 256), (2000, 2056, 200), (4100, 2056, 144), (3000, 4104, 80), (3000, 4104, 256),
+              # long K, few tiles: the four-stage configurations (128x128, 128x64, 64x64)
+              (1000, 3080, 8200), (500, 3072, 8192), (200, 520, 8320)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_CASES)
