@@ -87,6 +87,23 @@ __device__ __forceinline__ constexpr int waitcnt_vm(int n) {
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
+// One wave-wide global -> LDS load of 16 bytes per lane (lane l lands at lds_base + 16 l), issued
+// from inline assembly on purpose: the compiler knows nothing of an LDS write in flight, so it does
+// not put a full vmcnt(0) wait in front of every later LDS read (it cannot prove that the reads
+// touch another stage).  The waits for these loads are the explicit s_waitcnt of the main loop.
+__device__ __forceinline__ void dma16(v4i rsrc, uint32_t lds_base, uint32_t voffset, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory", "m0");
+}
+
+__device__ __forceinline__ v4i make_rsrc(const void *p, uint32_t bytes) {
+    const uint64_t a = (uint64_t)p;
+    v4i r = {(int)(uint32_t)a, (int)((uint32_t)(a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+    return r;
+}
+
 template <int OUT>
 struct OutElem {
     static constexpr int BYTES = (OUT == OUT_BF16 || OUT == OUT_F16) ? 2 : 4;
@@ -205,8 +222,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // load costs no vector arithmetic; rows beyond the matrix carry an out-of-range vector offset
     // and are zero-filled by the buffer bounds check (which looks at the vector offset only).
     const int K = g.K;
-    __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)((int64_t)g.M * K), 0x00020000);
-    __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)g.w, 0, (int)((int64_t)g.N * K), 0x00020000);
+    const v4i rx = make_rsrc(g.x, (uint32_t)((int64_t)g.M * K));
+    const v4i rw = make_rsrc(g.w, (uint32_t)((int64_t)g.N * K));
     const uint32_t OOB = 0x7ffffff0u;
 
     uint32_t xoff[C::X_LOADS], woff[C::W_LOADS];  // byte offset of this lane's chunk at k-tile 0
@@ -233,29 +250,24 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // `live` false (a tile index past the end, at the tail of the loop) turns every lane's offset
     // out of range: the instruction is still issued, which keeps the loop body free of branches,
     // but moves no data.
-    auto issue = [&](int kt, bool live) {
-        char *st = smem + (kt % S) * C::STAGE_BYTES + wave * 1024;
+    // load r of tile kt: r < X_LOADS fetches a piece of the X tile, the others a piece of the W tile
+    const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
+    auto issue_one = [&](int kt, bool live, int r) {
+        const uint32_t st = smem_base + (kt % S) * C::STAGE_BYTES + wave * 1024;
         const int kb = kt * BK;
-#pragma unroll
-        for (int t = 0; t < C::X_LOADS; ++t) {
-            uint32_t vo = live ? xoff[t] : OOB;
-            int so = kb;
-            if constexpr (KTAIL) {  // chunks past K are forced out of range per lane
-                vo = (kb + xck[t] < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
-                so = 0;
-            }
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(st + t * NW * 1024), 16, vo, so, 0, 0);
+        const bool is_x = r < C::X_LOADS;
+        const int t = is_x ? r : r - C::X_LOADS;
+        uint32_t vo = live ? (is_x ? xoff[t] : woff[t]) : OOB;
+        int so = kb;
+        if constexpr (KTAIL) {  // chunks past K are forced out of range per lane
+            vo = (kb + (is_x ? xck[t] : wck[t]) < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
+            so = 0;
         }
+        dma16(is_x ? rx : rw, st + (is_x ? 0 : C::X_BYTES) + t * NW * 1024, vo, so);
+    };
+    auto issue = [&](int kt, bool live) {
 #pragma unroll
-        for (int t = 0; t < C::W_LOADS; ++t) {
-            uint32_t vo = live ? woff[t] : OOB;
-            int so = kb;
-            if constexpr (KTAIL) {
-                vo = (kb + wck[t] < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
-                so = 0;
-            }
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(st + C::X_BYTES + t * NW * 1024), 16, vo, so, 0, 0);
-        }
+        for (int r = 0; r < C::LOADS; ++r) issue_one(kt, live, r);
     };
 
     // ---- LDS -> register plan ----------------------------------------------------------
@@ -283,24 +295,32 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
     };
-    auto mma = [&](const v4i (&xf)[MI], const v4i (&wf)[NI]) {
-#pragma unroll
-        for (int i = 0; i < MI; ++i)
-#pragma unroll
-            for (int j = 0; j < NI; ++j)
+    // fragment idx of a k-step: the NI W fragments first, then the MI X fragments
+    auto load_frag_one = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI], int idx) {
+        if (idx < NI) wf[idx] = *(const v4i *)(st + wrow_off + idx * 32 * BK + koff[ks]);
+        else xf[idx - NI] = *(const v4i *)(st + xrow_off + (idx - NI) * 32 * BK + koff[ks]);
+    };
+    auto mma_one = [&](const v4i (&xf)[MI], const v4i (&wf)[NI], int r) {
+        const int i = r / NI, j = r % NI;
 #ifndef I8F_ABLATE_MFMA
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
 #else
-                acc[i][j][0] += xf[i][0] ^ wf[j][0];
+        acc[i][j][0] += xf[i][0] ^ wf[j][0];
 #endif
     };
 
     // ---- prologue: S tiles in flight, fragments of the first k-step in registers --------------
+    // Two ways to keep the stages full.  With two stages a stage is refilled in one burst, right
+    // after the barrier that frees it (tile kt+S during the last phase of iteration kt).  With three
+    // or more the refill of the stage freed by the PREVIOUS iteration is dealt out over the whole of
+    // iteration kt (tile kt+S-1): a wave that issues many loads at once blocks on the load queue, and
+    // while it is blocked it issues no MFMAs either.  Loads past the last tile are issued all the
+    // same (they move nothing), so the number of loads in flight at any point is a constant.
+    constexpr bool SPREAD_DMA = S >= 3;
+    constexpr int PRE = SPREAD_DMA ? S - 1 : S;  // tiles issued before the loop
 #pragma unroll
-    for (int s = 0; s < S; ++s)
-        if (s < KT) issue(s, true);
-    if (KT >= S) __builtin_amdgcn_s_waitcnt(waitcnt_vm((S - 1) * C::LOADS));  // tiles 1..S-1 may be in flight
-    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    for (int s = 0; s < PRE; ++s) issue(s, s < KT);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((PRE - 1) * C::LOADS));  // tiles 1..PRE-1 may be in flight
     __syncthreads();  // tile 0 and the staged epilogue operands are visible to everyone
 #ifdef I8F_TRACE
     if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 1] = wall_clock64();
@@ -326,55 +346,57 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const bool last = ks == KS - 1;
+            constexpr int MN = MI * NI, NF = MI + NI;
             if (last) {
-                // my part of tile kt+1 has landed (tiles kt+2 .. kt+S-1 may still be in flight) and
-                // my LDS reads of tile kt have returned
-                if (kt + S - 1 < KT) __builtin_amdgcn_s_waitcnt(waitcnt_vm((S - 2) * C::LOADS) & 0xF0FF);
-                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0) & 0xF0FF);
+                // my part of tile kt+1 has landed and my LDS reads of tile kt have returned; what may
+                // still be in flight are the younger tiles (and, spread, the part of the newest one
+                // that the earlier phases of this iteration have issued)
+                constexpr int YOUNGER = SPREAD_DMA ? (S - 3) * C::LOADS + (KS - 1) * C::LOADS / KS : (S - 2) * C::LOADS;
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm(YOUNGER) & 0xF0FF);
                 __builtin_amdgcn_s_barrier();
             }
             v4i(&xc)[MI] = (ks & 1) ? xb : xa;
             v4i(&wc)[NI] = (ks & 1) ? wb : wa;
             v4i(&xn)[MI] = (ks & 1) ? xa : xb;
             v4i(&wn_)[NI] = (ks & 1) ? wa : wb;
+            // One wave per SIMD (4 waves with large wave tiles): nothing but this wave feeds the
+            // matrix pipe, so its LDS reads are dealt out between the MFMAs as well instead of being
+            // issued in a burst in front of them.
+            constexpr bool SPREAD_LDS = (NW == 4 && MN >= 8);
             // past the last tile the next-fragment reads fetch stale LDS that nobody uses
-            if (!last) load_frags(st, ks + 1, xn, wn_);
-            else load_frags(nx, 0, xn, wn_);
+            const char *fsrc = last ? nx : st;
+            const int fks = last ? 0 : ks + 1;
+            if constexpr (!SPREAD_LDS) load_frags(fsrc, fks, xn, wn_);
+            __builtin_amdgcn_sched_barrier(0);
+            const int ft = SPREAD_DMA ? kt + S - 1 : kt + S;  // the tile being fetched
+            const bool live = ft < KT;
+            (void)live;
+            // this phase's share of its loads: all of them in the last phase (burst), 1/KS of them (spread)
+            const int la = SPREAD_DMA ? ks * C::LOADS / KS : 0;
+            const int lb = SPREAD_DMA ? (ks + 1) * C::LOADS / KS : (last ? C::LOADS : 0);
+#pragma unroll
+            for (int r = 0; r < MN; ++r) {
+                mma_one(xc, wc, r);
 #ifndef I8F_ABLATE_DMA
-            if (last) issue(kt + S, kt + S < KT);  // refills the stage tile kt was in
-#endif
-            mma(xc, wc);
-            // Issue order inside the phase: all LDS reads of the NEXT k-step first, so that they
-            // complete under this phase's MFMAs; in the last phase the global loads of tile kt+S
-            // are spread between the MFMAs.
-#ifndef I8F_SCHED
-#define I8F_SCHED 0
-#endif
-            if constexpr (I8F_SCHED == 0) {  // all LDS reads first
-                __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-                if (last) {
 #pragma unroll
-                    for (int r = 0; r < C::LOADS; ++r) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                    }
-                    if (MI * NI > C::LOADS) __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - C::LOADS, 0);
-                } else {
-                    __builtin_amdgcn_sched_group_barrier(0x008, MI * NI, 0);
-                }
-            } else {  // one LDS read after each of the first MFMAs (and one global load in the last phase)
+                for (int l = la + r * (lb - la) / MN; l < la + (r + 1) * (lb - la) / MN; ++l) issue_one(ft, live, l);
+#endif
+                if constexpr (SPREAD_LDS) {
+#ifndef I8F_ABLATE_LDSREAD
 #pragma unroll
-                for (int r = 0; r < MI * NI; ++r) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    if (r < MI + NI) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    if (last && r < C::LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    for (int f = r * NF / MN; f < (r + 1) * NF / MN; ++f) load_frag_one(fsrc, fks, xn, wn_, f);
+#endif
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     }
 
     // ---- epilogue ----------------------------------------------------------------------
+    // The loads issued past the last tile move no data from memory but still zero-fill their LDS
+    // destination: they must have landed before the stages are reused.
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();  // the stages are dead; reuse them as per-wave transpose buffers
 #ifdef I8F_TRACE
     if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 2] = wall_clock64();
@@ -590,6 +612,10 @@ int launch(GemmArgs &g, hipStream_t st) {
     if (I8F_FORCE_CFG == 2) return launch_cfg<CfgB192, OUT>(g, st);
     if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
     if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64, OUT>(g, st);
+    if (I8F_FORCE_CFG == 5) return launch_cfg<Cfg<256, 256, 128, 2, 2, 2, 6>, OUT>(g, st);
+    if (I8F_FORCE_CFG == 6) return launch_cfg<Cfg<256, 256, 64, 2, 4, 4, 6>, OUT>(g, st);
+    if (I8F_FORCE_CFG == 7) return launch_cfg<Cfg<256, 256, 64, 2, 2, 4, 6>, OUT>(g, st);
+    if (I8F_FORCE_CFG == 8) return launch_cfg<Cfg<256, 256, 64, 2, 4, 3, 6>, OUT>(g, st);
 #endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
