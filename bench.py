@@ -79,10 +79,10 @@ def make_config(i: int, rows: int | None = None) -> dict:
 
 # HBM-side bytes per GEMM launch of config 1, from two rocprofv3 --pmc runs of
 # comfyui-int8-fast_amd/profiling/traffic_probe.py (summary in profiles/hbm_traffic_fetch_write_size.txt):
-# FETCH_SIZE 189790 KiB / WRITE_SIZE 110592 KiB for 4608x12288x3072 and 153780 / 27648 KiB for
+# FETCH_SIZE 139354 KiB / WRITE_SIZE 110592 KiB for 4608x12288x3072 and 153783 / 27648 KiB for
 # 4608x3072x12288; a 256 MiB device copy reads 131084 / 262144 KiB on the same counters, so fetches
 # scale by 2.00 and writes by 1.00.  The mean of the two launches:
-GEMM_TRAFFIC_BYTES = int(((189790 * 2.0 + 110592) + (153780 * 2.0 + 27648)) / 2 * 1024)
+GEMM_TRAFFIC_BYTES = int(((139354 * 2.0 + 110592) + (153783 * 2.0 + 27648)) / 2 * 1024)
 
 
 # --------------------------------------------------------------------------- timing helpers
