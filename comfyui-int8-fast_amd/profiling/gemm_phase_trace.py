@@ -57,9 +57,16 @@ def main():
         BM, BN = (int(v) for v in a.tile.split("x"))
     else:   # the host-side choice of gemm_i8.hip
         cd = lambda p, q: (p + q - 1) // q
-        big = cd(M, 256) * cd(N, 256)
-        cost = lambda bm, bn: cd(cd(M, bm) * cd(N, bn), 256) * bm * bn
-        BM, BN = (128, 128) if big < 128 else ((256, 192) if cost(256, 192) < cost(256, 256) else (256, 256))
+        big, mid = cd(M, 256) * cd(N, 256), cd(M, 128) * cd(N, 128)
+        cost = lambda bm, bn, per_op: cd(cd(M, bm) * cd(N, bn), 256) * bm * bn * per_op
+        if big >= 128:
+            BM, BN = (256, 192) if cost(256, 192, 108) < cost(256, 256, 100) else (256, 256)
+        elif mid >= 256 or (K >= 8192 and mid >= 192):
+            BM, BN = 128, 128
+        elif K >= 8192 and cd(M, 128) * cd(N, 64) >= 192:
+            BM, BN = 128, 64
+        else:
+            BM, BN = 64, 64
     dev = torch.device("cuda:0")
     x, w = operands(M, N, K, a.data, dev)
     xs, ws = torch.rand(M, device=dev) * 0.01, torch.rand(N, device=dev) * 0.01
