@@ -486,7 +486,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #else
                 if (mm < g.M && nn < g.N)
 #endif
-                    *(uint4 *)((char *)g.out + ((int64_t)mm * g.N + nn) * OB) = val;
+                    stream_store16((char *)g.out + ((int64_t)mm * g.N + nn) * OB, val);
             }
             __builtin_amdgcn_wave_barrier();
 #ifdef I8F_TRACE

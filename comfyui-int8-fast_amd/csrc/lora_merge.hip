@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void lora_merge_kernel(const MergeArgs a) {
         uint32_t o = 0;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o |= ((uint32_t)q[e] & 0xffu) << (8 * e);
-        *(uint32_t *)(a.out + base) = o;
+        stream_store4(a.out + base, o);
     } else {
         if (a.w) q[0] = sat8((int)a.w[base] + q[0]);
         a.out[base] = (int8_t)q[0];
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void lora_merge_band_kernel(const MergeArgs a,
             const int wv = (int)(int8_t)(wp_cur >> (8 * e));
             o |= ((uint32_t)sat8(wv + dq) & 0xffu) << (8 * e);
         }
-        *(uint32_t *)(a.out + n * a.K + k0) = o;
+        stream_store4(a.out + n * a.K + k0, o);
     }
 }
 

@@ -157,7 +157,7 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void quant_rows_kernel(
                 packed[j] = w;
             }
             if constexpr (EPC == 8) {
-                *(uint2 *)(qrow + (int64_t)c * 8) = make_uint2(packed[0], packed[1]);
+                stream_store8(qrow + (int64_t)c * 8, make_uint2(packed[0], packed[1]));
             } else {
                 *(uint32_t *)(qrow + (int64_t)c * 4) = packed[0];
             }
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
                     o.y = quant4_magic(v[r][4], v[r][5], v[r][6], v[r][7], inv);
                     o.z = quant4_magic(v[r][8], v[r][9], v[r][10], v[r][11], inv);
                     o.w = quant4_magic(v[r][12], v[r][13], v[r][14], v[r][15], inv);
-                    *(uint4 *)(qrow + (int64_t)R * 16) = o;
+                    stream_store16(qrow + (int64_t)R * 16, o);
                 }
             }
             if (t == 0) scale[m] = s;
@@ -477,7 +477,7 @@ __device__ __forceinline__ void store_chunk(void *p, const float (&v)[Elem<DT>::
             if constexpr (DT == I8F_BF16) w[j] = f32x2_to_bf16x2_bits(v[2 * j], v[2 * j + 1]);
             else w[j] = f32x2_to_f16x2_bits(v[2 * j], v[2 * j + 1]);
         }
-        *(uint4 *)p = make_uint4(w[0], w[1], w[2], w[3]);
+        stream_store16(p, make_uint4(w[0], w[1], w[2], w[3]));
     }
 }
 
