@@ -18,6 +18,7 @@ import argparse
 import ctypes
 import os
 import sys
+import time
 
 import numpy as np
 import torch
@@ -75,15 +76,23 @@ def main():
     tr = torch.zeros(nblk * 8, dtype=torch.int64, device=dev)
     os.environ["I8F_TRACE_PTR"] = str(tr.data_ptr())
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(4):
-        tr.zero_()
-        torch.cuda.synchronize()
-        e0.record()
+    # the stamps read back are those of the LAST launch of a back-to-back series that is long enough
+    # for the GPU to reach its sustained clocks (about 30 ms after idle); every launch overwrites them
+    def launch():
         rc = lib.i8f_linear_w8a8(x.data_ptr(), xs.data_ptr(), w.data_ptr(), ws.data_ptr(), 0.0, 1, None, 0,
                                  out.data_ptr(), 0, M, N, K, 0, None)
-        e1.record()
-        torch.cuda.synchronize()
         assert rc == 0, rc
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.1:
+        for _ in range(20):
+            launch()
+        torch.cuda.synchronize()
+    for _ in range(50):
+        launch()
+    e0.record()
+    launch()
+    e1.record()
+    torch.cuda.synchronize()
     t = tr.cpu().numpy().reshape(nblk, 8).astype(np.float64) * 10e-3     # 100 MHz ticks -> microseconds
     if not t[:, 3].all():
         sys.exit("some workgroups left no stamp: --tile does not match what the library launched")
