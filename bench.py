@@ -170,7 +170,7 @@ def extras(L, dev, quick=False):
                                           "tops": round(tops, 1), "frac_of_int8_peak": round(tops / PEAK_INT8_TOPS, 4)}
 
     # fused rotate + quant at the same shape, cycling 8 buffer sets (> 256 MB in total), bursts of 8
-    # launches per event pair; a plain device copy of the same byte count is the practical ceiling
+    # launches per event pair; a plain device copy of the same byte count is timed beside them
     sets = 8
     xs = [x] + [_acts(g, M, K, 0.01, 20.0).to(dev) for _ in range(sets - 1)]
     qs = [torch.empty(M, K, dtype=torch.int8, device=dev) for _ in range(sets)]
@@ -191,7 +191,7 @@ def extras(L, dev, quick=False):
     dsts = [torch.empty(half, dtype=torch.uint8, device=dev) for _ in range(sets)]
     t = time_kernel(lambda i: dsts[i].copy_(srcs[i]), reps, sets=sets, burst=sets)
     out["device_copy_same_bytes"] = {"median_us": round(t["median_us"], 2), "gbs": round(2 * half / t["median_us"] / 1e3, 1),
-                                     "note": "torch copy_ of 21.2 MB -> 21.2 MB, same rotation of buffers: the practical HBM ceiling at this size"}
+                                     "note": "torch copy_ of 21.2 MB -> 21.2 MB over the same rotation of buffers, for comparison"}
     del xs, qs, ss, srcs, dsts
 
     # config 4: stochastic LoRA merge (rank 32 rebuilt in the kernel, float noise) and the skinny GEMM

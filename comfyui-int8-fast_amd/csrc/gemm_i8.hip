@@ -295,11 +295,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
     };
-    // fragment idx of a k-step: the NI W fragments first, then the MI X fragments
-    auto load_frag_one = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI], int idx) {
-        if (idx < NI) wf[idx] = *(const v4i *)(st + wrow_off + idx * 32 * BK + koff[ks]);
-        else xf[idx - NI] = *(const v4i *)(st + xrow_off + (idx - NI) * 32 * BK + koff[ks]);
-    };
     auto mma_one = [&](const v4i (&xf)[MI], const v4i (&wf)[NI], int r) {
         const int i = r / NI, j = r % NI;
 #ifndef I8F_ABLATE_MFMA
@@ -346,7 +341,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const bool last = ks == KS - 1;
-            constexpr int MN = MI * NI, NF = MI + NI;
+            constexpr int MN = MI * NI;
             if (last) {
                 // my part of tile kt+1 has landed and my LDS reads of tile kt have returned; what may
                 // still be in flight are the younger tiles (and, spread, the part of the newest one
@@ -359,14 +354,10 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
             v4i(&wc)[NI] = (ks & 1) ? wb : wa;
             v4i(&xn)[MI] = (ks & 1) ? xa : xb;
             v4i(&wn_)[NI] = (ks & 1) ? wa : wb;
-            // One wave per SIMD (4 waves with large wave tiles): nothing but this wave feeds the
-            // matrix pipe, so its LDS reads are dealt out between the MFMAs as well instead of being
-            // issued in a burst in front of them.
-            constexpr bool SPREAD_LDS = (NW == 4 && MN >= 8);
             // past the last tile the next-fragment reads fetch stale LDS that nobody uses
             const char *fsrc = last ? nx : st;
             const int fks = last ? 0 : ks + 1;
-            if constexpr (!SPREAD_LDS) load_frags(fsrc, fks, xn, wn_);
+            load_frags(fsrc, fks, xn, wn_);
             __builtin_amdgcn_sched_barrier(0);
             const int ft = SPREAD_DMA ? kt + S - 1 : kt + S;  // the tile being fetched
             const bool live = ft < KT;
@@ -381,12 +372,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
                 for (int l = la + r * (lb - la) / MN; l < la + (r + 1) * (lb - la) / MN; ++l) issue_one(ft, live, l);
 #endif
-                if constexpr (SPREAD_LDS) {
-#ifndef I8F_ABLATE_LDSREAD
-#pragma unroll
-                    for (int f = r * NF / MN; f < (r + 1) * NF / MN; ++f) load_frag_one(fsrc, fks, xn, wn_, f);
-#endif
-                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -612,10 +597,6 @@ int launch(GemmArgs &g, hipStream_t st) {
     if (I8F_FORCE_CFG == 2) return launch_cfg<CfgB192, OUT>(g, st);
     if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
     if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64, OUT>(g, st);
-    if (I8F_FORCE_CFG == 5) return launch_cfg<Cfg<256, 256, 128, 2, 2, 2, 6>, OUT>(g, st);
-    if (I8F_FORCE_CFG == 6) return launch_cfg<Cfg<256, 256, 64, 2, 4, 4, 6>, OUT>(g, st);
-    if (I8F_FORCE_CFG == 7) return launch_cfg<Cfg<256, 256, 64, 2, 2, 4, 6>, OUT>(g, st);
-    if (I8F_FORCE_CFG == 8) return launch_cfg<Cfg<256, 256, 64, 2, 4, 3, 6>, OUT>(g, st);
 #endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
