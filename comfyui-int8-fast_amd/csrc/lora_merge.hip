@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void lora_merge_kernel(const MergeArgs a) {
     }
 }
 
-// Fused low-rank form, the fast kernel.  A thread owns 4 consecutive columns and keeps the RANK x 4
+// Fused low-rank form on the vector ALUs (K not a multiple of 32).  A thread owns 4 consecutive columns and keeps the RANK x 4
 // slice of `down` it needs in registers for the whole kernel; the block then walks a band of rows.
 // Per row and thread that leaves 16 bytes of noise and 4 bytes of weight to read, 4 bytes to write,
 // and the row of `up`, which is the same for every lane and comes through scalar loads.  (Indexing
@@ -161,6 +161,130 @@ __global__ __launch_bounds__(256) void lora_merge_band_kernel(const MergeArgs a,
     }
 }
 
+// The same fused form on the matrix cores.  v_mfma_f32_32x32x2_f32 adds two products per output to
+// its accumulator, the k = 0 product first and each with a single rounding, so a sequence of them
+// over j = (0,1), (2,3), ... is the fma chain in increasing j of the definition above, bit for bit
+// (checked against the CPU oracle by the parity tests).  The output block is computed transposed,
+// D[k][n] = sum_j down[j][k] * up[n][j]: a lane then holds, for ONE weight row n, four groups of
+// four consecutive k, so the rounding step works on 16-byte noise and 4-byte weight pieces.
+//
+// A workgroup of 8 waves owns 256 columns and walks a band of rows in blocks of 32.  Its threads
+// fetch a block row by row (one wave instruction = 1 KB of one noise row) into an LDS tile, from
+// which every wave takes the 32 x 32 piece of its own 32 columns in the layout above; results go
+// back through the tile so that they leave in 256-byte runs.  Each wave keeps its slice of `down`
+// in RANK/2 registers; `up` is fetched once per block for all eight waves.  The operands of the
+// next block are in flight while this one is computed.
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int RANK>
+struct MfmaMergeLds {
+    static constexpr int WAVES = 8, COLS = WAVES * 32;
+    static constexpr int NZ_PITCH = COLS * 4 + 16;   // 260 words: the column reads of 16 rows hit 16 different bank groups
+    static constexpr int UP_PITCH = RANK * 4 + 4;
+    static constexpr int WB_PITCH = COLS + 16;
+    static constexpr int NZ = 0, UP = NZ + 32 * NZ_PITCH, WB = UP + ((32 * UP_PITCH + 15) / 16) * 16;
+    static constexpr int BYTES = WB + 32 * WB_PITCH;
+};
+
+template <int RANK>
+__global__ __launch_bounds__(512) void lora_merge_mfma_kernel(const MergeArgs a, int blocks_per_band) {
+    using T = MfmaMergeLds<RANK>;
+    __shared__ __attribute__((aligned(16))) char lds[T::BYTES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int64_t k0 = (int64_t)blockIdx.x * T::COLS;     // first column of the workgroup (K % 32 == 0 here)
+    const int64_t kbase = k0 + wave * 32;                  // first column of this wave
+    const bool wave_live = kbase < a.K;
+    float da[RANK / 2];
+#pragma unroll
+    for (int p = 0; p < RANK / 2; ++p) da[p] = wave_live ? a.down[(int64_t)(2 * p + half) * a.K + kbase + l32] : 0.0f;
+
+    const int64_t nblocks = (a.N + 31) / 32;
+    const int64_t nb_begin = (int64_t)blockIdx.y * blocks_per_band;
+    const int64_t nb_end = nb_begin + blocks_per_band < nblocks ? nb_begin + blocks_per_band : nblocks;
+
+    // what a thread fetches of a block: 4 pieces of noise (piece c = tid + 512 i: row c / 64, 16-byte
+    // column c % 64), one 16-byte piece of weight (row tid / 16, column tid % 16) and, threads below
+    // 8 RANK, one 16-byte piece of the contiguous 32 x RANK block of `up`
+    constexpr int UP_THREADS = 32 * RANK / 4;
+    const bool nz_col_ok = k0 + (tid & 63) * 4 < a.K, wb_col_ok = k0 + (tid & 15) * 16 < a.K;
+    auto clampn = [&](int64_t n) { return n < a.N ? n : a.N - 1; };  // rows past the end repeat the last one, unstored
+    auto fetch = [&](int64_t nb, v4f (&nz)[4], v4f &up, v4u_t &wb, float &sc) __attribute__((always_inline)) {
+        const int64_t n0 = nb * 32;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (nz_col_ok) nz[i] = *(const v4f *)(a.noise + clampn(n0 + (tid >> 6) + 8 * i) * a.K + k0 + (tid & 63) * 4);
+        if (tid < UP_THREADS) up = *(const v4f *)(a.up + clampn(n0 + tid * 4 / RANK) * RANK + (tid * 4) % RANK);
+        if (wb_col_ok) wb = *(const v4u_t *)(a.w + clampn(n0 + (tid >> 4)) * a.K + k0 + (tid & 15) * 16);
+        sc = a.ws ? a.ws[a.row_scale ? clampn(n0 + l32) : 0] : a.ws_host;
+    };
+
+    v4f nz_r[4] = {}, up_r = {};
+    v4u_t wb_r = {};
+    float sc_r = 1.0f;
+    if (nb_begin < nb_end) fetch(nb_begin, nz_r, up_r, wb_r, sc_r);
+    for (int64_t nb = nb_begin; nb < nb_end; ++nb) {
+        // registers -> LDS tile; the same registers then receive the next block
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(v4f *)(lds + T::NZ + ((tid >> 6) + 8 * i) * T::NZ_PITCH + (tid & 63) * 16) = nz_r[i];
+        if (tid < UP_THREADS) {
+            float *dst = (float *)(lds + T::UP + (tid * 4 / RANK) * T::UP_PITCH + ((tid * 4) % RANK) * 4);
+            dst[0] = up_r.x, dst[1] = up_r.y, dst[2] = up_r.z, dst[3] = up_r.w;
+        }
+        *(v4u_t *)(lds + T::WB + (tid >> 4) * T::WB_PITCH + (tid & 15) * 16) = wb_r;
+        const float sc = sc_r;
+        __syncthreads();
+        if (nb + 1 < nb_end) fetch(nb + 1, nz_r, up_r, wb_r, sc_r);
+
+        v16f acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+        for (int p = 0; p < RANK / 2; ++p) {
+            const float u = *(const float *)(lds + T::UP + l32 * T::UP_PITCH + (2 * p + half) * 4);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(da[p], u, acc, 0, 0, 0);
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const v4f nz = *(const v4f *)(lds + T::NZ + l32 * T::NZ_PITCH + wave * 128 + (2 * q + half) * 16);
+            const uint32_t wp = *(const uint32_t *)(lds + T::WB + l32 * T::WB_PITCH + wave * 32 + 8 * q + 4 * half);
+            const float nzv[4] = {nz.x, nz.y, nz.z, nz.w};
+            o[q] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int dq = sr_one(acc[4 * q + e] * a.lora_scale, sc, nzv[e]);
+                const int wv = (int)(int8_t)(wp >> (8 * e));
+                o[q] |= ((uint32_t)sat8(wv + dq) & 0xffu) << (8 * e);
+            }
+        }
+        // results: back through the weight tile (each lane overwrites exactly the bytes it read),
+        // then one 16-byte store per thread
+#pragma unroll
+        for (int q = 0; q < 4; ++q) *(uint32_t *)(lds + T::WB + l32 * T::WB_PITCH + wave * 32 + 8 * q + 4 * half) = o[q];
+        __syncthreads();
+        const v4u_t obv = *(const v4u_t *)(lds + T::WB + (tid >> 4) * T::WB_PITCH + (tid & 15) * 16);
+        const int64_t nrow = nb * 32 + (tid >> 4);
+        if (nrow < a.N && wb_col_ok) stream_store16(a.out + nrow * a.K + k0 + (tid & 15) * 16, make_uint4(obv.x, obv.y, obv.z, obv.w));
+        __syncthreads();  // the tile is free for the next block
+    }
+}
+
+template <int RANK>
+int launch_mfma(const MergeArgs &a, hipStream_t st) {
+    const unsigned col_blocks = (unsigned)((a.K + 255) / 256);
+    const int64_t nblocks = (a.N + 31) / 32;
+    const int64_t target_wgs = 256 * 12;  // short bands: several workgroups per CU take turns at the barriers
+    int64_t bands = (target_wgs + col_blocks - 1) / col_blocks;
+    int64_t per = (nblocks + bands - 1) / bands;
+    if (per < 2) per = 2;
+    bands = (nblocks + per - 1) / per;
+    if (bands > 65535) return I8F_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((lora_merge_mfma_kernel<RANK>), dim3(col_blocks, (unsigned)bands), dim3(512), 0, st, a, (int)per);
+    return check_launch();
+}
+
 template <int RANK>
 int launch_band(const MergeArgs &a, hipStream_t st) {
     const unsigned col_blocks = (unsigned)((a.K + 1023) / 1024);
@@ -181,6 +305,15 @@ int run(MergeArgs &a, hipStream_t st) {
     auto al = [](const void *p, int n) { return p == nullptr || (uintptr_t)p % n == 0; };
     const bool vec = a.K % 4 == 0 && al(a.w, 4) && al(a.out, 4) && al(a.noise, 16) && al(a.delta, 16) &&
                      (!fused || al(a.down, 16));
+    if (fused && vec && a.w && a.N < (1ll << 31) && a.K % 32 == 0 && al(a.up, 16) && al(a.w, 16) && al(a.out, 16)) {
+        switch (a.rank) {
+        case 4: return launch_mfma<4>(a, st);
+        case 8: return launch_mfma<8>(a, st);
+        case 16: return launch_mfma<16>(a, st);
+        case 32: return launch_mfma<32>(a, st);
+        default: break;
+        }
+    }
     if (fused && vec && a.w && a.N < (1ll << 31)) {
         switch (a.rank) {
         case 4: return launch_band<4>(a, st);

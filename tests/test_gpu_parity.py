@@ -283,7 +283,9 @@ def test_small_m_w8a16_within_tolerance(L, dev, M, N, K, dt, rel, absf):
 
 
 # ------------------------------------------------------------------ stochastic merge (a9, a10, a11)
-@pytest.mark.parametrize("N,K,r,row", [(256, 1024, 32, True), (100, 77, 8, False), (512, 3072, 32, True), (3, 5, 1, True), (64, 130, 256, False)])
+@pytest.mark.parametrize("N,K,r,row", [(256, 1024, 32, True), (100, 77, 8, False), (512, 3072, 32, True), (3, 5, 1, True), (64, 130, 256, False),
+                                          (100, 96, 8, True), (70, 128, 4, False), (33, 64, 16, True), (1, 32, 32, True),
+                                          (64, 100, 8, True), (300, 544, 32, True), (96, 288, 16, False)])
 def test_lora_merge_bit_exact(L, dev, N, K, r, row):
     w = i8(N, K)
     ws = torch.rand(N if row else 1, generator=G) * 0.002 + 0.0005
