@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void lora_merge_band_kernel(const MergeArgs a,
 // The same fused form on the matrix cores.  v_mfma_f32_32x32x2_f32 adds two products per output to
 // its accumulator, the k = 0 product first and each with a single rounding, so a sequence of them
 // over j = (0,1), (2,3), ... is the fma chain in increasing j of the definition above, bit for bit
-// (checked against the CPU oracle by the parity tests).  The output block is computed transposed,
+// (the parity tests check this against a CPU fmaf chain).  The output block is computed transposed,
 // D[k][n] = sum_j down[j][k] * up[n][j]: a lane then holds, for ONE weight row n, four groups of
 // four consecutive k, so the rounding step works on 16-byte noise and 4-byte weight pieces.
 //
