@@ -167,3 +167,33 @@ def test_quantize_helpers_on_device(pkg, dev):
     assert s3.shape == (3, 5, 1) and np.array_equal(q3.cpu().numpy().reshape(15, 64), qo3)
     r = pkg.quarot.rotate_activation(x3[..., :128].contiguous() if x3.shape[-1] >= 128 else torch.randn(2, 3, 128, device=dev))
     assert r.shape[-1] == 128
+
+
+@pytest.mark.parametrize("rows", [64, 8])
+def test_forward_under_hip_graph_replays_like_eager(pkg, dev, rows):
+    """The library allocates nothing, synchronises nothing and launches on the caller's stream, so a
+    forward can be captured in a HIP graph.  Every replay, with new input contents and eager work in
+    between, must give the eager result bit for bit."""
+    ops = pkg.Int8TensorwiseOps
+    ops.dynamic_quantize, ops.enable_quarot = True, True
+    w = (torch.randn(256, 384, generator=G) * 0.02).bfloat16()
+    b = (torch.randn(256, generator=G) * 0.01).bfloat16()
+    lin = load(ops.Linear(384, 256, bias=True), {"l.weight": w, "l.bias": b}).to(dev)
+    static_x = torch.zeros(rows, 384, dtype=torch.bfloat16, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            lin(static_x)                       # warm-up outside the capture (library load, device check)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = lin(static_x)
+    for i in range(4):
+        x = torch.randn(rows, 384, generator=G).bfloat16().to(dev) * (i + 1)
+        want = lin(x)                           # eager work between the replays
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y.view(torch.int16), want.view(torch.int16)), f"replay {i}"
