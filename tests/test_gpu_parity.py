@@ -239,6 +239,30 @@ def test_config2_quarot_full_size_and_error_vs_bf16(L, dev):
     assert err_rot < 0.5 * err_plain and err_rot < 0.03       # the rotation is what makes the outliers quantisable
 
 
+def test_config3_dit_block_linears_full_size(L, dev):
+    """Every W8A8 linear of the double-stream block (image stream M = 4096, text stream M = 512) and the
+    adaLN projection at M = 1: the first two run through each tile configuration the host picks for them."""
+    c = make_config(3)
+    g = torch.Generator().manual_seed(1003)
+    for name in ("qkv", "proj", "up", "down"):
+        n_out, k_in = c["linears"][name]
+        w = torch.randn(n_out, k_in, generator=g) * 0.02
+        b = (torch.randn(n_out, generator=g) * 0.01).bfloat16()
+        wq, ws = L.quant_rowwise(w.to(dev))
+        for m in (c["img"], c["txt"]):
+            x = acts(m, k_in)
+            rows = torch.randperm(m, generator=G)[:12].sort().values
+            _check_rows(L, dev, x, wq, ws, b, rows)
+    n_out, k_in = c["linears"]["adaln"]
+    w = torch.randn(n_out, k_in, generator=g) * 0.02
+    wq, ws = L.quant_rowwise(w.to(dev))
+    vec = torch.randn(1, k_in, generator=g).bfloat16()
+    y = L.linear_w8a16_small_m(vec.to(dev), wq, ws, None).float().cpu().numpy()
+    xa, code = O.from_torch(vec)
+    ref = O.to_f32(O.linear_w8a16(xa, code, wq.cpu().numpy(), ws.cpu().numpy()), code)
+    assert np.all(np.abs(y - ref) <= 2.0**-7 * np.abs(ref) + 2.0**-8 * np.abs(ref).max())
+
+
 def test_config4_merge_full_size_then_skinny_gemm(L, dev):
     c = make_config(4)
     wq, ws = L.quant_rowwise(c["w"].to(dev))
