@@ -119,6 +119,20 @@ def test_gemm_i32_bit_exact(L, dev, M, N, K):
     assert np.array_equal(acc.cpu().numpy(), O.gemm_i32(a.numpy(), w.numpy()))
 
 
+def test_gemm_i32_random_shapes(L, dev):
+    """40 seeded random shapes, ragged in every dimension, spread over all tile configurations."""
+    rng = np.random.default_rng(20240)
+    for _ in range(40):
+        M = int(rng.integers(1, 2600))
+        N = int(rng.integers(1, 330)) * 8 if rng.random() < 0.8 else int(rng.integers(1, 2600))
+        K = int(rng.integers(1, 80)) * 16 if rng.random() < 0.8 else int(rng.integers(1, 1300))
+        if rng.random() < 0.15:
+            K = int(rng.integers(512, 640)) * 16            # long K: the four-stage configurations
+        a, w = i8(M, K), i8(N, K)
+        acc = L.gemm_i32(a.to(dev), w.to(dev))
+        assert np.array_equal(acc.cpu().numpy(), O.gemm_i32(a.numpy(), w.numpy())), (M, N, K)
+
+
 def test_gemm_i32_saturating_inputs_at_largest_k(L, dev):
     K = 12288
     a = torch.full((64, K), -128, dtype=torch.int8)
