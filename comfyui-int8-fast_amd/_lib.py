@@ -54,10 +54,11 @@ def lib() -> ctypes.CDLL:
     L.i8f_rotate128.argtypes = [vp, i32, i64, i64, i64, vp, vp]
     L.i8f_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp, vp]
     L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
+    L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8",
+    for name in ("i8f_quant_rowwise", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -66,7 +67,7 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
-    "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+    "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
 
@@ -193,8 +194,9 @@ def _bias_arg(bias, N, device):
     return bias, dtype_code(bias.dtype)
 
 
-def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None):
-    """Quantised activations (a int8 [M,K], a_scale [M,1]) times int8 weight [N,K] with the fused dequant epilogue."""
+def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None, addend=None):
+    """Quantised activations (a int8 [M,K], a_scale [M,1]) times int8 weight [N,K] with the fused dequant epilogue.
+    addend ([M,N] of the output dtype) is added to the rounded result in the epilogue and the sum rounded again."""
     a, w = _i8_matrix(a, "a"), _i8_matrix(w, "w")
     M, K = a.shape
     N, K2 = w.shape
@@ -209,9 +211,15 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
     bias, bcode = _bias_arg(bias, N, a.device)
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    if addend is not None:
+        _dev(addend, "addend")
+        if addend.numel() != M * N or addend.dtype != out.dtype:
+            raise ValueError(f"addend must have {M * N} elements of {out.dtype}")
+        addend = addend.reshape(M, N).contiguous()
     with torch.cuda.device(a.device):
-        _check(lib().i8f_linear_w8a8(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
-                                     _ptr(out), dtype_code(out.dtype), M, N, K, order, _stream(a)), "i8f_linear_w8a8")
+        _check(lib().i8f_linear_w8a8_add(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
+                                         _ptr(addend), _ptr(out), dtype_code(out.dtype), M, N, K, order, _stream(a)),
+               "i8f_linear_w8a8_add")
     return out
 
 

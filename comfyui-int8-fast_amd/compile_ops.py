@@ -65,16 +65,19 @@ def _(a, a_scale, weight, weight_scale, weight_scale_value, bias, out_dtype, ord
 
 @torch.library.custom_op(f"{NAMESPACE}::int8_linear", mutates_args=())
 def int8_linear(x: Tensor, weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
-                bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int) -> Tensor:
-    """Quantise the activations per token (rotated first when `rotate`) and run the W8A8 linear."""
+                bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int,
+                addend: Optional[Tensor] = None) -> Tensor:
+    """Quantise the activations per token (rotated first when `rotate`) and run the W8A8 linear;
+    `addend` (shape and dtype of the result) is added inside the epilogue."""
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate)
-    y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order)
+    y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order,
+                         addend=addend)
     return y.reshape(*lead, weight.shape[0])
 
 
 @int8_linear.register_fake
-def _(x, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order):
+def _(x, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, addend=None):
     return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
 
 

@@ -48,6 +48,7 @@ struct GemmArgs {
     const void *bias;
     int bias_dtype;
     int order;
+    const void *addend;  // nullptr or [M,N] of the output dtype, added to the rounded result
     void *out;
     int tiles_m, tiles_n;
 #ifdef I8F_TRACE
@@ -145,6 +146,36 @@ __device__ __forceinline__ void epilogue_quad(const int (&a4)[4], float xs, cons
         *(uint2 *)dst = make_uint2(f32x2_to_f16x2_bits(y[0], y[1]), f32x2_to_f16x2_bits(y[2], y[3]));
     } else {
         *(float4 *)dst = make_float4(y[0], y[1], y[2], y[3]);
+    }
+}
+
+// Eight (or four) outputs of one 16-byte piece plus the addend's, rounded once more to the output
+// dtype: what the reference's `y + side.to(y.dtype)` computes on its rounded tensors.
+template <int OUT>
+__device__ __forceinline__ uint4 add_rounded(uint4 y, uint4 s) {
+    if constexpr (OUT == OUT_F32) {
+        return make_uint4(__float_as_uint(__uint_as_float(y.x) + __uint_as_float(s.x)),
+                          __float_as_uint(__uint_as_float(y.y) + __uint_as_float(s.y)),
+                          __float_as_uint(__uint_as_float(y.z) + __uint_as_float(s.z)),
+                          __float_as_uint(__uint_as_float(y.w) + __uint_as_float(s.w)));
+    } else if constexpr (OUT == OUT_I32) {
+        return y;
+    } else {
+        const uint32_t yv[4] = {y.x, y.y, y.z, y.w}, sv[4] = {s.x, s.y, s.z, s.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (OUT == OUT_BF16) {
+                const float lo = bf16_bits_to_f32(yv[e] & 0xffffu) + bf16_bits_to_f32(sv[e] & 0xffffu);
+                const float hi = bf16_bits_to_f32(yv[e] >> 16) + bf16_bits_to_f32(sv[e] >> 16);
+                o[e] = f32x2_to_bf16x2_bits(lo, hi);
+            } else {
+                const float lo = f16_bits_to_f32(yv[e] & 0xffffu) + f16_bits_to_f32(sv[e] & 0xffffu);
+                const float hi = f16_bits_to_f32(yv[e] >> 16) + f16_bits_to_f32(sv[e] >> 16);
+                o[e] = f32x2_to_f16x2_bits(lo, hi);
+            }
+        }
+        return make_uint4(o[0], o[1], o[2], o[3]);
     }
 }
 
@@ -471,7 +502,12 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #else
                 if (mm < g.M && nn < g.N)
 #endif
-                    stream_store16((char *)g.out + ((int64_t)mm * g.N + nn) * OB, val);
+                {
+                    const int64_t off = ((int64_t)mm * g.N + nn) * OB;
+                    uint4 v = val;
+                    if (g.addend) v = add_rounded<OUT>(v, *(const uint4 *)((const char *)g.addend + off));
+                    stream_store16((char *)g.out + off, v);
+                }
             }
             __builtin_amdgcn_wave_barrier();
 #ifdef I8F_TRACE
@@ -539,6 +575,7 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
             t = a * sc;
             if (g.bias) t = t + b;
         }
+        if (g.addend) t = round_to_dtype<DT>(t) + load_as_f32<DT>(g.addend, idx);
         store_from_f32<DT>(g.out, idx, t);
     }
 }
@@ -574,7 +611,7 @@ int launch(GemmArgs &g, hipStream_t st) {
                       ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.M * g.K < (1ll << 31)) &&
                       ((int64_t)g.N * g.K < (1ll << 31)) &&
                       (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) &&
-                      (!g.bias || (uintptr_t)g.bias % 16 == 0);
+                      (!g.bias || (uintptr_t)g.bias % 16 == 0) && (!g.addend || (uintptr_t)g.addend % 16 == 0);
     (void)ob;
     if (!fast) {
         const int64_t total = (int64_t)g.M * g.N;
@@ -636,9 +673,10 @@ extern "C" int i8f_gemm_i32(const int8_t *a, const int8_t *w, int64_t M, int64_t
     return launch<OUT_I32>(g, (hipStream_t)stream);
 }
 
-extern "C" int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
-                               float w_scale_host, int scale_mode, const void *bias, int bias_dtype, void *out,
-                               int out_dtype, int64_t M, int64_t N, int64_t K, int order, void *stream) {
+extern "C" int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                                   float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                                   const void *addend, void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                   int order, void *stream) {
     using namespace i8f;
     if (int rc = validate(a, w, M, N, K, out)) return rc;
     if (!valid_dtype(out_dtype) || (bias && !valid_dtype(bias_dtype))) return I8F_ERR_INVALID;
@@ -651,11 +689,18 @@ extern "C" int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8
     GemmArgs g{};
     g.x = a, g.w = w, g.M = (int)M, g.N = (int)N, g.K = (int)K, g.out = out;
     g.xs = a_scale, g.ws = w_scale, g.ws_host = w_scale_host, g.row_scale = scale_mode == I8F_SCALE_ROW;
-    g.bias = bias, g.bias_dtype = bias_dtype, g.order = order;
+    g.bias = bias, g.bias_dtype = bias_dtype, g.order = order, g.addend = addend;
     hipStream_t st = (hipStream_t)stream;
     switch (out_dtype) {
     case I8F_BF16: return launch<OUT_BF16>(g, st);
     case I8F_F16: return launch<OUT_F16>(g, st);
     default: return launch<OUT_F32>(g, st);
     }
+}
+
+extern "C" int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                               float w_scale_host, int scale_mode, const void *bias, int bias_dtype, void *out,
+                               int out_dtype, int64_t M, int64_t N, int64_t K, int order, void *stream) {
+    return i8f_linear_w8a8_add(a, a_scale, w, w_scale, w_scale_host, scale_mode, bias, bias_dtype, nullptr, out,
+                               out_dtype, M, N, K, order, stream);
 }

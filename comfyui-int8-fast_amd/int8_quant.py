@@ -79,16 +79,16 @@ def stochastic_round_int8_delta(x: Tensor, scale, seed: int = 0, noise: Tensor |
 # --------------------------------------------------------------------------- forward functions
 @torch.no_grad()
 def int8_forward_dynamic(x: Tensor, weight: Tensor, weight_scale, bias, compute_dtype: torch.dtype,
-                         rotate: bool = False) -> Tensor:
+                         rotate: bool = False, addend: Tensor | None = None) -> Tensor:
     """Dynamic per-token activation quantisation, ONE weight scale (int8_quant.py:68-88)."""
-    return hip_int8_linear(x, weight, weight_scale, bias, compute_dtype, rotate=rotate)
+    return hip_int8_linear(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend)
 
 
 @torch.no_grad()
 def int8_forward_dynamic_per_row(x: Tensor, weight: Tensor, weight_scale: Tensor, bias,
-                                 compute_dtype: torch.dtype, rotate: bool = False) -> Tensor:
+                                 compute_dtype: torch.dtype, rotate: bool = False, addend: Tensor | None = None) -> Tensor:
     """Dynamic per-token activation quantisation, per-row weight scales [N,1] (int8_quant.py:92-119)."""
-    return hip_int8_linear_per_row(x, weight, weight_scale, bias, compute_dtype, rotate=rotate)
+    return hip_int8_linear_per_row(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend)
 
 
 # --------------------------------------------------------------------------- LoRA delta reconstruction
@@ -429,37 +429,44 @@ class Int8TensorwiseOps(manual_cast):
             x_2d = x.reshape(-1, x.shape[-1])
             rotate = bool(getattr(self, "_use_quarot", False))
 
-            if torch.compiler.is_compiling():
-                # under torch.compile the same two branches go through the registered operators
-                ws_t, ws_v = compile_ops.split_scale(w_scale)
-                if x_2d.shape[0] > SMALL_BATCH_ROWS:
-                    y = torch.ops.i8f.int8_linear(x_2d, weight, ws_t, ws_v, bias, compute_dtype, rotate,
-                                                  int8_fused_kernel.DEFAULT_EPILOGUE)
-                else:
-                    y = torch.ops.i8f.linear_w8a16_small_m(x_2d, weight, ws_t, ws_v, bias, rotate)
-            elif x_2d.shape[0] > SMALL_BATCH_ROWS:
-                fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
-                y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate)
-            else:
-                # W8A16: activations keep their dtype (rotated first when the weight is rotated)
-                x_in = _lib.rotate128(x_2d) if rotate else x_2d
-                y = _lib.linear_w8a16_small_m(x_in, weight, w_scale, bias)
-
+            # Dynamic (unmerged) LoRA side branch, float; it is fed the rotated activations when QuaRot
+            # is on, as in the reference (int8_quant.py:741-744,768).  On the W8A8 path its sum with the
+            # main result happens inside the GEMM epilogue (same rounding as the reference's
+            # `y + lora_out.to(y.dtype)`, one pass over [M,N] less).
+            side = None
+            compiling = torch.compiler.is_compiling()
             if self.lora_A is not None and self.lora_B is not None:
-                # dynamic (unmerged) LoRA side branch; fed the rotated activations when QuaRot is on,
-                # as in the reference (int8_quant.py:741-744,768)
                 lA = self.lora_A.to(x.device, non_blocking=True)
                 lB = self.lora_B.to(x.device, non_blocking=True)
                 if not rotate:
                     x_side = x_2d
-                elif torch.compiler.is_compiling():
+                elif compiling:
                     x_side = torch.ops.i8f.rotate128(x_2d)
                 else:
                     x_side = _lib.rotate128(x_2d)
                 side = F.linear(F.linear(x_side.to(lA.dtype), lA), lB)
                 if self.lora_alpha is not None:
                     side = side * self.lora_alpha
-                y = y + side.to(y.dtype)
+
+            if x_2d.shape[0] > SMALL_BATCH_ROWS:
+                addend = None if side is None else side.to(compute_dtype)
+                if compiling:  # under torch.compile the call goes through the registered operator
+                    ws_t, ws_v = compile_ops.split_scale(w_scale)
+                    y = torch.ops.i8f.int8_linear(x_2d, weight, ws_t, ws_v, bias, compute_dtype, rotate,
+                                                  int8_fused_kernel.DEFAULT_EPILOGUE, addend)
+                else:
+                    fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
+                    y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend)
+            else:
+                # W8A16: activations keep their dtype (rotated first when the weight is rotated)
+                if compiling:
+                    ws_t, ws_v = compile_ops.split_scale(w_scale)
+                    y = torch.ops.i8f.linear_w8a16_small_m(x_2d, weight, ws_t, ws_v, bias, rotate)
+                else:
+                    x_in = _lib.rotate128(x_2d) if rotate else x_2d
+                    y = _lib.linear_w8a16_small_m(x_in, weight, w_scale, bias)
+                if side is not None:
+                    y = y + side.to(y.dtype)
 
             if managed:
                 uncast_bias_weight(self, weight, bias, offload_stream)

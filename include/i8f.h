@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define I8F_VERSION 100 /* major*10000 + minor*100 + patch */
+#define I8F_VERSION 101 /* major*10000 + minor*100 + patch */
 
 typedef enum i8f_status {
     I8F_OK = 0,
@@ -130,6 +130,20 @@ int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8_t *w, cons
                     float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
                     void *out, int out_dtype, int64_t M, int64_t N, int64_t K, int order,
                     void *stream);
+
+/*
+ * The same, with a second matrix added to the result inside the epilogue:
+ *   out[m,n] = round( i8f_linear_w8a8(...)[m,n] + addend[m,n] )
+ * Replaces the addition of the dynamic (unmerged) LoRA side branch at the end of
+ * Linear.forward (int8_quant.py:762-774: y = y + lora_out.to(y.dtype)), which in
+ * the reference is a separate elementwise pass over [M,N].  The sum is rounded once
+ * more to out_dtype, as the reference's tensor addition does.
+ *   addend    [M,N] of out_dtype, contiguous; NULL gives i8f_linear_w8a8 exactly
+ */
+int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                        float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                        const void *addend, void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                        int order, void *stream);
 
 /*
  * Small-batch W8A16 path, M <= 16: activations stay in their dtype, the int8

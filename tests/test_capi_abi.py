@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 10
+    assert len(names) == 11
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -59,6 +59,8 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_linear_w8a8(one, one, one, one, 1.0, 5, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID             # bad scale mode
     assert lib.i8f_linear_w8a8(one, one, one, one, 1.0, 0, null, 0, one, L.BF16, 4, 4, 4, 9, null) == INVALID             # bad epilogue order
     assert lib.i8f_linear_w8a8(one, null, one, one, 1.0, 0, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID            # activation scales missing
+    assert lib.i8f_linear_w8a8_add(one, one, one, one, 1.0, 0, null, 0, one, null, L.BF16, 4, 4, 4, 0, null) == INVALID   # no output
+    assert lib.i8f_linear_w8a8_add(one, one, one, one, 1.0, 0, null, 0, one, one, 9, 4, 4, 4, 0, null) == INVALID         # bad output dtype
     assert lib.i8f_linear_w8a16_small_m(one, L.BF16, 17, 8, 8, one, one, 1.0, 0, null, 0, one, 4, null) == UNSUPPORTED    # M > 16
     assert lib.i8f_sr_quant_delta(null, one, 1.0, 0, one, 4, 4, one, null) == INVALID
     assert lib.i8f_lora_merge_sr(one, one, 1.0, 0, null, null, null, 8, 1.0, one, 4, 4, one, null) == INVALID             # neither delta nor factors

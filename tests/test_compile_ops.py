@@ -37,6 +37,8 @@ def test_shape_only_implementations(pkg):
     assert y.shape == (3, 7, 96) and y.dtype == torch.float16
     y = ops.int8_linear(x, w, None, 0.02, None, torch.bfloat16, True, 1)
     assert y.shape == (3, 7, 96) and y.dtype == torch.bfloat16
+    y = ops.int8_linear(x, w, None, 0.02, None, torch.bfloat16, True, 1, torch.empty(3, 7, 96, dtype=torch.bfloat16, device="meta"))
+    assert y.shape == (3, 7, 96)
     q, s = ops.quantize_rowwise(x.reshape(21, 256), True)
     assert q.shape == (21, 256) and q.dtype == torch.int8 and s.shape == (21, 1) and s.dtype == torch.float32
     y = ops.linear_w8a8(q, s, w, ws, 0.0, None, torch.float32, 0)

@@ -197,3 +197,24 @@ def test_forward_under_hip_graph_replays_like_eager(pkg, dev, rows):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(static_y.view(torch.int16), want.view(torch.int16)), f"replay {i}"
+
+
+@pytest.mark.parametrize("rows,quarot", [(40, False), (40, True), (6, True)])
+def test_dynamic_lora_side_branch_is_added_like_the_reference(pkg, dev, rows, quarot):
+    """lora_A / lora_B set: y = y + ((x @ A.T) @ B.T * alpha).to(y.dtype), the sum formed inside the GEMM
+    epilogue on the W8A8 path (int8_quant.py:762-774)."""
+    ops = pkg.Int8TensorwiseOps
+    ops.dynamic_quantize, ops.enable_quarot = True, quarot
+    w = (torch.randn(256, 384, generator=G) * 0.02).bfloat16()
+    b = (torch.randn(256, generator=G) * 0.01).bfloat16()
+    lin = load(ops.Linear(384, 256, bias=True), {"l.weight": w, "l.bias": b}).to(dev)
+    x = torch.randn(rows, 384, generator=G).bfloat16().to(dev)
+    plain = lin(x)
+    A = (torch.randn(16, 384, generator=G) * 0.05).bfloat16().to(dev)
+    B = (torch.randn(256, 16, generator=G) * 0.05).bfloat16().to(dev)
+    lin.lora_A, lin.lora_B, lin.lora_alpha = A, B, 0.5
+    got = lin(x)
+    x_side = pkg._lib.rotate128(x) if quarot else x
+    side = torch.nn.functional.linear(torch.nn.functional.linear(x_side, A), B) * 0.5
+    want = plain + side.to(plain.dtype)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))

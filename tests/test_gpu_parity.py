@@ -183,6 +183,24 @@ def test_linear_w8a8_bit_exact(L, dev, M, N, K, row, bdt, odt, order):
         assert np.array_equal(bits(got2), want)
 
 
+@pytest.mark.parametrize("M,N,K,odt,order", [(300, 520, 1040, torch.bfloat16, 0), (2000, 2056, 200, torch.float16, 1),
+                                             (4100, 2056, 144, torch.bfloat16, 0), (64, 50, 50, torch.bfloat16, 0),
+                                             (256, 256, 512, torch.float32, 0)])
+def test_linear_w8a8_with_addend_rounds_like_a_tensor_addition(L, dev, M, N, K, odt, order):
+    """out = round(linear + addend): the sum of two ROUNDED tensors, rounded once more (int8_quant.py:774)."""
+    x = acts(M, K)
+    wq, ws = L.quant_rowwise((torch.randn(N, K, generator=G) * 0.02).to(dev))
+    bias = (torch.randn(N, generator=G) * 0.01).to(odt).to(dev)
+    addend = (torch.randn(M, N, generator=G) * 0.3).to(odt).to(dev)
+    q, s = L.quant_rowwise(x.to(dev))
+    plain = L.linear_w8a8(q, s, wq, ws, bias, odt, order)          # bit-exact against the oracle by the tests above
+    got = L.linear_w8a8(q, s, wq, ws, bias, odt, order, addend=addend)
+    code = {torch.bfloat16: O.BF16, torch.float16: O.F16, torch.float32: O.F32}[odt]
+    want = O.round_to(O.to_f32(bits(plain), code) + O.to_f32(bits(addend), code), code)
+    assert np.array_equal(bits(got), want)
+    assert torch.equal(got, plain + addend)                          # and what torch's own addition gives
+
+
 def test_linear_accumulator_beyond_2_pow_24_rounds_like_the_oracle(L, dev):
     K = 4096
     a = torch.full((32, K), 127, dtype=torch.int8)
