@@ -607,12 +607,25 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
 template <int OUT>
 int launch(GemmArgs &g, hipStream_t st) {
     const int ob = OutElem<OUT>::BYTES;
-    const bool fast = (g.K % 16 == 0) && (g.N % 8 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
-                      ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.M * g.K < (1ll << 31)) &&
-                      ((int64_t)g.N * g.K < (1ll << 31)) &&
-                      (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) &&
-                      (!g.bias || (uintptr_t)g.bias % 16 == 0) && (!g.addend || (uintptr_t)g.addend % 16 == 0);
-    (void)ob;
+    const bool aligned = (g.K % 16 == 0) && (g.N % 8 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
+                         ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.N * g.K < (1ll << 31)) &&
+                         (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) &&
+                         (!g.bias || (uintptr_t)g.bias % 16 == 0) && (!g.addend || (uintptr_t)g.addend % 16 == 0);
+    // The buffer descriptors address 2^31 bytes: more activations than that go in row blocks.
+    if (aligned && (int64_t)g.M * g.K >= (1ll << 31) && (int64_t)256 * g.K < (1ll << 31)) {
+        const int rows_per = (int)((((1ll << 31) - 1) / g.K) / 256 * 256);
+        for (int64_t m0 = 0; m0 < g.M; m0 += rows_per) {
+            GemmArgs sub = g;
+            sub.M = (int)(g.M - m0 < rows_per ? g.M - m0 : rows_per);
+            sub.x = g.x + m0 * g.K;
+            if (g.xs) sub.xs = g.xs + m0;
+            sub.out = (char *)g.out + m0 * g.N * ob;
+            if (g.addend) sub.addend = (const char *)g.addend + m0 * g.N * ob;
+            if (int rc = launch<OUT>(sub, st)) return rc;
+        }
+        return I8F_OK;
+    }
+    const bool fast = aligned && ((int64_t)g.M * g.K < (1ll << 31));
     if (!fast) {
         const int64_t total = (int64_t)g.M * g.N;
         hipLaunchKernelGGL((gemm_i8_generic_kernel<OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, g);

@@ -67,6 +67,18 @@ def test_quant_rowwise_strided_and_misaligned_views(L, dev):
             assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(s.cpu().numpy(), so)
 
 
+def test_quant_rowwise_more_than_2_pow_31_elements(L, dev):
+    M, K = 131200, 16384                         # 2.15e9 elements: offsets need 64 bits
+    x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+    rows = torch.cat([torch.arange(0, 8), torch.arange(131072 - 8, 131072 + 8), torch.arange(M - 8, M)])
+    for rot in (False, True):
+        q, s = L.quant_rowwise(x, rotate=rot)
+        xa, code = O.from_torch(x[rows].cpu())
+        qo, so = O.quant_rowwise(xa, code, 128 if rot else 0)
+        assert np.array_equal(q[rows].cpu().numpy(), qo) and np.array_equal(s[rows].cpu().numpy(), so)
+        del q, s
+
+
 def test_quant_rowwise_empty(L, dev):
     q, s = L.quant_rowwise(torch.empty(0, 256, dtype=torch.bfloat16, device=dev))
     assert q.shape == (0, 256) and s.shape == (0, 1)
@@ -131,6 +143,22 @@ def test_gemm_i32_random_shapes(L, dev):
         a, w = i8(M, K), i8(N, K)
         acc = L.gemm_i32(a.to(dev), w.to(dev))
         assert np.array_equal(acc.cpu().numpy(), O.gemm_i32(a.numpy(), w.numpy())), (M, N, K)
+
+
+def test_linear_with_more_than_2_gib_of_activations(L, dev):
+    """M * K >= 2^31 bytes: the launcher walks the rows in blocks; rows on both sides of the seam are checked."""
+    M, N, K = 131200, 16, 16384
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=dev)
+    w = torch.randint(-128, 128, (N, K), dtype=torch.int8, device=dev)
+    xs = torch.rand(M, device=dev) * 0.01
+    ws = torch.rand(N, device=dev) * 0.01
+    y = L.linear_w8a8(a, xs, w, ws, None, torch.bfloat16, 0)
+    acc = L.gemm_i32(a, w)
+    rows = torch.cat([torch.arange(0, 40), torch.arange(131072 - 300, 131072 + 128), torch.arange(M - 40, M)])
+    acc_o = O.gemm_i32(a[rows].cpu().numpy(), w.cpu().numpy())
+    assert np.array_equal(acc[rows].cpu().numpy(), acc_o)
+    want = O.epilogue(acc_o, xs[rows].cpu().numpy(), ws.cpu().numpy(), None, O.BF16, O.BF16)
+    assert np.array_equal(bits(y[rows]), want)
 
 
 def test_gemm_i32_saturating_inputs_at_largest_k(L, dev):
