@@ -229,6 +229,21 @@ def test_linear_w8a8_with_addend_rounds_like_a_tensor_addition(L, dev, M, N, K, 
     assert torch.equal(got, plain + addend)                          # and what torch's own addition gives
 
 
+@pytest.mark.parametrize("M,N,K", [(4608, 3072, 3072), (512, 3072, 12288), (4096, 9216, 3072)])
+def test_linear_w8a8_gives_the_same_bits_on_every_launch(L, dev, M, N, K):
+    """300 back-to-back launches (no synchronisation between them) against the first result: a missing
+    wait or barrier in the pipelined loop would show up as a rare differing tile."""
+    q, s = L.quant_rowwise(acts(M, K).to(dev))
+    wq, ws = L.quant_rowwise((torch.randn(N, K, generator=G) * 0.02).to(dev))
+    first = L.linear_w8a8(q, s, wq, ws, None, torch.bfloat16, 0)
+    out = torch.empty_like(first)
+    bad = torch.zeros((), dtype=torch.int64, device=dev)
+    for _ in range(300):
+        L.linear_w8a8(q, s, wq, ws, None, torch.bfloat16, 0, out)
+        bad += (out.view(torch.int16) != first.view(torch.int16)).sum()
+    assert int(bad.item()) == 0
+
+
 def test_linear_accumulator_beyond_2_pow_24_rounds_like_the_oracle(L, dev):
     K = 4096
     a = torch.full((32, K), 127, dtype=torch.int8)
