@@ -584,9 +584,9 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6>;   // 8 waves, 2 x 64 KB stages, one workgroup per CU
 using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
-using CfgT64 = Cfg<64, 64, 128, 2, 2, 2, 8>;     // 4 waves of 32 x 32, 2 x 16 KB stages: outputs of few tiles still fill the chip
-// Few tiles and a long K: about one workgroup per CU, so nothing hides the latency of the
-// global->LDS loads but the loads in flight; four stages instead of two.
+// Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
+// loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
+// flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
 using CfgMidDeep = Cfg<128, 128, 128, 2, 2, 4, 8>;
 using CfgS64Deep = Cfg<128, 64, 128, 2, 2, 4, 8>;
 using CfgT64Deep = Cfg<64, 64, 128, 2, 2, 4, 8>;
@@ -634,8 +634,8 @@ int launch(GemmArgs &g, hipStream_t st) {
     // Tile choice.  With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
     // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
     // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA).  Outputs of fewer than 128
-    // such tiles take 128 x 128 tiles if that gives at least one workgroup per CU, else 64 x 64
-    // (with a long K: deeper pipelines, see the configurations above).
+    // such tiles take 128 x 128 tiles with two stages if that gives at least one workgroup per CU,
+    // else the four-stage configurations above.
     const int64_t CUS = 256;
     auto rounds_cost = [&](int bm, int bn, int per_op_cost) {
         const int64_t tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
@@ -646,17 +646,14 @@ int launch(GemmArgs &g, hipStream_t st) {
     if (I8F_FORCE_CFG == 1) return launch_cfg<CfgBig, OUT>(g, st);
     if (I8F_FORCE_CFG == 2) return launch_cfg<CfgB192, OUT>(g, st);
     if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
-    if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64, OUT>(g, st);
+    if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64Deep, OUT>(g, st);
 #endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
         if (mid_tiles >= CUS) return launch_cfg<CfgMid, OUT>(g, st);
-        if (g.K >= 8192) {  // the largest tile that still gives 192 workgroups
-            if (mid_tiles >= 192) return launch_cfg<CfgMidDeep, OUT>(g, st);
-            if ((int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) >= 192) return launch_cfg<CfgS64Deep, OUT>(g, st);
-            return launch_cfg<CfgT64Deep, OUT>(g, st);
-        }
-        return launch_cfg<CfgT64, OUT>(g, st);
+        if (mid_tiles >= 192) return launch_cfg<CfgMidDeep, OUT>(g, st);
+        if ((int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) >= 192) return launch_cfg<CfgS64Deep, OUT>(g, st);
+        return launch_cfg<CfgT64Deep, OUT>(g, st);
     }
     if (rounds_cost(256, 192, 108) < rounds_cost(256, 256, 100)) return launch_cfg<CfgB192, OUT>(g, st);
     return launch_cfg<CfgBig, OUT>(g, st);

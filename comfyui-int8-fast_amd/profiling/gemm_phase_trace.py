@@ -62,9 +62,9 @@ def main():
         cost = lambda bm, bn, per_op: cd(cd(M, bm) * cd(N, bn), 256) * bm * bn * per_op
         if big >= 128:
             BM, BN = (256, 192) if cost(256, 192, 108) < cost(256, 256, 100) else (256, 256)
-        elif mid >= 256 or (K >= 8192 and mid >= 192):
+        elif mid >= 192:
             BM, BN = 128, 128
-        elif K >= 8192 and cd(M, 128) * cd(N, 64) >= 192:
+        elif cd(M, 128) * cd(N, 64) >= 192:
             BM, BN = 128, 64
         else:
             BM, BN = 64, 64
