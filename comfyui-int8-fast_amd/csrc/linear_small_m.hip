@@ -7,9 +7,13 @@
 // (Linear.forward, int8_quant.py:756-760: the dequantised weight and the bias
 // are cast to x.dtype before F.linear).  The reference writes the whole
 // dequantised weight to memory and reads it back on every call; here the weight
-// is read once as int8.  One wavefront owns one output column n: 64 lanes x 16
-// weights per step, partial sums as fmaf chains in binary32, then a butterfly
-// reduction across the wavefront.
+// is read once as int8.  Two kernels: binary16/bfloat16 activations with
+// 16-byte aligned rows go to the matrix cores (small_m_lds_kernel); anything
+// else to small_m_kernel, where one wavefront owns one output column n (64 lanes
+// x 16 weights per step, partial sums as fmaf chains in binary32, then a
+// butterfly reduction across the wavefront).  The order of the binary32 sums
+// differs between the two; the result is compared with a tolerance of one
+// rounding step of the output type.
 #include "i8f_common.hpp"
 
 namespace i8f {
@@ -120,10 +124,161 @@ __global__ __launch_bounds__(256) void small_m_kernel(const SmallMArgs a) {
     }
 }
 
+// ---- matrix-core variant (binary16 / bfloat16 activations, K % 16 == 0) ---------------------------
+// The weight stream is the only traffic that counts (N*K bytes); the work per weight on the vector
+// ALUs is what decides whether the stream runs at memory speed.  Here it is convert, scale, round
+// (2.5 instructions per weight for bfloat16) and the multiply-adds go to v_mfma_f32_16x16x32: the
+// dequantised weights of 16 output columns are the A operand, the (up to 16) activation rows the B
+// operand, so the arithmetic costs the same for every M <= 16.  A wave owns NB blocks of 16 output
+// columns and every WAVES-th 128-byte step along K.  Lane (r = lane % 16, g = lane / 16) feeds
+// weight row r, bytes 32 g + 8 j .. + 8 of the step, to MFMA j = 0..3 and the activations of row r
+// at the same k; which k a lane group holds does not matter as long as both operands agree.  The
+// WAVES partial sums meet in LDS and are added in wave order, so results do not depend on timing.
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+
+template <int DT>
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t word, int e, float ws) {
+    const float a = (float)(int)(int8_t)(word >> (8 * e)) * ws;
+    const float b = (float)(int)(int8_t)(word >> (8 * e + 8)) * ws;
+    if constexpr (DT == I8F_BF16) return f32x2_to_bf16x2_bits(a, b);
+    else return f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+}
+
+template <int DT>
+__device__ __forceinline__ v4f_t mma8(uint32_t wlo, uint32_t whi, v4u_t xk, float ws, v4f_t acc) {
+    v4u_t a;
+    a.x = dequant_pair<DT>(wlo, 0, ws);
+    a.y = dequant_pair<DT>(wlo, 2, ws);
+    a.z = dequant_pair<DT>(whi, 0, ws);
+    a.w = dequant_pair<DT>(whi, 2, ws);
+    if constexpr (DT == I8F_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, a), __builtin_bit_cast(v8bf_t, xk), acc, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h_t, a), __builtin_bit_cast(v8h_t, xk), acc, 0, 0, 0);
+}
+
+// The weight fetch is fully coalesced: a wave instruction reads 8 rows x 128 contiguous bytes
+// (8 cache lines, adjacent lanes adjacent 16 bytes); the wave parks them in its own LDS tile and
+// reads them back in the MFMA operand layout (8 bytes per lane and MFMA).  The tile is private to
+// the wave, so no barrier is involved.  Fetching straight into the operand layout (16 rows per
+// instruction, 16 or more cache lines) measured 12 % slower, and slower still the more lines an
+// instruction touched.
+template <int DT, int NB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void small_m_lds_kernel(const SmallMArgs a) {
+    constexpr int COLS = NB * 16;
+    constexpr int PITCH = 144;
+    __shared__ float red[WAVES][COLS][16];
+    __shared__ __attribute__((aligned(16))) char tiles[WAVES][COLS * PITCH];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int lr = lane >> 3, lc = lane & 7;   // fetch layout: row within 8, 16-byte column
+    const int64_t n0 = (int64_t)blockIdx.x * COLS;
+    const int K = (int)a.K;
+    const int nsteps = (K + 127) / 128;
+    const bool xrow = r < (int)a.M;
+    const char *xp = (const char *)a.x + (int64_t)(xrow ? r : 0) * a.ldx * 2;
+    char *tile = tiles[wave];
+
+    const int8_t *frow[NB][2];
+    float wsn[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            int64_t n = n0 + b * 16 + h * 8 + lr;
+            n = n < a.N ? n : a.N - 1;
+            frow[b][h] = a.w + n * a.K + lc * 16;
+        }
+        int64_t n = n0 + b * 16 + r;
+        n = n < a.N ? n : a.N - 1;
+        wsn[b] = a.ws ? a.ws[a.row_scale ? n : 0] : a.ws_host;
+    }
+
+    const v4u_t zero = {0u, 0u, 0u, 0u};
+    v4u_t wq[2][NB][2], xq[2][4];
+    auto fetch = [&](int t, int buf) __attribute__((always_inline)) {
+        const int kw = t * 128;
+        const bool wok = kw + lc * 16 + 16 <= K;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) wq[buf][b][h] = wok ? *(const v4u_t *)(frow[b][h] + kw) : zero;
+        const int k = kw + g * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            xq[buf][j] = (xrow && k + 8 * j + 8 <= K) ? *(const v4u_t *)(xp + (int64_t)(k + 8 * j) * 2) : zero;
+    };
+    v4f_t acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[b] = v4f_t{0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) *(v4u_t *)(tile + (b * 16 + h * 8 + lr) * PITCH + lc * 16) = wq[buf][b][h];
+        v2u_t wa[NB][4];
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wa[b][j] = *(const v2u_t *)(tile + (b * 16 + r) * PITCH + g * 32 + 8 * j);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[b] = mma8<DT>(wa[b][j].x, wa[b][j].y, xq[buf][j], wsn[b], acc[b]);
+    };
+
+    int t = wave;
+    if (t < nsteps) fetch(t, 0);
+    for (; t < nsteps; t += 2 * WAVES) {
+        if (t + WAVES < nsteps) fetch(t + WAVES, 1);
+        compute(0);
+        if (t + WAVES < nsteps) {
+            if (t + 2 * WAVES < nsteps) fetch(t + 2 * WAVES, 0);
+            compute(1);
+        }
+    }
+
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave][b * 16 + 4 * g + i][r] = acc[b][i];
+    __syncthreads();
+    for (int o = threadIdx.x; o < COLS * 16; o += WAVES * 64) {
+        const int m = o / COLS, c = o % COLS;
+        const int64_t n = n0 + c;
+        if (m < (int)a.M && n < a.N) {
+            float s = red[0][c][m];
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) s += red[w][c][m];
+            float bv = 0.0f;
+            if (a.bias) {
+                if (a.bias_dtype == I8F_F32) bv = ((const float *)a.bias)[n];
+                else if (a.bias_dtype == I8F_BF16) bv = bf16_bits_to_f32(((const uint16_t *)a.bias)[n]);
+                else bv = f16_bits_to_f32(((const uint16_t *)a.bias)[n]);
+                bv = round_to_dtype<DT>(bv);
+            }
+            store_from_f32<DT>(a.out, (int64_t)m * a.N + n, s + bv);
+        }
+    }
+}
+
+template <int DT, int NB, int WAVES>
+int launch_lds(const SmallMArgs &a, hipStream_t st) {
+    const int64_t cols = NB * 16;
+    hipLaunchKernelGGL((small_m_lds_kernel<DT, NB, WAVES>), dim3((unsigned)((a.N + cols - 1) / cols)), dim3(WAVES * 64), 0, st, a);
+    return check_launch();
+}
+
 template <int DT>
 int launch(const SmallMArgs &a, hipStream_t st) {
     const size_t es = dtype_size(DT);
     const bool vec = a.K % 16 == 0 && (uintptr_t)a.w % 16 == 0 && (uintptr_t)a.x % 16 == 0 && (a.ldx * es) % 16 == 0;
+    if constexpr (DT != I8F_F32) {
+        if (vec && a.K < (1ll << 30)) return launch_lds<DT, 2, 8>(a, st);
+    }
     dim3 grid((unsigned)((a.N + 3) / 4));
     if (vec) hipLaunchKernelGGL((small_m_kernel<DT, true>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((small_m_kernel<DT, false>), grid, dim3(256), 0, st, a);

@@ -33,6 +33,10 @@ def bits(t):
     return O.from_torch(t.cpu())[0]
 
 
+def _raw16(t):
+    return t.contiguous().view(torch.int16)
+
+
 # ------------------------------------------------------------------ quantiser (a1, a3, a4)
 QUANT_CASES = [
     # M, K, dtype, rotate
@@ -366,6 +370,8 @@ def test_config4_merge_full_size_then_skinny_gemm(L, dev):
 @pytest.mark.parametrize("M,N,K,dt,rel,absf", [
     (1, 18432, 3072, torch.bfloat16, 2.0**-7, 2.0**-8), (16, 260, 1024, torch.bfloat16, 2.0**-7, 2.0**-8),
     (3, 100, 77, torch.float16, 2.0**-10, 2.0**-11), (2, 64, 256, torch.float32, 1e-5, 1e-6), (7, 33, 4096, torch.float16, 2.0**-10, 2.0**-11),
+    (5, 48, 272, torch.bfloat16, 2.0**-7, 2.0**-8), (16, 31, 144, torch.float16, 2.0**-10, 2.0**-11), (1, 1, 16, torch.bfloat16, 2.0**-7, 2.0**-8),
+    (13, 513, 2064, torch.bfloat16, 2.0**-7, 2.0**-8), (2, 96, 12288, torch.float16, 2.0**-10, 2.0**-11),
 ])
 def test_small_m_w8a16_within_tolerance(L, dev, M, N, K, dt, rel, absf):
     x = torch.randn(M, K, generator=G).to(dt)
@@ -379,6 +385,25 @@ def test_small_m_w8a16_within_tolerance(L, dev, M, N, K, dt, rel, absf):
     got_t = L.linear_w8a16_small_m(x.to(dev), wq.to(dev), 0.004, None).float().cpu().numpy()
     ref_t = O.to_f32(O.linear_w8a16(xa, code, wq.numpy(), np.float32(0.004)), code)
     assert (np.abs(got_t - ref_t) <= rel * np.abs(ref_t) + absf * np.abs(ref_t).max()).all()
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_small_m_rows_are_independent_and_strided_rows_work(L, dev, dt):
+    """A token's result must not depend on how many other tokens share the call (the matrix-core
+    kernel computes 16 token columns at once), nor on the row stride of x."""
+    N, K = 200, 1040
+    wide = torch.randn(16, K + 24, generator=G).to(dt).to(dev)
+    x = wide[:, :K]                               # row stride K + 24 elements
+    wq = i8(N, K).to(dev)
+    ws = (torch.rand(N, generator=G) * 0.01 + 0.001).to(dev)
+    bias = (torch.randn(N, generator=G) * 0.1).to(dt).to(dev)
+    y16 = L.linear_w8a16_small_m(x, wq, ws, bias)
+    assert torch.equal(_raw16(y16), _raw16(L.linear_w8a16_small_m(x.contiguous(), wq, ws, bias)))
+    for m in (0, 3, 15):
+        y1 = L.linear_w8a16_small_m(x[m:m + 1].contiguous(), wq, ws, bias)
+        assert torch.equal(_raw16(y1[0]), _raw16(y16[m]))
+    y5 = L.linear_w8a16_small_m(x[4:9], wq, ws, bias)
+    assert torch.equal(_raw16(y5), _raw16(y16[4:9]))
 
 
 # ------------------------------------------------------------------ stochastic merge (a9, a10, a11)
