@@ -198,6 +198,28 @@ __device__ __forceinline__ void expand16(const uint4 &a, const uint4 &b, float (
     }
 }
 
+// v[j] += sign * (v[j] of the partner lane) for 16 registers: v_fmac_f32 with a DPP source.  The
+// compiler does not fold a DPP move into a fused multiply-add, hence the assembly.  A DPP read of a
+// register needs two wait states after a vector write of it, which the compiler cannot see inside
+// the block: the s_nop covers the instruction in front of it, and inside it every instruction
+// touches another register.
+#define I8F_DPP_FMAC(n, ctrl) "v_fmac_f32_dpp %" #n ", %" #n ", %16 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"
+#define I8F_DPP_FMAC16(ctrl)                                                                                       \
+    asm volatile("s_nop 1\n\t" I8F_DPP_FMAC(0, ctrl) I8F_DPP_FMAC(1, ctrl) I8F_DPP_FMAC(2, ctrl) I8F_DPP_FMAC(3, ctrl)  \
+                 I8F_DPP_FMAC(4, ctrl) I8F_DPP_FMAC(5, ctrl) I8F_DPP_FMAC(6, ctrl) I8F_DPP_FMAC(7, ctrl)             \
+                 I8F_DPP_FMAC(8, ctrl) I8F_DPP_FMAC(9, ctrl) I8F_DPP_FMAC(10, ctrl) I8F_DPP_FMAC(11, ctrl)           \
+                 I8F_DPP_FMAC(12, ctrl) I8F_DPP_FMAC(13, ctrl) I8F_DPP_FMAC(14, ctrl) I8F_DPP_FMAC(15, ctrl)         \
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]),  \
+                   "+v"(v[8]), "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]),         \
+                   "+v"(v[15])                                                                                     \
+                 : "v"(sign))
+template <int STAGE>
+__device__ __forceinline__ void dpp_fmac16(float (&v)[16], float sign) {
+    if constexpr (STAGE == 0) I8F_DPP_FMAC16("quad_perm:[1,0,3,2]");
+    else if constexpr (STAGE == 1) I8F_DPP_FMAC16("quad_perm:[2,3,0,1]");
+    else I8F_DPP_FMAC16("row_half_mirror");
+}
+
 template <int DT>
 __device__ __forceinline__ void rotate_run16(float (&v)[16], float s0, float s1, float s2) {
 #pragma unroll
@@ -211,29 +233,16 @@ __device__ __forceinline__ void rotate_run16(float (&v)[16], float s0, float s1,
             }
         }
     }
-    // lower lane: own + other; upper lane: other - own  ==  other + sign * own (the product is exact)
-    // (all products first, then the DPP adds: a DPP instruction needs two wait states after a VALU
-    // write of any of its sources, which back-to-back pairs would pay as s_nop)
-    float w[16];
-#pragma unroll
-    for (int j = 0; j < 16; ++j) w[j] = v[j] * s0;
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < 16; ++j) v[j] = dpp_f32<0xB1>(v[j]) + w[j];   // quad_perm [1,0,3,2]
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < 16; ++j) w[j] = v[j] * s1;
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < 16; ++j) v[j] = dpp_f32<0x4E>(v[j]) + w[j];   // quad_perm [2,3,0,1]
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < 16; ++j) w[j] = v[j] * s2;
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < 16; ++j) v[j] = dpp_f32<0x141>(v[j]) + w[j];  // row_half_mirror
-    __builtin_amdgcn_sched_barrier(0);
-    const float h = hadamard_entry<DT>();
+    // Across lanes a stage is own + sign * other: the lower lane gets own + other, the upper lane
+    // own - other, which is the negative of the butterfly's other - own.  Negation is exact and
+    // commutes with every rounding, both lanes of a later pair carry the same accumulated sign, and
+    // the product of the three signs is folded into the final multiplication (hs = +-h).  One
+    // fused multiply-add with a DPP operand per element and stage; the product by +-1 is exact, so
+    // the sum is rounded once, as an addition would be.
+    dpp_fmac16<0>(v, s0);   // quad_perm [1,0,3,2]
+    dpp_fmac16<1>(v, s1);   // quad_perm [2,3,0,1]
+    dpp_fmac16<2>(v, s2);   // row_half_mirror
+    const float h = hadamard_entry<DT>() * (s0 * s1 * s2);
 #pragma unroll
     for (int j = 0; j < 16; j += 2) {
         const float a = v[j] * h, b = v[j + 1] * h;
