@@ -65,12 +65,15 @@ struct Cfg {
     static constexpr int MI = WTM / 32, NI = WTN / 32;  // 32x32 MFMA blocks per wave
     static constexpr int CPR = BK / 16;                 // 16-byte chunks per LDS row
     static constexpr int X_BYTES = BM * BK, W_BYTES = BN * BK;
-    static constexpr int STAGE_BYTES = X_BYTES + W_BYTES;
-    static constexpr int X_LOADS = X_BYTES / 1024 / NW, W_LOADS = W_BYTES / 1024 / NW;
+    // every wave issues the same number of 1 KB loads per tile; a tile that does not split evenly
+    // over the waves is rounded up, and the surplus loads are out of range (they move nothing)
+    static constexpr int X_LOADS = (X_BYTES / 1024 + NW - 1) / NW, W_LOADS = (W_BYTES / 1024 + NW - 1) / NW;
+    static constexpr int X_ALLOC = X_LOADS * NW * 1024, W_ALLOC = W_LOADS * NW * 1024;
+    static constexpr int STAGE_BYTES = X_ALLOC + W_ALLOC;
     static constexpr int LOADS = X_LOADS + W_LOADS;
     static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
-    static_assert(X_BYTES % (1024 * NW) == 0 && W_BYTES % (1024 * NW) == 0, "tile must split into whole wave loads");
+    static_assert(X_BYTES % 1024 == 0 && W_BYTES % 1024 == 0, "tile must split into whole wave loads");
     static_assert(BK == 64 || BK == 128, "BK");
 };
 
@@ -265,7 +268,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         const int row = gidx / CPR, cl = gidx % CPR;
         xck[t] = (cl ^ swz<CPR>(row)) * 16;
         const int64_t grow = (int64_t)m0 + row;
-        xoff[t] = grow < g.M ? (uint32_t)(grow * K + xck[t]) : OOB;
+        xoff[t] = (row < BM && grow < g.M) ? (uint32_t)(grow * K + xck[t]) : OOB;
     }
 #pragma unroll
     for (int t = 0; t < C::W_LOADS; ++t) {
@@ -273,7 +276,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         const int row = gidx / CPR, cl = gidx % CPR;
         wck[t] = (cl ^ swz<CPR>(row)) * 16;
         const int64_t grow = (int64_t)n0 + row;
-        woff[t] = grow < g.N ? (uint32_t)(grow * K + wck[t]) : OOB;
+        woff[t] = (row < BN && grow < g.N) ? (uint32_t)(grow * K + wck[t]) : OOB;
     }
 
     const int KT = (K + BK - 1) / BK;
@@ -294,7 +297,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
             vo = (kb + (is_x ? xck[t] : wck[t]) < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
             so = 0;
         }
-        dma16(is_x ? rx : rw, st + (is_x ? 0 : C::X_BYTES) + t * NW * 1024, vo, so);
+        dma16(is_x ? rx : rw, st + (is_x ? 0 : C::X_ALLOC) + t * NW * 1024, vo, so);
     };
     auto issue = [&](int kt, bool live) {
 #pragma unroll
@@ -307,7 +310,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) koff[ks] = ((ks * 2 + lhalf) ^ sw) * 16;
     const int xrow_off = (wm * C::WTM + l32) * BK;
-    const int wrow_off = C::X_BYTES + (wn * C::WTN + l32) * BK;
+    const int wrow_off = C::X_ALLOC + (wn * C::WTN + l32) * BK;
 
     v16i acc[MI][NI];
 #pragma unroll
@@ -584,6 +587,7 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6>;   // 8 waves, 2 x 64 KB stages, one workgroup per CU
 using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
+using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8>;  // 12 waves of 96 x 64, 2 x 72 KB stages
 // Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
 // loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
 // flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
@@ -633,7 +637,9 @@ int launch(GemmArgs &g, hipStream_t st) {
     }
     // Tile choice.  With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
     // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
-    // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA).  Outputs of fewer than 128
+    // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA) and the 288 x 256 tile of
+    // twelve waves about 12 % (it pays where it saves a round: 4608 x 12288 takes 768 of them, three
+    // rounds, instead of 864 of 256 x 256, four).  Outputs of fewer than 128
     // such tiles take 128 x 128 tiles with two stages if that gives at least one workgroup per CU,
     // else the four-stage configurations above.
     const int64_t CUS = 256;
@@ -647,6 +653,7 @@ int launch(GemmArgs &g, hipStream_t st) {
     if (I8F_FORCE_CFG == 2) return launch_cfg<CfgB192, OUT>(g, st);
     if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
     if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64Deep, OUT>(g, st);
+    if (I8F_FORCE_CFG == 5) return launch_cfg<CfgTall, OUT>(g, st);
 #endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
@@ -655,7 +662,9 @@ int launch(GemmArgs &g, hipStream_t st) {
         if ((int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) >= 192) return launch_cfg<CfgS64Deep, OUT>(g, st);
         return launch_cfg<CfgT64Deep, OUT>(g, st);
     }
-    if (rounds_cost(256, 192, 108) < rounds_cost(256, 256, 100)) return launch_cfg<CfgB192, OUT>(g, st);
+    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108), c_tall = rounds_cost(288, 256, 112);
+    if (c_tall < c_big && c_tall < c_192) return launch_cfg<CfgTall, OUT>(g, st);
+    if (c_192 < c_big) return launch_cfg<CfgB192, OUT>(g, st);
     return launch_cfg<CfgBig, OUT>(g, st);
 }
 

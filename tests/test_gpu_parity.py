@@ -124,6 +124,8 @@ GEMM_CASES = [(256, 256, 64), (256, 256, 3072), (300, 520, 1040), (128, 128, 128
               (1, 8, 16), (17, 3072, 3072), (1024, 768, 12288), (513, 1032, 80), (40, 24, 16), (31, 33, 35), (512, 512, 0),
               # one ragged case per tile configuration of the fast kernel: 128x128, 256x192, 256x256 (K tails included)
               (2048, 2048, 256), (2000, 2056, 200), (4100, 2056, 144), (3000, 4104, 80), (3000, 4104, 256),
+              # 288x256 tiles of twelve waves (chosen where they save a round over 256 CUs), ragged in M, N and K
+              (4500, 4088, 144), (4330, 4096, 256),
               # long K, few tiles: the four-stage configurations (128x128, 128x64, 64x64)
               (1000, 3080, 8200), (500, 3072, 8192), (200, 520, 8320)]
 
@@ -193,6 +195,9 @@ LIN_CASES = [
     (1030, 264, 272, False, torch.float32, torch.float16, 1), (40, 24, 16, False, None, torch.float16, 1),
     (2000, 2056, 200, True, torch.bfloat16, torch.bfloat16, 0), (4100, 2056, 144, True, torch.float16, torch.float16, 1),
     (3000, 4104, 80, False, torch.bfloat16, torch.bfloat16, 0), (3000, 4104, 256, True, None, torch.float32, 1),
+    # 288x256 tiles
+    (4500, 4088, 80, True, torch.bfloat16, torch.bfloat16, 0), (4400, 4088, 128, False, torch.float16, torch.float32, 1),
+    (4608, 4096, 144, True, torch.float32, torch.float16, 1),
 ]
 
 
