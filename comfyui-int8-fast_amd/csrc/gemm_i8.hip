@@ -426,8 +426,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // scale, bias, round.  The per-column operands (4 consecutive n per lane and MFMA block) are
     // fetched from LDS into registers once, in front of the strips: fetched inside, every group of
     // four values would wait for an LDS round trip.
-    auto convert_strip = [&](int i, char *dst_rows, const float4 (&wr)[NI][4], const float4 (&br)[NI][4], auto ORDER,
-                             auto ROW, auto BIAS) {
+    auto convert_strip = [&](int i, char *dst_rows, const auto &wr, const auto &br, auto ORDER, auto ROW, auto BIAS) {
         const float xs = s_xs[wm * C::WTM + i * 32 + l32];
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
@@ -449,19 +448,26 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // The whole epilogue is instantiated once per variant and the variant is chosen ONCE, so that
     // the instructions a wave executes are contiguous in memory (the epilogue runs once per wave,
     // straight from a cold instruction cache).
+    // With more than 8 waves a wave has fewer registers than the accumulators plus the operands of
+    // all its columns need: the column operands are then fetched per 32-column block, and a block is
+    // converted for all staged strips before the next one is fetched.
+    constexpr bool PRELOAD_ALL = C::NT <= 512;
     auto run_epilogue = [&](auto ORDER, auto ROW, auto BIAS) {
-        float4 wr[NI][4], br[NI][4];
-        if constexpr (OUT != OUT_I32) {
+        constexpr int NPRE = PRELOAD_ALL ? NI : 1;
+        float4 wr[NPRE][4], br[NPRE][4];
+        auto fetch_cols = [&](int j, float4 (&wj)[4], float4 (&bj)[4]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
+            for (int qd = 0; qd < 4; ++qd) {
+                const int nl = wn * C::WTN + j * 32 + qd * 8 + lhalf * 4;
+                if constexpr (decltype(ROW)::value) wj[qd] = *(const float4 *)&s_ws[nl];
+                else wj[qd] = make_float4(s_ws[0], s_ws[0], s_ws[0], s_ws[0]);
+                if constexpr (decltype(BIAS)::value) bj[qd] = *(const float4 *)&s_bias[nl];
+                else bj[qd] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        };
+        if constexpr (OUT != OUT_I32 && PRELOAD_ALL) {
 #pragma unroll
-                for (int qd = 0; qd < 4; ++qd) {
-                    const int nl = wn * C::WTN + j * 32 + qd * 8 + lhalf * 4;
-                    if constexpr (decltype(ROW)::value) wr[j][qd] = *(const float4 *)&s_ws[nl];
-                    else wr[j][qd] = make_float4(s_ws[0], s_ws[0], s_ws[0], s_ws[0]);
-                    if constexpr (decltype(BIAS)::value) br[j][qd] = *(const float4 *)&s_bias[nl];
-                    else br[j][qd] = make_float4(0.f, 0.f, 0.f, 0.f);
-                }
+            for (int j = 0; j < NI; ++j) fetch_cols(j, wr[j], br[j]);
         }
 #ifdef I8F_TRACE
         if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 4] = wall_clock64();
@@ -481,8 +487,26 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
                             v4i o = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
                             *(v4i *)(rows + l32 * PITCH + nl * 4) = o;
                         }
-                } else {
+                } else if constexpr (PRELOAD_ALL) {
                     convert_strip(i, rows, wr, br, ORDER, ROW, BIAS);
+                }
+            }
+            if constexpr (OUT != OUT_I32 && !PRELOAD_ALL) {
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    fetch_cols(j, wr[0], br[0]);
+#pragma unroll
+                    for (int is = 0; is < EPI_STRIPS; ++is) {
+                        const int i = i0 + is;
+                        const float xs = s_xs[wm * C::WTM + i * 32 + l32];
+#pragma unroll
+                        for (int qd = 0; qd < 4; ++qd) {
+                            const int nl = j * 32 + qd * 8 + lhalf * 4;
+                            const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
+                            epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value>(
+                                a4, xs, wr[0][qd], br[0][qd], ebuf + (is * 32 + l32) * PITCH + nl * OB);
+                        }
+                    }
                 }
             }
             __builtin_amdgcn_wave_barrier();
