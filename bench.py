@@ -82,7 +82,7 @@ def make_config(i: int, rows: int | None = None) -> dict:
 # FETCH_SIZE 139354 KiB / WRITE_SIZE 110592 KiB for 4608x12288x3072 and 153783 / 27648 KiB for
 # 4608x3072x12288; a 256 MiB device copy reads 131084 / 262144 KiB on the same counters, so fetches
 # scale by 2.00 and writes by 1.00.  The mean of the two launches:
-GEMM_TRAFFIC_BYTES = int(((139354 * 2.0 + 110592) + (153783 * 2.0 + 27648)) / 2 * 1024)
+GEMM_TRAFFIC_BYTES = int(((120105 * 2.0 + 110679) + (153807 * 2.0 + 27648)) / 2 * 1024)
 
 
 # --------------------------------------------------------------------------- timing helpers

@@ -662,7 +662,7 @@ int launch(GemmArgs &g, hipStream_t st) {
     // Tile choice.  With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
     // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
     // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA) and the 288 x 256 tile of
-    // twelve waves about 12 % (it pays where it saves a round: 4608 x 12288 takes 768 of them, three
+    // twelve waves about 2 % (it pays where it saves a round: 4608 x 12288 takes 768 of them, three
     // rounds, instead of 864 of 256 x 256, four).  Outputs of fewer than 128
     // such tiles take 128 x 128 tiles with two stages if that gives at least one workgroup per CU,
     // else the four-stage configurations above.
@@ -686,7 +686,7 @@ int launch(GemmArgs &g, hipStream_t st) {
         if ((int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) >= 192) return launch_cfg<CfgS64Deep, OUT>(g, st);
         return launch_cfg<CfgT64Deep, OUT>(g, st);
     }
-    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108), c_tall = rounds_cost(288, 256, 112);
+    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108), c_tall = rounds_cost(288, 256, 102);
     if (c_tall < c_big && c_tall < c_192) return launch_cfg<CfgTall, OUT>(g, st);
     if (c_192 < c_big) return launch_cfg<CfgB192, OUT>(g, st);
     return launch_cfg<CfgBig, OUT>(g, st);

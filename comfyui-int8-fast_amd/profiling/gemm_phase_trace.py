@@ -61,7 +61,7 @@ def main():
         big, mid = cd(M, 256) * cd(N, 256), cd(M, 128) * cd(N, 128)
         cost = lambda bm, bn, per_op: cd(cd(M, bm) * cd(N, bn), 256) * bm * bn * per_op
         if big >= 128:
-            c_big, c_192, c_tall = cost(256, 256, 100), cost(256, 192, 108), cost(288, 256, 112)
+            c_big, c_192, c_tall = cost(256, 256, 100), cost(256, 192, 108), cost(288, 256, 102)
             BM, BN = (288, 256) if c_tall < min(c_big, c_192) else ((256, 192) if c_192 < c_big else (256, 256))
         elif mid >= 192:
             BM, BN = 128, 128
