@@ -25,6 +25,7 @@
 #include <type_traits>
 
 #include "i8f_common.hpp"
+#include <algorithm>
 #ifdef I8F_TRACE
 #include <cstdlib>
 #endif
@@ -612,6 +613,7 @@ using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6>;   // 8 waves, 2 x 64 KB stages, o
 using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
 using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8>;  // 12 waves of 96 x 64, 2 x 72 KB stages
+using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8>;  // 12 waves of 64 x 96, the same transposed
 // Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
 // loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
 // flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
@@ -662,8 +664,9 @@ int launch(GemmArgs &g, hipStream_t st) {
     // Tile choice.  With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
     // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
     // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA) and the 288 x 256 tile of
-    // twelve waves about 2 % (it pays where it saves a round: 4608 x 12288 takes 768 of them, three
-    // rounds, instead of 864 of 256 x 256, four).  Outputs of fewer than 128
+    // twelve waves, or 256 x 288, about 2 % (they pay where they save a round: 4608 x 12288 takes 768
+    // tiles of 288 x 256, three rounds, instead of 864 of 256 x 256, four; 4096 x 9216 takes 512 of
+    // 256 x 288, two rounds).  Outputs of fewer than 128
     // such tiles take 128 x 128 tiles with two stages if that gives at least one workgroup per CU,
     // else the four-stage configurations above.
     const int64_t CUS = 256;
@@ -678,6 +681,7 @@ int launch(GemmArgs &g, hipStream_t st) {
     if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
     if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64Deep, OUT>(g, st);
     if (I8F_FORCE_CFG == 5) return launch_cfg<CfgTall, OUT>(g, st);
+    if (I8F_FORCE_CFG == 6) return launch_cfg<CfgWide, OUT>(g, st);
 #endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
@@ -686,10 +690,13 @@ int launch(GemmArgs &g, hipStream_t st) {
         if ((int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) >= 192) return launch_cfg<CfgS64Deep, OUT>(g, st);
         return launch_cfg<CfgT64Deep, OUT>(g, st);
     }
-    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108), c_tall = rounds_cost(288, 256, 102);
-    if (c_tall < c_big && c_tall < c_192) return launch_cfg<CfgTall, OUT>(g, st);
-    if (c_192 < c_big) return launch_cfg<CfgB192, OUT>(g, st);
-    return launch_cfg<CfgBig, OUT>(g, st);
+    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108);
+    const int64_t c_tall = rounds_cost(288, 256, 102), c_wide = rounds_cost(256, 288, 102);
+    const int64_t c_min = std::min(std::min(c_big, c_192), std::min(c_tall, c_wide));
+    if (c_big == c_min) return launch_cfg<CfgBig, OUT>(g, st);
+    if (c_tall == c_min) return launch_cfg<CfgTall, OUT>(g, st);
+    if (c_wide == c_min) return launch_cfg<CfgWide, OUT>(g, st);
+    return launch_cfg<CfgB192, OUT>(g, st);
 }
 
 int validate(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K, const void *out) {

@@ -61,8 +61,9 @@ def main():
         big, mid = cd(M, 256) * cd(N, 256), cd(M, 128) * cd(N, 128)
         cost = lambda bm, bn, per_op: cd(cd(M, bm) * cd(N, bn), 256) * bm * bn * per_op
         if big >= 128:
-            c_big, c_192, c_tall = cost(256, 256, 100), cost(256, 192, 108), cost(288, 256, 102)
-            BM, BN = (288, 256) if c_tall < min(c_big, c_192) else ((256, 192) if c_192 < c_big else (256, 256))
+            cands = [(cost(256, 256, 100), (256, 256)), (cost(288, 256, 102), (288, 256)),
+                     (cost(256, 288, 102), (256, 288)), (cost(256, 192, 108), (256, 192))]
+            BM, BN = min(cands, key=lambda c: c[0])[1]      # ties go to the first, as in the library
         elif mid >= 192:
             BM, BN = 128, 128
         elif cd(M, 128) * cd(N, 64) >= 192:

@@ -126,6 +126,8 @@ GEMM_CASES = [(256, 256, 64), (256, 256, 3072), (300, 520, 1040), (128, 128, 128
               (2048, 2048, 256), (2000, 2056, 200), (4100, 2056, 144), (3000, 4104, 80), (3000, 4104, 256),
               # 288x256 tiles of twelve waves (chosen where they save a round over 256 CUs), ragged in M, N and K
               (4500, 4088, 144), (4330, 4096, 256),
+              # 256x288 tiles of twelve waves
+              (4090, 4600, 144), (4096, 4608, 128),
               # long K, few tiles: the four-stage configurations (128x128, 128x64, 64x64)
               (1000, 3080, 8200), (500, 3072, 8192), (200, 520, 8320)]
 
@@ -198,6 +200,8 @@ LIN_CASES = [
     # 288x256 tiles
     (4500, 4088, 80, True, torch.bfloat16, torch.bfloat16, 0), (4400, 4088, 128, False, torch.float16, torch.float32, 1),
     (4608, 4096, 144, True, torch.float32, torch.float16, 1),
+    # 256x288 tiles
+    (4090, 4600, 80, True, torch.bfloat16, torch.bfloat16, 0), (4096, 4608, 128, False, torch.float32, torch.float32, 1),
 ]
 
 
