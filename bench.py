@@ -217,27 +217,37 @@ def extras(L, dev, quick=False):
 
     # config 3: the linears of one double-stream DiT block (attention stays bf16 and is not counted)
     c3 = make_config(3)
-    lin = {}
-    for name, (n_out, k_in) in c3["linears"].items():
-        wq_, ws_ = L.quant_rowwise(torch.randn(n_out, k_in, device=dev) * 0.02)
-        lin[name] = (wq_, ws_, (torch.randn(n_out, device=dev) * 0.01).bfloat16())
+    lin = {m: {} for m in (4096, 512)}   # the image and the text stream have their own weights
+    for m in lin:
+        for name, (n_out, k_in) in c3["linears"].items():
+            wq_, ws_ = L.quant_rowwise(torch.randn(n_out, k_in, device=dev) * 0.02)
+            lin[m][name] = (wq_, ws_, (torch.randn(n_out, device=dev) * 0.01).bfloat16())
     acts = {m: {k: torch.randn(m, k, device=dev).bfloat16() for k in (3072, 12288)} for m in (4096, 512)}
     vec = torch.randn(1, 3072, device=dev).bfloat16()
     bufs = {(m, n): torch.empty(m, n, dtype=torch.bfloat16, device=dev) for m in (4096, 512) for n in (9216, 3072, 12288)}
 
     def block(_i):
         for m in (4096, 512):   # image stream, text stream
-            L.linear_w8a16_small_m(vec, lin["adaln"][0], lin["adaln"][1], lin["adaln"][2])
+            L.linear_w8a16_small_m(vec, *lin[m]["adaln"])
             for name, k in (("qkv", 3072), ("proj", 3072), ("up", 3072), ("down", 12288)):
-                wq_, ws_, b_ = lin[name]
+                wq_, ws_, b_ = lin[m][name]
                 q_, s_ = L.quant_rowwise(acts[m][k])
                 L.linear_w8a8(q_, s_, wq_, ws_, b_, torch.bfloat16, L.EPI_TORCH, bufs[(m, wq_.shape[0])])
+
+    # the adaLN projection alone (M = 1, W8A16): a stream over the int8 weight, two weight sets in turn
+    ada = [lin[m]["adaln"] for m in (4096, 512)]
+    t = time_kernel(lambda i: L.linear_w8a16_small_m(vec, *ada[i]), max(10, iters // 4), sets=2, burst=8)
+    abytes = ada[0][0].numel()
+    out["adaln_w8a16_m1_18432x3072"] = {"median_us": round(t["median_us"], 2), "gbs": round(abytes / t["median_us"] / 1e3, 1),
+                                        "frac_of_hbm_peak": round(abytes / t["median_us"] / 1e3 / PEAK_HBM_GBS, 4), "bytes": abytes,
+                                        "note": "two 56.6 MB weights in turn: partly served by the 256 MB memory-side cache"}
 
     t = time_kernel(block, max(10, iters // 4))
     ops = sum(2 * m * n * k for m in (4096, 512) for (n, k) in [c3["linears"][x] for x in ("qkv", "proj", "up", "down")])
     out["dit_block_linears"] = {"ms": round(t["median_us"] / 1e3, 4), "gemm_gop": round(ops / 1e9, 1),
                                 "tops": round(ops / t["median_us"] / 1e6, 1),
-                                "note": "8 W8A8 linears (quantise + GEMM) and 2 adaLN W8A16 linears at M=1; attention not included"}
+                                "note": "8 W8A8 linears (quantise + GEMM) and 2 adaLN W8A16 linears at M=1, separate weights for "
+                                        "the image and the text stream (340 MB in all); attention not included"}
     return out
 
 

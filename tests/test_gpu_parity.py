@@ -226,7 +226,9 @@ def test_linear_w8a8_bit_exact(L, dev, M, N, K, row, bdt, odt, order):
 
 @pytest.mark.parametrize("M,N,K,odt,order", [(300, 520, 1040, torch.bfloat16, 0), (2000, 2056, 200, torch.float16, 1),
                                              (4100, 2056, 144, torch.bfloat16, 0), (64, 50, 50, torch.bfloat16, 0),
-                                             (256, 256, 512, torch.float32, 0)])
+                                             (256, 256, 512, torch.float32, 0),
+                                             (4500, 4088, 144, torch.bfloat16, 0),    # 288x256 tiles
+                                             (4090, 4600, 80, torch.float16, 1)])     # 256x288 tiles
 def test_linear_w8a8_with_addend_rounds_like_a_tensor_addition(L, dev, M, N, K, odt, order):
     """out = round(linear + addend): the sum of two ROUNDED tensors, rounded once more (int8_quant.py:774)."""
     x = acts(M, K)
