@@ -218,3 +218,38 @@ def test_dynamic_lora_side_branch_is_added_like_the_reference(pkg, dev, rows, qu
     side = torch.nn.functional.linear(torch.nn.functional.linear(x_side, A), B) * 0.5
     want = plain + side.to(plain.dtype)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_dynamic_lora_hook_drives_the_side_branch(pkg, dev):
+    """transformer_options["dynamic_loras"] -> hook -> lora_A / lora_B of the layer -> forward with the side branch
+    (int8_quant.py:415-507 feeding :762-774)."""
+    dl = pkg.dynamic_lora
+
+    class Tiny(torch.nn.Module):
+        def __init__(self, lin):
+            super().__init__()
+            self.proj = lin
+
+        def forward(self, x, transformer_options=None):
+            return self.proj(x)
+
+    wq = torch.randint(-128, 128, (64, 128), dtype=torch.int8, generator=G)
+    lin = load(pkg.Int8TensorwiseOps.Linear(128, 64, bias=False), {"l.weight": wq, "l.weight_scale": torch.rand(64, 1) * 0.01})
+    model = Tiny(lin).to(dev)
+    x = torch.randn(40, 128, generator=G).bfloat16().to(dev)
+    base = model(x)
+
+    class Adapter:
+        def __init__(self, up, down, alpha):
+            self.weights = (up, down, alpha, None, None, None)
+
+    up, down = (torch.randn(64, 4, generator=G) * 0.1).bfloat16(), (torch.randn(4, 128, generator=G) * 0.1).bfloat16()
+    options = {}
+    dl.append_entry(options, "a", 0.5, {"diffusion_model.proj.weight": Adapter(up, down, 8.0)})
+    dl.DynamicLoRAHook.register(model)
+    got = model(x, transformer_options=options["transformer_options"])
+    a_dev = (down * (8.0 / 4 * 0.5)).to(dev)
+    side = torch.nn.functional.linear(torch.nn.functional.linear(x, a_dev), up.to(dev))
+    assert model.proj.lora_A.device.type == "cuda"
+    assert torch.equal(got, base + side.to(base.dtype))
+    assert torch.equal(model(x), base)                     # no entries in this call: the branch is gone again
