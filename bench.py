@@ -79,7 +79,7 @@ def make_config(i: int, rows: int | None = None) -> dict:
 
 # HBM-side bytes per GEMM launch of config 1, from two rocprofv3 --pmc runs of
 # comfyui-int8-fast_amd/profiling/traffic_probe.py (summary in profiles/hbm_traffic_fetch_write_size.txt):
-# FETCH_SIZE 139354 KiB / WRITE_SIZE 110592 KiB for 4608x12288x3072 and 153783 / 27648 KiB for
+# FETCH_SIZE 120105 KiB / WRITE_SIZE 110679 KiB for 4608x12288x3072 and 153807 / 27648 KiB for
 # 4608x3072x12288; a 256 MiB device copy reads 131084 / 262144 KiB on the same counters, so fetches
 # scale by 2.00 and writes by 1.00.  The mean of the two launches:
 GEMM_TRAFFIC_BYTES = int(((120105 * 2.0 + 110679) + (153807 * 2.0 + 27648)) / 2 * 1024)
@@ -214,6 +214,31 @@ def extras(L, dev, quick=False):
     out["skinny_gemm_256x12288x3072"] = {"median_us": round(t["median_us"], 2),
                                          "tops": round(2 * 256 * Nw * Kw / t["median_us"] / 1e6, 1)}
     del noises, outs
+
+    # config 2: QuaRot layer (width 3840, 2 % of the channels x50): time of the rotated path and what the
+    # rotation buys in accuracy against the bf16 product
+    c2 = make_config(2)
+    x2, w2 = c2["x"].to(dev), c2["w"].to(dev)
+    wq_r, ws_r = L.quant_rowwise(w2, rotate=True)
+    wq_p, ws_p = L.quant_rowwise(w2)
+    y2 = torch.empty(x2.shape[0], w2.shape[0], dtype=torch.bfloat16, device=dev)
+
+    def rot_linear(_i):
+        q_, s_ = L.quant_rowwise(x2, rotate=True)
+        L.linear_w8a8(q_, s_, wq_r, ws_r, None, torch.bfloat16, L.EPI_TORCH, y2)
+
+    t = time_kernel(rot_linear, max(10, iters // 4))
+    ref2 = x2.float() @ w2.bfloat16().float().T
+    rot_linear(0)
+    err_rot = ((y2.float() - ref2).norm() / ref2.norm()).item()
+    q_, s_ = L.quant_rowwise(x2)
+    err_plain = ((L.linear_w8a8(q_, s_, wq_p, ws_p, None, torch.bfloat16, L.EPI_TORCH).float() - ref2).norm() / ref2.norm()).item()
+    out["quarot_linear_4096x3840x3840"] = {"median_us": round(t["median_us"], 2),
+                                           "tops": round(2 * 4096 * 3840 * 3840 / t["median_us"] / 1e6, 1),
+                                           "rel_frobenius_error_rotated": round(err_rot, 5),
+                                           "rel_frobenius_error_unrotated": round(err_plain, 5),
+                                           "note": "rotate + quantise + GEMM; errors against the bf16 product x @ W.T"}
+    del x2, w2, ref2, y2
 
     # config 3: the linears of one double-stream DiT block (attention stays bf16 and is not counted)
     c3 = make_config(3)
