@@ -359,40 +359,14 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
     }
 }
 
-// rows a wave walks; development probes may override it through I8F_QUANT_NROW
-static int nrow_for(int64_t M) {
-    static const int forced = [] {
-        const char *e = getenv("I8F_QUANT_NROW");
-        return e ? atoi(e) : 0;
-    }();
-    if (forced >= 1 && forced <= 4) return forced;
-    return 1;
-}
-
-// development probe: dynamic LDS per block, which caps the blocks resident on a CU
-static unsigned lds_probe() {
-    static const unsigned v = [] {
-        const char *e = getenv("I8F_QUANT_LDS");
-        return e ? (unsigned)atoi(e) : 0u;
-    }();
-    return v;
-}
-
 template <int DT, bool ROT, int WPR, int RUNS>
 int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st) {
+    // One row per wave (NROW = 1): walking several rows per wave with the next row's loads in flight
+    // measured slower at every size (fewer, longer-lived waves ramp up and drain more slowly).
     constexpr int ROWS = 256 / (64 * WPR);
-    const int nrow = WPR == 1 ? nrow_for(M) : 1;
-    const int64_t blocks = (M + (int64_t)ROWS * nrow - 1) / ((int64_t)ROWS * nrow);
-    const char *xc = (const char *)x;
-    if constexpr (WPR == 1) {
-        switch (nrow) {
-        case 2: hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 2>), dim3((unsigned)blocks), dim3(256), 0, st, xc, M, K, ldx * 2, q, scale); return check_launch();
-        case 3: hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 3>), dim3((unsigned)blocks), dim3(256), 0, st, xc, M, K, ldx * 2, q, scale); return check_launch();
-        case 4: hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 4>), dim3((unsigned)blocks), dim3(256), 0, st, xc, M, K, ldx * 2, q, scale); return check_launch();
-        default: break;
-        }
-    }
-    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1>), dim3((unsigned)blocks), dim3(256), lds_probe(), st, xc, M, K, ldx * 2, q, scale);
+    const int64_t blocks = (M + ROWS - 1) / ROWS;
+    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1>), dim3((unsigned)blocks), dim3(256), 0, st, (const char *)x, M, K,
+                       ldx * 2, q, scale);
     return check_launch();
 }
 
