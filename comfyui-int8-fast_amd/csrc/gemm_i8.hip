@@ -618,6 +618,7 @@ using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8>;  // 12 waves of 64 x 96, the sam
 // loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
 // flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
 using CfgMidDeep = Cfg<128, 128, 128, 2, 2, 4, 8>;
+using CfgM96Deep = Cfg<128, 96, 128, 4, 1, 4, 8>;
 using CfgS64Deep = Cfg<128, 64, 128, 2, 2, 4, 8>;
 using CfgT64Deep = Cfg<64, 64, 128, 2, 2, 4, 8>;
 
@@ -682,12 +683,25 @@ int launch(GemmArgs &g, hipStream_t st) {
     if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64Deep, OUT>(g, st);
     if (I8F_FORCE_CFG == 5) return launch_cfg<CfgTall, OUT>(g, st);
     if (I8F_FORCE_CFG == 6) return launch_cfg<CfgWide, OUT>(g, st);
+    if (I8F_FORCE_CFG == 7) return launch_cfg<CfgM96Deep, OUT>(g, st);
+    if (I8F_FORCE_CFG == 8) return launch_cfg<CfgMidDeep, OUT>(g, st);
+    if (I8F_FORCE_CFG == 9) return launch_cfg<CfgS64Deep, OUT>(g, st);
 #endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
         if (mid_tiles >= CUS) return launch_cfg<CfgMid, OUT>(g, st);
-        if (mid_tiles >= 192) return launch_cfg<CfgMidDeep, OUT>(g, st);
-        if ((int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64) >= 192) return launch_cfg<CfgS64Deep, OUT>(g, st);
+        // Few tiles: the global->LDS path of a CU is what bounds these shapes, so a configuration costs
+        // the bytes its busiest CU has to fetch: (BM + BN) per K-step times the tiles that CU gets.
+        // Ties go to the larger tile (less traffic in total).
+        auto fetch_cost = [&](int bm, int bn) {
+            const int64_t tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
+            return ((tiles + CUS - 1) / CUS) * (bm + bn);
+        };
+        const int64_t f_mid = fetch_cost(128, 128), f_96 = fetch_cost(128, 96), f_s64 = fetch_cost(128, 64), f_t64 = fetch_cost(64, 64);
+        const int64_t f_min = std::min(std::min(f_mid, f_96), std::min(f_s64, f_t64));
+        if (f_mid == f_min) return launch_cfg<CfgMidDeep, OUT>(g, st);
+        if (f_96 == f_min) return launch_cfg<CfgM96Deep, OUT>(g, st);
+        if (f_s64 == f_min) return launch_cfg<CfgS64Deep, OUT>(g, st);
         return launch_cfg<CfgT64Deep, OUT>(g, st);
     }
     const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108);

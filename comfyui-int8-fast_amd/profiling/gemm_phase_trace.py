@@ -64,12 +64,11 @@ def main():
             cands = [(cost(256, 256, 100), (256, 256)), (cost(288, 256, 102), (288, 256)),
                      (cost(256, 288, 102), (256, 288)), (cost(256, 192, 108), (256, 192))]
             BM, BN = min(cands, key=lambda c: c[0])[1]      # ties go to the first, as in the library
-        elif mid >= 192:
+        elif mid >= 256:
             BM, BN = 128, 128
-        elif cd(M, 128) * cd(N, 64) >= 192:
-            BM, BN = 128, 64
-        else:
-            BM, BN = 64, 64
+        else:   # few tiles: bytes the busiest CU fetches per K-step; ties go to the first, as in the library
+            fetch = lambda bm, bn: cd(cd(M, bm) * cd(N, bn), 256) * (bm + bn)
+            BM, BN = min([(128, 128), (128, 96), (128, 64), (64, 64)], key=lambda t: fetch(*t))
     dev = torch.device("cuda:0")
     x, w = operands(M, N, K, a.data, dev)
     xs, ws = torch.rand(M, device=dev) * 0.01, torch.rand(N, device=dev) * 0.01
