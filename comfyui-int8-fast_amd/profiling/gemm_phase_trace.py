@@ -61,8 +61,8 @@ def main():
         big, mid = cd(M, 256) * cd(N, 256), cd(M, 128) * cd(N, 128)
         cost = lambda bm, bn, per_op: cd(cd(M, bm) * cd(N, bn), 256) * bm * bn * per_op
         if big >= 128:
-            cands = [(cost(256, 256, 100), (256, 256)), (cost(288, 256, 102), (288, 256)),
-                     (cost(256, 288, 102), (256, 288)), (cost(256, 192, 108), (256, 192))]
+            cands = [(cost(256, 256, 100), (256, 256)), (cd(mid, 512) * 2 * 128 * 128 * 141, (128, 128)),
+                     (cost(288, 256, 102), (288, 256)), (cost(256, 288, 102), (256, 288)), (cost(256, 192, 108), (256, 192))]
             BM, BN = min(cands, key=lambda c: c[0])[1]      # ties go to the first, as in the library
         elif mid >= 256:
             BM, BN = 128, 128
