@@ -617,6 +617,7 @@ using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8>;  // 12 waves of 64 x 96, the sam
 // Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
 // loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
 // flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
+using CfgW96 = Cfg<256, 96, 128, 8, 1, 3, 8>;      // 8 waves of 32 x 96, 3 x 44 KB stages
 using CfgMidDeep = Cfg<128, 128, 128, 2, 2, 4, 8>;
 using CfgM96Deep = Cfg<128, 96, 128, 4, 1, 4, 8>;
 using CfgS64Deep = Cfg<128, 64, 128, 2, 2, 4, 8>;
@@ -686,10 +687,19 @@ int launch(GemmArgs &g, hipStream_t st) {
     if (I8F_FORCE_CFG == 7) return launch_cfg<CfgM96Deep, OUT>(g, st);
     if (I8F_FORCE_CFG == 8) return launch_cfg<CfgMidDeep, OUT>(g, st);
     if (I8F_FORCE_CFG == 9) return launch_cfg<CfgS64Deep, OUT>(g, st);
+    if (I8F_FORCE_CFG == 10) return launch_cfg<CfgW96, OUT>(g, st);
 #endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
-        if (mid_tiles >= CUS) return launch_cfg<CfgMid, OUT>(g, st);
+        if (mid_tiles >= CUS) {
+            // Two 128 x 128 tiles to a CU fetch 2 x 256 rows per K-step, one 256 x 96 tile 352: the
+            // narrow tile wins where it still covers the output in one round (512 x 12288: 256 tiles).
+            const int64_t w96_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 95) / 96);
+            const int64_t f_w96 = ((w96_tiles + CUS - 1) / CUS) * (256 + 96);
+            const int64_t f_mid2 = ((mid_tiles + 2 * CUS - 1) / (2 * CUS)) * 2 * (128 + 128);
+            if (f_w96 < f_mid2) return launch_cfg<CfgW96, OUT>(g, st);
+            return launch_cfg<CfgMid, OUT>(g, st);
+        }
         // Few tiles: the global->LDS path of a CU is what bounds these shapes, so a configuration costs
         // the bytes its busiest CU has to fetch: (BM + BN) per K-step times the tiles that CU gets.
         // Ties go to the larger tile (less traffic in total).

@@ -65,7 +65,8 @@ def main():
                      (cost(288, 256, 102), (288, 256)), (cost(256, 288, 102), (256, 288)), (cost(256, 192, 108), (256, 192))]
             BM, BN = min(cands, key=lambda c: c[0])[1]      # ties go to the first, as in the library
         elif mid >= 256:
-            BM, BN = 128, 128
+            w96 = cd(M, 256) * cd(N, 96)
+            BM, BN = (256, 96) if cd(w96, 256) * 352 < cd(mid, 512) * 512 else (128, 128)
         else:   # few tiles: bytes the busiest CU fetches per K-step; ties go to the first, as in the library
             fetch = lambda bm, bn: cd(cd(M, bm) * cd(N, bn), 256) * (bm + bn)
             BM, BN = min([(128, 128), (128, 96), (128, 64), (64, 64)], key=lambda t: fetch(*t))

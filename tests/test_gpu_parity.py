@@ -129,7 +129,9 @@ GEMM_CASES = [(256, 256, 64), (256, 256, 3072), (300, 520, 1040), (128, 128, 128
               # 256x288 tiles of twelve waves
               (4090, 4600, 144), (4096, 4608, 128),
               # long K, few tiles: the four-stage configurations (128x128, 128x64, 64x64, 128x96)
-              (1000, 3080, 8200), (500, 3072, 8192), (200, 520, 8320), (250, 9200, 144), (256, 12288, 256)]
+              (1000, 3080, 8200), (500, 3072, 8192), (200, 520, 8320), (250, 9200, 144), (256, 12288, 256),
+              # 256x96 tiles, three stages (one round of them instead of two 128x128 tiles per CU)
+              (500, 9200, 144), (512, 12288, 384)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_CASES)
@@ -204,6 +206,9 @@ LIN_CASES = [
     (4090, 4600, 80, True, torch.bfloat16, torch.bfloat16, 0), (4096, 4608, 128, False, torch.float32, torch.float32, 1),
     # 128x96 tiles (four waves of 32x96)
     (250, 9200, 144, True, torch.bfloat16, torch.bfloat16, 0), (256, 9216, 128, False, torch.float16, torch.float32, 1),
+    # 256x96 tiles
+    (500, 9200, 144, True, torch.bfloat16, torch.bfloat16, 0), (512, 9216, 128, False, torch.float32, torch.float32, 1),
+    (384, 12288, 272, True, torch.float16, torch.float16, 1),
 ]
 
 
