@@ -231,6 +231,36 @@ def test_linear_w8a8_bit_exact(L, dev, M, N, K, row, bdt, odt, order):
         assert np.array_equal(bits(got2), want)
 
 
+def test_linear_w8a8_random_shapes_and_flags(L, dev):
+    """24 seeded cases over the whole range of output sizes (every tile configuration the host can pick),
+    with the scale mode, bias dtype, output dtype and operation order drawn at random; K stays short so
+    that the CPU side finishes in seconds."""
+    rng = np.random.default_rng(777)
+    dts = [torch.bfloat16, torch.float16, torch.float32]
+    sizes = [(4608, 12288), (4096, 9216), (4608, 3072), (2048, 4096), (640, 12288), (512, 12288), (512, 9216), (256, 9216),
+             (512, 3072), (256, 3072), (1024, 3072), (100, 18432)]
+    for case in range(24):
+        M0, N0 = sizes[case % len(sizes)]
+        M = int(M0 - rng.integers(0, 40))
+        N = int(N0 - 8 * rng.integers(0, 12))
+        K = int(rng.integers(1, 20)) * 16
+        row, order = bool(rng.integers(0, 2)), int(rng.integers(0, 2))
+        bdt = [None, *dts][int(rng.integers(0, 4))]
+        odt = dts[int(rng.integers(0, 3))] if case % 4 == 0 else dts[int(rng.integers(0, 2))]
+        x = acts(M, K)
+        wf = torch.randn(N, K, generator=G) * 0.02
+        wq, ws = O.quant_rowwise(wf.numpy(), O.F32) if row else O.quant_tensorwise(wf.numpy(), O.F32)
+        bias = None if bdt is None else (torch.randn(N, generator=G) * 0.01).to(bdt)
+        xa, code = O.from_torch(x)
+        ocode = {torch.bfloat16: O.BF16, torch.float16: O.F16, torch.float32: O.F32}[odt]
+        ba, bcode = (None, O.BF16) if bias is None else O.from_torch(bias)
+        want = O.linear_w8a8(xa, code, wq, ws, ba, bcode, ocode, 0, order)
+        q, s = L.quant_rowwise(x.to(dev))
+        ws_arg = torch.from_numpy(ws).to(dev) if row else float(ws[0])
+        got = L.linear_w8a8(q, s, torch.from_numpy(wq).to(dev), ws_arg, None if bias is None else bias.to(dev), odt, order)
+        assert np.array_equal(bits(got), want), (M, N, K, row, bdt, odt, order)
+
+
 @pytest.mark.parametrize("M,N,K,odt,order", [(300, 520, 1040, torch.bfloat16, 0), (2000, 2056, 200, torch.float16, 1),
                                              (4100, 2056, 144, torch.bfloat16, 0), (64, 50, 50, torch.bfloat16, 0),
                                              (256, 256, 512, torch.float32, 0),
