@@ -209,8 +209,13 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
     a_scale = a_scale.contiguous()
     ws, ws_host, mode = _scale(w_scale, N, a.device)
     bias, bcode = _bias_arg(bias, N, a.device)
+    for name, t in (("w", w), ("a_scale", a_scale), ("addend", addend), ("out", out)):
+        if isinstance(t, torch.Tensor) and t.device != a.device:
+            raise ValueError(f"{name} is on {t.device}, a is on {a.device}")
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    elif tuple(out.shape) != (M, N) or not out.is_contiguous() or out.dtype not in _DT:
+        raise ValueError(f"out must be a contiguous [{M},{N}] tensor of bfloat16, float16 or float32")
     if addend is not None:
         _dev(addend, "addend")
         if addend.numel() != M * N or addend.dtype != out.dtype:

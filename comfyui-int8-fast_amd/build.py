@@ -92,45 +92,9 @@ def build(force: bool = False, keep_temps: bool = False, verbose: bool = True) -
     return LIB
 
 
-# Instrumented builds of the GEMM for profiling/gemm_phase_trace.py: the product sources compiled
-# with per-workgroup time stamps (I8F_TRACE) and, for the ablations, with one part of the main loop
-# removed.  They are separate libraries; the product library contains none of this.
-PROBES = {
-    "trace": [],
-    "mfma_only": ["-DI8F_ABLATE_DMA", "-DI8F_ABLATE_LDSREAD"],
-    "dma_only": ["-DI8F_ABLATE_MFMA", "-DI8F_ABLATE_LDSREAD"],
-    "no_store": ["-DI8F_ABLATE_STORE"],
-}
-
-
-def probe_path(name: str) -> str:
-    return os.path.join(HERE, "profiling", f"libi8f_probe_{name}.so")
-
-
-def build_probes(names=None, force: bool = False) -> list[str]:
-    cc = hipcc()
-    srcs = [os.path.join(CSRC, "gemm_i8.hip"), os.path.join(CSRC, "i8f_api.hip")]
-    deps = srcs + glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(HERE, "..", "include", "*.h"))
-    todo = [n for n in (names or PROBES) if force or _stale(probe_path(n), deps)]
-
-    def run(name):
-        cmd = [cc, *FLAGS, "-DI8F_TRACE", *PROBES[name], "-shared", "-o", probe_path(name), *srcs]
-        p = subprocess.run(cmd, capture_output=True, text=True)
-        if p.returncode != 0:
-            raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + p.stderr)
-        return probe_path(name)
-
-    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as ex:
-        list(ex.map(run, todo))
-    return [probe_path(n) for n in (names or PROBES)]
-
-
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
     ap.add_argument("--keep-temps", action="store_true")
-    ap.add_argument("--probes", action="store_true", help="also build the instrumented GEMM libraries under profiling/")
     a = ap.parse_args()
     print(build(force=a.force, keep_temps=a.keep_temps))
-    if a.probes:
-        print("\n".join(build_probes(force=a.force)))

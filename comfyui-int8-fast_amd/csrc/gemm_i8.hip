@@ -26,9 +26,6 @@
 
 #include "i8f_common.hpp"
 #include <algorithm>
-#ifdef I8F_TRACE
-#include <cstdlib>
-#endif
 
 namespace i8f {
 namespace {
@@ -52,9 +49,6 @@ struct GemmArgs {
     const void *addend;  // nullptr or [M,N] of the output dtype, added to the rounded result
     void *out;
     int tiles_m, tiles_n;
-#ifdef I8F_TRACE
-    long long *trace;  // [blocks][8] wall-clock stamps: start, first tile landed, loop done, end, + epilogue detail
-#endif
 };
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_>
@@ -226,9 +220,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         tile_n = r / gsz;
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-#ifdef I8F_TRACE
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 0] = wall_clock64();
-#endif
 
     // ---- epilogue operands: fetched once, long before they are needed ----------------------
     if constexpr (OUT != OUT_I32) {
@@ -321,10 +312,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    auto load_frags = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI], bool force = false) {
-#ifdef I8F_ABLATE_LDSREAD  // development probe: fragments are read once, before the loop
-        if (!force) return;
-#endif
+    auto load_frags = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI]) {
 #pragma unroll
         for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ks]);
 #pragma unroll
@@ -332,11 +320,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     };
     auto mma_one = [&](const v4i (&xf)[MI], const v4i (&wf)[NI], int r) {
         const int i = r / NI, j = r % NI;
-#ifndef I8F_ABLATE_MFMA
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
-#else
-        acc[i][j][0] += xf[i][0] ^ wf[j][0];
-#endif
     };
 
     // ---- prologue: S tiles in flight, fragments of the first k-step in registers --------------
@@ -352,9 +336,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     for (int s = 0; s < PRE; ++s) issue(s, s < KT);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm((PRE - 1) * C::LOADS));  // tiles 1..PRE-1 may be in flight
     __syncthreads();  // tile 0 and the staged epilogue operands are visible to everyone
-#ifdef I8F_TRACE
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 1] = wall_clock64();
-#endif
 
     // Fragments are double-buffered in registers: the LDS reads of k-step s+1 are issued before
     // the MFMAs of k-step s, so the matrix pipe does not wait for LDS.  There is one barrier per
@@ -362,10 +343,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // (its last fragments are in registers), so the stage of tile kt is refilled with tile kt+S
     // right away, and tile kt+1 is known to have landed, so its first fragments can be fetched.
     v4i xa[MI] = {}, wa[NI] = {}, xb[MI] = {}, wb[NI] = {};
-    if (KT > 0) load_frags(smem, 0, xa, wa, true);
-#ifdef I8F_ABLATE_LDSREAD
-    load_frags(smem, 1, xb, wb, true);
-#endif
+    if (KT > 0) load_frags(smem, 0, xa, wa);
     // Drain scalar loads (kernel arguments) here: a scalar load still pending at the loop header
     // would turn every LDS wait inside the loop into a full lgkmcnt(0).
     __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -403,10 +381,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < MN; ++r) {
                 mma_one(xc, wc, r);
-#ifndef I8F_ABLATE_DMA
 #pragma unroll
                 for (int l = la + r * (lb - la) / MN; l < la + (r + 1) * (lb - la) / MN; ++l) issue_one(ft, live, l);
-#endif
                 __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -418,9 +394,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // destination: they must have landed before the stages are reused.
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();  // the stages are dead; reuse them as per-wave transpose buffers
-#ifdef I8F_TRACE
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 2] = wall_clock64();
-#endif
     char *ebuf = smem + wave * WAVE_BYTES;
 
     // scale, bias, round: the flags are wave-uniform, so the variant is chosen once
@@ -470,9 +443,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
             for (int j = 0; j < NI; ++j) fetch_cols(j, wr[j], br[j]);
         }
-#ifdef I8F_TRACE
-        if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 4] = wall_clock64();
-#endif
 #pragma unroll
         for (int i0 = 0; i0 < MI; i0 += EPI_STRIPS) {
 #pragma unroll
@@ -511,9 +481,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
                 }
             }
             __builtin_amdgcn_wave_barrier();
-#ifdef I8F_TRACE
-            if (tid == 0 && g.trace && i0 == 0) g.trace[blockIdx.x * 8 + 5] = wall_clock64();
-#endif
             // read the staged rows back row-contiguously and store 16 bytes per lane
             constexpr int CPO = ROW_BYTES / 16;      // chunks per output row
             constexpr int EPCO = 16 / OB;            // output elements per chunk
@@ -525,11 +492,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
                 const uint4 val = *(const uint4 *)(ebuf + row * PITCH + cc * 16);
                 const int mm = m0 + wm * C::WTM + i0 * 32 + row;
                 const int nn = n0 + wn * C::WTN + cc * EPCO;
-#ifdef I8F_ABLATE_STORE  // development probe: the store is kept in the code but never taken
-                if (mm < g.M && nn < g.N && val.x == 0x12345678u && val.y == 0x9abcdef0u)
-#else
                 if (mm < g.M && nn < g.N)
-#endif
                 {
                     const int64_t off = ((int64_t)mm * g.N + nn) * OB;
                     uint4 v = val;
@@ -538,9 +501,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
                 }
             }
             __builtin_amdgcn_wave_barrier();
-#ifdef I8F_TRACE
-            if (tid == 0 && g.trace && i0 == 0) g.trace[blockIdx.x * 8 + 6] = wall_clock64();
-#endif
         }
     };
     if constexpr (OUT == OUT_I32) {
@@ -557,11 +517,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         default: run_epilogue(O1{}, T_{}, T_{}); break;
         }
     }
-#ifdef I8F_TRACE
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 7] = wall_clock64();
-    __syncthreads();
-    if (tid == 0 && g.trace) g.trace[blockIdx.x * 8 + 3] = wall_clock64();
-#endif
 }
 
 // ---- slow but shape-agnostic kernel: one thread per output -----------------------------
@@ -628,9 +583,6 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
     g.tiles_m = (g.M + C::BM - 1) / C::BM;
     g.tiles_n = (g.N + C::BN - 1) / C::BN;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-#ifdef I8F_TRACE
-    g.trace = (long long *)(getenv("I8F_TRACE_PTR") ? strtoull(getenv("I8F_TRACE_PTR"), nullptr, 0) : 0ull);
-#endif
     if (g.K % C::BK) hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g);
     else hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g);
     return check_launch();
@@ -677,18 +629,6 @@ int launch(GemmArgs &g, hipStream_t st) {
         return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn * per_op_cost;
     };
     const int64_t big_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
-#ifdef I8F_FORCE_CFG  // development probe: one fixed configuration
-    if (I8F_FORCE_CFG == 1) return launch_cfg<CfgBig, OUT>(g, st);
-    if (I8F_FORCE_CFG == 2) return launch_cfg<CfgB192, OUT>(g, st);
-    if (I8F_FORCE_CFG == 3) return launch_cfg<CfgMid, OUT>(g, st);
-    if (I8F_FORCE_CFG == 4) return launch_cfg<CfgT64Deep, OUT>(g, st);
-    if (I8F_FORCE_CFG == 5) return launch_cfg<CfgTall, OUT>(g, st);
-    if (I8F_FORCE_CFG == 6) return launch_cfg<CfgWide, OUT>(g, st);
-    if (I8F_FORCE_CFG == 7) return launch_cfg<CfgM96Deep, OUT>(g, st);
-    if (I8F_FORCE_CFG == 8) return launch_cfg<CfgMidDeep, OUT>(g, st);
-    if (I8F_FORCE_CFG == 9) return launch_cfg<CfgS64Deep, OUT>(g, st);
-    if (I8F_FORCE_CFG == 10) return launch_cfg<CfgW96, OUT>(g, st);
-#endif
     if (big_tiles < 128) {
         const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
         if (mid_tiles >= CUS) {

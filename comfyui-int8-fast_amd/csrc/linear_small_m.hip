@@ -219,11 +219,16 @@ __global__ __launch_bounds__(WAVES * 64) void small_m_lds_kernel(const SmallMArg
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int h = 0; h < 2; ++h) *(v4u_t *)(tile + (b * 16 + h * 8 + lr) * PITCH + lc * 16) = wq[buf][b][h];
+        // the tile is private to the wave, but a lane reads what other lanes wrote: fence the exchange
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         v2u_t wa[NB][4];
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int j = 0; j < 4; ++j) wa[b][j] = *(const v2u_t *)(tile + (b * 16 + r) * PITCH + g * 32 + 8 * j);
+        __builtin_amdgcn_wave_barrier();  // every lane has its operands before the tile is overwritten
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll

@@ -21,6 +21,7 @@ from ._comfy_compat import (
     uncast_bias_weight,
 )
 from .int8_fused_kernel import hip_int8_linear, hip_int8_linear_per_row
+from .dynamic_lora import DynamicLoRAHook  # noqa: F401  (int8_dynamic_lora.py:40 of the reference imports it from here)
 
 # Rows at or below this use the W8A16 small-batch kernel (int8_quant.py:751 of the reference).
 SMALL_BATCH_ROWS = 16

@@ -57,8 +57,14 @@ typedef enum i8f_scale_mode { I8F_SCALE_TENSOR = 0, I8F_SCALE_ROW = 1 } i8f_scal
  *                  the bias (itself rounded to the output dtype) and round again.
  *                  Bit-identical to that path on the CPU.  The default of the
  *                  Python host layer.
- *   I8F_EPI_FUSED  the reference's fused kernels (int8_fused_kernel.py:156-173,
- *                  310-324): acc * (xs * ws) + bias in binary32, one rounding.
+ *   I8F_EPI_FUSED  the operation order of the reference's fused kernels
+ *                  (int8_fused_kernel.py:156-173, 310-324): acc * (xs * ws),
+ *                  then + bias, each a rounded binary32 operation, then one
+ *                  rounding to the output dtype.  The reference's compiler may
+ *                  contract the multiply and the add into one fused multiply-add
+ *                  on its device; this library never does, so bit-for-bit parity
+ *                  with those kernels is unpinned (the two differ by at most one
+ *                  binary32 rounding before the final rounding).
  */
 typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
 
