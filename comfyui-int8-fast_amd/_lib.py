@@ -52,13 +52,16 @@ def lib() -> ctypes.CDLL:
     L.i8f_last_hip_error.restype = i32
     L.i8f_quant_rowwise.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, vp]
     L.i8f_rotate128.argtypes = [vp, i32, i64, i64, i64, vp, vp]
+    L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
+    L.i8f_quant_tensorwise_workspace_bytes.restype = i64
+    L.i8f_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp, vp, i64, vp]
     L.i8f_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp, vp]
     L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
+    for name in ("i8f_quant_rowwise", "i8f_quant_tensorwise", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -67,6 +70,7 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
+    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise",
     "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
@@ -144,6 +148,23 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False):
     with torch.cuda.device(x.device):
         _check(lib().i8f_quant_rowwise(_ptr(x), dtype_code(x.dtype), M, K, ldx, 128 if rotate else 0, _ptr(q), _ptr(s),
                                        _stream(x)), "i8f_quant_rowwise")
+    return q, s
+
+
+def quant_tensorwise(x: torch.Tensor):
+    """x (any shape; bf16/fp16/fp32, cuda) -> (int8 like x, 0-dim float32 scale): one absmax scale for the tensor."""
+    _dev(x, "x")
+    if x.dtype not in _DT:
+        raise TypeError(f"unsupported dtype {x.dtype}; expected bfloat16, float16 or float32")
+    xc = x if x.is_contiguous() else x.contiguous()
+    n = xc.numel()
+    q = torch.empty(xc.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty((), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        nbytes = lib().i8f_quant_tensorwise_workspace_bytes(n)
+        ws = torch.empty(max(1, nbytes // 4), dtype=torch.float32, device=x.device)
+        _check(lib().i8f_quant_tensorwise(_ptr(xc), dtype_code(x.dtype), n, _ptr(q), _ptr(s), _ptr(ws), ws.numel() * 4,
+                                          _stream(x)), "i8f_quant_tensorwise")
     return q, s
 
 

@@ -51,9 +51,13 @@ struct GemmArgs {
     int tiles_m, tiles_n;
 };
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_>
+// SPLIT_ (two-stage configurations): how a wave's loads of one K-tile are dealt over the phases that
+// follow the barrier which frees their stage, one hex digit per phase, first phase in the top digit
+// (0 = all of them in the first phase).
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_, int SPLIT_ = 0>
 struct Cfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_, GROUP_M = GROUP_M_;
+    static constexpr int SPLIT = SPLIT_;
     static constexpr int NW = WM * WN;
     static constexpr int NT = NW * 64;
     static constexpr int WTM = BM / WM, WTN = BN / WN;  // per-wave tile
@@ -324,17 +328,33 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     };
 
     // ---- prologue: S tiles in flight, fragments of the first k-step in registers --------------
-    // Two ways to keep the stages full.  With two stages a stage is refilled in one burst, right
-    // after the barrier that frees it (tile kt+S during the last phase of iteration kt).  With three
+    // Two ways to keep the stages full.  With two stages a stage is refilled right after the barrier
+    // that frees it (tile kt+S from the last phase of iteration kt on), in one burst or, by the SPLIT
+    // of the configuration, over that phase and the following ones of iteration kt+1.  With three
     // or more the refill of the stage freed by the PREVIOUS iteration is dealt out over the whole of
     // iteration kt (tile kt+S-1): a wave that issues many loads at once blocks on the load queue, and
     // while it is blocked it issues no MFMAs either.  Loads past the last tile are issued all the
     // same (they move nothing), so the number of loads in flight at any point is a constant.
     constexpr bool SPREAD_DMA = S >= 3;
     constexpr int PRE = SPREAD_DMA ? S - 1 : S;  // tiles issued before the loop
+    // two stages: loads [cut(p), cut(p+1)) of a tile go out in the p-th phase after the barrier
+    auto cut = [](int p) constexpr {
+        if (C::SPLIT == 0) return p <= 0 ? 0 : C::LOADS;
+        int c = 0;
+        for (int q = 0; q < p && q < KS; ++q) c += (C::SPLIT >> (4 * (KS - 1 - q))) & 0xf;
+        return c;
+    };
+    static_assert(SPREAD_DMA || cut(KS) == C::LOADS, "the split has to cover every load of a tile");
 #pragma unroll
-    for (int s = 0; s < PRE; ++s) issue(s, s < KT);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm((PRE - 1) * C::LOADS));  // tiles 1..PRE-1 may be in flight
+    for (int s = 0; s < PRE; ++s) {
+        if (!SPREAD_DMA && s == PRE - 1) {
+#pragma unroll
+            for (int r = 0; r < cut(1); ++r) issue_one(s, s < KT, r);  // the rest follows inside the loop
+        } else {
+            issue(s, s < KT);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(SPREAD_DMA ? (PRE - 1) * C::LOADS : cut(1)));  // younger tiles may be in flight
     __syncthreads();  // tile 0 and the staged epilogue operands are visible to everyone
 
     // Fragments are double-buffered in registers: the LDS reads of k-step s+1 are issued before
@@ -359,7 +379,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
                 // my part of tile kt+1 has landed and my LDS reads of tile kt have returned; what may
                 // still be in flight are the younger tiles (and, spread, the part of the newest one
                 // that the earlier phases of this iteration have issued)
-                constexpr int YOUNGER = SPREAD_DMA ? (S - 3) * C::LOADS + (KS - 1) * C::LOADS / KS : (S - 2) * C::LOADS;
+                constexpr int YOUNGER = SPREAD_DMA ? (S - 3) * C::LOADS + (KS - 1) * C::LOADS / KS : 0;
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(YOUNGER) & 0xF0FF);
                 __builtin_amdgcn_s_barrier();
             }
@@ -372,12 +392,14 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
             const int fks = last ? 0 : ks + 1;
             load_frags(fsrc, fks, xn, wn_);
             __builtin_amdgcn_sched_barrier(0);
-            const int ft = SPREAD_DMA ? kt + S - 1 : kt + S;  // the tile being fetched
+            // the tile being fetched: two stages refill the stage that this iteration's barrier frees
+            // (tile kt+2) from the last phase on and finish in the following phases of the next iteration
+            const int ft = SPREAD_DMA ? kt + S - 1 : (last ? kt + S : kt + S - 1);
             const bool live = ft < KT;
             (void)live;
-            // this phase's share of its loads: all of them in the last phase (burst), 1/KS of them (spread)
-            const int la = SPREAD_DMA ? ks * C::LOADS / KS : 0;
-            const int lb = SPREAD_DMA ? (ks + 1) * C::LOADS / KS : (last ? C::LOADS : 0);
+            // this phase's share of its loads
+            const int la = SPREAD_DMA ? ks * C::LOADS / KS : (last ? 0 : cut(ks + 1));
+            const int lb = SPREAD_DMA ? (ks + 1) * C::LOADS / KS : (last ? cut(1) : cut(ks + 2));
 #pragma unroll
             for (int r = 0; r < MN; ++r) {
                 mma_one(xc, wc, r);
@@ -564,7 +586,7 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 }
 
 // tile configurations
-using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6>;   // 8 waves, 2 x 64 KB stages, one workgroup per CU
+using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400>;  // 8 waves, 2 x 64 KB stages, one workgroup per CU; refill in two halves (2-3 % faster than one burst)
 using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
 using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8>;  // 12 waves of 96 x 64, 2 x 72 KB stages

@@ -96,6 +96,23 @@ int i8f_quant_rowwise(const void *x, int x_dtype, int64_t M, int64_t K, int64_t 
                       int rotate_block, int8_t *q, float *scale, void *stream);
 
 /*
+ * One absmax scale for a whole tensor, then int8 quantisation with it.
+ * Replaces quantize_int8_tensorwise (int8_quant.py:23-26), the load-time
+ * quantiser of tensorwise checkpoints and of BASELINE config 0's weight:
+ *   scale = max(float(max|x|) / 127, 1e-30),  q = sat8(rne(float(x) * (1 / scale)))
+ * in two launches that use the whole GPU (the partial maxima of the first launch
+ * are what the workspace holds).
+ *   x        n elements of x_dtype, contiguous      q   n int8      scale   1 float
+ *   workspace        device memory of at least i8f_quant_tensorwise_workspace_bytes(n)
+ *                    bytes, 4-byte aligned, owned by the caller; contents need no
+ *                    initialisation and are garbage afterwards
+ * n == 0 writes scale = 1e-30.
+ */
+int64_t i8f_quant_tensorwise_workspace_bytes(int64_t n);
+int i8f_quant_tensorwise(const void *x, int x_dtype, int64_t n, int8_t *q, float *scale,
+                         void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * Block rotation alone (no quantisation): every aligned block of 128 elements of
  * each row is multiplied by the normalised Hadamard matrix, result in x's dtype.
  * Replaces rotate_weight / rotate_activation (quarot.py:42-102) where the rotated

@@ -61,6 +61,41 @@ def test_quant_rowwise_bit_exact(L, dev, M, K, dt, rot):
     assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
 
 
+TENSORWISE_CASES = [
+    # shape, dtype
+    ((3072, 3072), torch.bfloat16), ((3072, 3072), torch.float32), ((1, 1), torch.float32), ((7,), torch.float16),
+    ((5, 1001), torch.bfloat16), ((16 * 1024 + 3,), torch.float32), ((1024 * 16 * 1024 + 40,), torch.bfloat16),
+    ((257, 4099), torch.float16), ((12288, 3072), torch.float32),
+]
+
+
+@pytest.mark.parametrize("shape,dt", TENSORWISE_CASES)
+def test_quant_tensorwise_bit_exact(L, dev, shape, dt):
+    """quantize_int8_tensorwise through i8f_quant_tensorwise: one slice, ragged slices, more slices than
+    partial slots; int8 and the scale bit-exact against the oracle."""
+    x = (torch.randn(*shape, generator=G) * 0.02).to(dt)
+    xa, code = O.from_torch(x)
+    qo, so = O.quant_tensorwise(xa, code)
+    q, s = L.quant_tensorwise(x.to(dev))
+    assert q.shape == x.shape and s.shape == ()
+    assert np.array_equal(q.cpu().numpy(), qo.reshape(x.shape))
+    assert np.array_equal(s.cpu().numpy().reshape(1).view(np.uint32), np.asarray(so).reshape(1).view(np.uint32))
+
+
+def test_quant_tensorwise_edge_cases(L, dev):
+    z = torch.zeros(4, 300, dtype=torch.bfloat16, device=dev)          # all zero: scale clamps to 1e-30
+    q, s = L.quant_tensorwise(z)
+    assert not q.any() and s.item() == np.float32(1e-30)
+    e = torch.empty(0, dtype=torch.float32, device=dev)                # empty: scale only
+    q, s = L.quant_tensorwise(e)
+    assert q.numel() == 0 and s.item() == np.float32(1e-30)
+    base = torch.randn(70001, generator=G).to(dev)                     # misaligned views take the scalar kernels
+    for view in (base[1:], base[3:40000]):
+        qo, so = O.quant_tensorwise(view.cpu().numpy().copy(), O.F32)
+        q, s = L.quant_tensorwise(view)
+        assert np.array_equal(q.cpu().numpy(), qo) and s.item() == so[0].item()
+
+
 def test_quant_rowwise_strided_and_misaligned_views(L, dev):
     big = acts(40, 1100).to(dev)
     for view in (big[:, :1024], big[:, 3:1027], big[::2, 8:520], big[5:6, 1:130]):
