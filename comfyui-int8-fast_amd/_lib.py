@@ -55,13 +55,14 @@ def lib() -> ctypes.CDLL:
     L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
     L.i8f_quant_tensorwise_workspace_bytes.restype = i64
     L.i8f_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp, vp, i64, vp]
+    L.i8f_quant_tensorwise_static.argtypes = [vp, i32, i64, vp, vp, vp]
     L.i8f_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp, vp]
     L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_tensorwise", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
+    for name in ("i8f_quant_rowwise", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -70,7 +71,7 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
-    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise",
+    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static",
     "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
@@ -151,8 +152,10 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False):
     return q, s
 
 
-def quant_tensorwise(x: torch.Tensor):
-    """x (any shape; bf16/fp16/fp32, cuda) -> (int8 like x, 0-dim float32 scale): one absmax scale for the tensor."""
+def quant_tensorwise(x: torch.Tensor, static_scratch: bool = False):
+    """x (any shape; bf16/fp16/fp32, cuda) -> (int8 like x, 0-dim float32 scale): one absmax scale for the tensor.
+    static_scratch=True uses the library's own device array for the partial maxima instead of a torch workspace
+    (the call then allocates nothing beyond q and scale, which the caller may also preallocate via the C ABI)."""
     _dev(x, "x")
     if x.dtype not in _DT:
         raise TypeError(f"unsupported dtype {x.dtype}; expected bfloat16, float16 or float32")
@@ -161,10 +164,14 @@ def quant_tensorwise(x: torch.Tensor):
     q = torch.empty(xc.shape, dtype=torch.int8, device=x.device)
     s = torch.empty((), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        nbytes = lib().i8f_quant_tensorwise_workspace_bytes(n)
-        ws = torch.empty(max(1, nbytes // 4), dtype=torch.float32, device=x.device)
-        _check(lib().i8f_quant_tensorwise(_ptr(xc), dtype_code(x.dtype), n, _ptr(q), _ptr(s), _ptr(ws), ws.numel() * 4,
-                                          _stream(x)), "i8f_quant_tensorwise")
+        if static_scratch:
+            _check(lib().i8f_quant_tensorwise_static(_ptr(xc), dtype_code(x.dtype), n, _ptr(q), _ptr(s), _stream(x)),
+                   "i8f_quant_tensorwise_static")
+        else:
+            nbytes = lib().i8f_quant_tensorwise_workspace_bytes(n)
+            ws = torch.empty(max(1, nbytes // 4), dtype=torch.float32, device=x.device)
+            _check(lib().i8f_quant_tensorwise(_ptr(xc), dtype_code(x.dtype), n, _ptr(q), _ptr(s), _ptr(ws), ws.numel() * 4,
+                                              _stream(x)), "i8f_quant_tensorwise")
     return q, s
 
 

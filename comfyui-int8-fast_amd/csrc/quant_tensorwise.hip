@@ -7,9 +7,12 @@
 //                                   derives scale and reciprocal exactly as the row quantiser does, and
 //                                   quantises its slice; workgroup 0 writes the scale
 //
-// The partial maxima are the only device memory beyond inputs and outputs; they live in a workspace
-// of the caller.  Nothing has to be cleared between calls: pass 1 writes every slot that pass 2 of
-// the same call reads.
+// The partial maxima are the only device memory beyond inputs and outputs.  They live either in a
+// workspace of the caller (i8f_quant_tensorwise) or in a file-scope device array of this library
+// (i8f_quant_tensorwise_static, for callers that cannot allocate).  Nothing has to be cleared between
+// calls: pass 1 writes every slot that pass 2 of the same call reads.
+#include <mutex>
+
 #include "i8f_common.hpp"
 
 namespace i8f {
@@ -18,6 +21,11 @@ namespace {
 constexpr int MAX_PARTIALS = 1024;               // slots of the partial-maximum buffer
 constexpr int TPB = 256;                         // threads per workgroup
 constexpr int64_t SLICE_MIN = 16 * 1024;         // elements: below this a slice is not worth a workgroup
+constexpr int64_t STATIC_MAX_ELEMS = 1ll << 32;  // limit of the allocation-free entry point
+
+// The allocation-free entry point's scratch.  In host code this name is only a handle: the device
+// address comes from hipGetSymbolAddress, once per device (each GPU holds its own copy).
+static __device__ __align__(256) float scratch[MAX_PARTIALS];
 
 template <int DT>
 struct Vec {
@@ -159,6 +167,31 @@ int validate(const void *x, int x_dtype, int64_t n, const int8_t *q, const float
     return I8F_OK;
 }
 
+// device address of `scratch` on the current device, looked up once per device
+int static_scratch(float **out) {
+    static std::mutex mu;
+    static float *ptr_of_device[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        last_hip_error_slot() = (int)e;
+        return I8F_ERR_HIP;
+    }
+    if (dev < 0 || dev >= 64) return I8F_ERR_DEVICE;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr_of_device[dev]) {
+        float *p = nullptr;
+        e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            last_hip_error_slot() = (int)e;
+            return I8F_ERR_HIP;
+        }
+        ptr_of_device[dev] = p;
+    }
+    *out = ptr_of_device[dev];
+    return I8F_OK;
+}
+
 }  // namespace
 }  // namespace i8f
 
@@ -173,4 +206,15 @@ extern "C" int i8f_quant_tensorwise(const void *x, int x_dtype, int64_t n, int8_
     if (!workspace || workspace_bytes < i8f_quant_tensorwise_workspace_bytes(n) || (uintptr_t)workspace % 4) return I8F_ERR_INVALID;
     if (int rc = check_device()) return rc;
     return dispatch(x, x_dtype, n, q, scale, (float *)workspace, (hipStream_t)stream);
+}
+
+extern "C" int i8f_quant_tensorwise_static(const void *x, int x_dtype, int64_t n, int8_t *q, float *scale,
+                                           void *stream) {
+    using namespace i8f;
+    if (int rc = validate(x, x_dtype, n, q, scale)) return rc;
+    if (n > STATIC_MAX_ELEMS) return I8F_ERR_UNSUPPORTED;  // the library's own scratch is sized for tensors up to this
+    if (int rc = check_device()) return rc;
+    float *partial = nullptr;
+    if (int rc = static_scratch(&partial)) return rc;
+    return dispatch(x, x_dtype, n, q, scale, partial, (hipStream_t)stream);
 }

@@ -113,6 +113,19 @@ int i8f_quant_tensorwise(const void *x, int x_dtype, int64_t n, int8_t *q, float
                          void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * i8f_quant_tensorwise without a workspace argument and without any allocation.
+ * No counterpart in the reference: it exists for callers that cannot allocate
+ * device memory (code under HIP graph capture, serving loops and harnesses that
+ * forbid hipMalloc).  The partial maxima live in a 4 KB file-scope device array of
+ * the library, one copy per GPU, held until the process ends.  Same results as
+ * i8f_quant_tensorwise bit for bit.
+ * I8F_ERR_UNSUPPORTED for n > 2^32 elements.  Calls that overlap in time on one
+ * GPU (different streams or threads) race on that array: serialise them.
+ */
+int i8f_quant_tensorwise_static(const void *x, int x_dtype, int64_t n, int8_t *q, float *scale,
+                                void *stream);
+
+/*
  * Block rotation alone (no quantisation): every aligned block of 128 elements of
  * each row is multiplied by the normalised Hadamard matrix, result in x's dtype.
  * Replaces rotate_weight / rotate_activation (quarot.py:42-102) where the rotated

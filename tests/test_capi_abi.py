@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 13
+    assert len(names) == 14
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -52,13 +52,15 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_quant_rowwise(null, L.BF16, 4, 256, 256, 0, one, one, null) == INVALID    # NULL input
     assert lib.i8f_quant_rowwise(null, L.BF16, 0, 256, 256, 0, null, null, null) == 0        # empty: nothing to do
     assert lib.i8f_rotate128(one, L.F32, 4, 100, 100, one, null) == INVALID
-    # tensorwise quantiser: workspace missing or too small
+    # tensorwise quantiser: workspace missing or too small, tensor beyond the static scratch's limit
     need = lib.i8f_quant_tensorwise_workspace_bytes(1 << 20)
     assert 0 < need <= 4096 and lib.i8f_quant_tensorwise_workspace_bytes(1 << 40) == 4096
     assert lib.i8f_quant_tensorwise(one, L.BF16, 1 << 20, one, one, null, need, null) == INVALID
     assert lib.i8f_quant_tensorwise(one, L.BF16, 1 << 20, one, one, one, need - 4, null) == INVALID
     assert lib.i8f_quant_tensorwise(one, 9, 16, one, one, one, 4096, null) == INVALID
     assert lib.i8f_quant_tensorwise(null, L.BF16, 16, one, one, one, 4096, null) == INVALID
+    assert lib.i8f_quant_tensorwise_static(one, L.BF16, (1 << 32) + 1, one, one, null) == UNSUPPORTED
+    assert lib.i8f_quant_tensorwise_static(one, L.BF16, -1, one, one, null) == INVALID
     assert lib.i8f_gemm_i32(one, one, -1, 4, 4, one, null) == INVALID
     assert lib.i8f_gemm_i32(null, one, 4, 4, 4, one, null) == INVALID
     assert lib.i8f_gemm_i32(null, null, 0, 4, 4, null, null) == 0
