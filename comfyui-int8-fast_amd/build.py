@@ -33,6 +33,7 @@ FLAGS = [
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall",
     "-Wno-unused-function",
     "-Wno-inline-asm",   # the global->LDS loads name m0 in their clobber list, which clang reports as "reserved"

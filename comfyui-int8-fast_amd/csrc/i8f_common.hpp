@@ -103,10 +103,23 @@ __device__ __forceinline__ int quant_i8(float v) {
     return (int)r;
 }
 
+// Maximum over the 64 lanes of a wave, returned to every lane.  Lane exchanges are DPP operands of
+// the max instructions (no LDS round trips: the butterfly through ds_bpermute costs six dependent
+// LDS latencies): quads, half rows and rows of 16 first, then row 0 -> 1, 2 -> 3 and rows 0..1 -> 2..3
+// by the row broadcasts, which leaves the result in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_max_step(float v) {
+    const float o = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+    return fmaxf(v, o);
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+    v = dpp_max_step<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v = dpp_max_step<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+    v = dpp_max_step<0x141, 0xf>(v);  // row_half_mirror
+    v = dpp_max_step<0x140, 0xf>(v);  // row_mirror: every lane of a row of 16 holds the row's maximum
+    v = dpp_max_step<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_max_step<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // ---- streaming stores and loads ------------------------------------------------------

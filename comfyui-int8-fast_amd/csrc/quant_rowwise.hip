@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
                                                        float *__restrict__ scale) {
     static_assert(WPR == 1 || NROW == 1, "rows are walked only by single-wave rows");
     constexpr int TPR = 64 * WPR;
-    constexpr int ROWS = 256 / TPR;
+    constexpr int ROWS = 256 / TPR;  // the workgroup has ROWS * TPR threads: 256, or 192 with three waves to a row
     const int t = threadIdx.x % TPR;
     const int rb = threadIdx.x / TPR;
     const int64_t row_stride = (int64_t)gridDim.x * ROWS;
@@ -365,7 +365,7 @@ int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
     // measured slower at every size (fewer, longer-lived waves ramp up and drain more slowly).
     constexpr int ROWS = 256 / (64 * WPR);
     const int64_t blocks = (M + ROWS - 1) / ROWS;
-    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1>), dim3((unsigned)blocks), dim3(256), 0, st, (const char *)x, M, K,
+    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1>), dim3((unsigned)blocks), dim3(ROWS * 64 * WPR), 0, st, (const char *)x, M, K,
                        ldx * 2, q, scale);
     return check_launch();
 }
