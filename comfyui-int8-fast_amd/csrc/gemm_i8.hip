@@ -182,8 +182,13 @@ __device__ __forceinline__ uint4 add_rounded(uint4 y, uint4 s) {
 }
 
 // KTAIL: K is not a multiple of BK (the last tile is ragged); the common case is the other kernel.
+// What the prologue needs (operand pointers, sizes, tile counts) comes first in the argument list: the
+// first 16 dwords of the kernel arguments are preloaded into SGPRs at wave launch, the rest (epilogue
+// operands) is fetched by scalar loads that have the whole main loop to land.
 template <class C, int OUT, bool KTAIL>
-__global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
+                                                        const float *gxs, const float *gws, const void *gbias, int flags,
+                                                        const GemmArgs g) {
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NI = C::NI, CPR = C::CPR;
     constexpr int S = C::STAGES;
     constexpr int OB = OutElem<OUT>::BYTES;
@@ -209,41 +214,21 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // ---- workgroup id -> output tile -------------------------------------------------
     int tile_m, tile_n;
     {
-        const int T = g.tiles_m * g.tiles_n;
+        const int T = tiles_m * tiles_n;
         const int bid = blockIdx.x;
         const int per = (T + 7) / 8;
         const int tall = (T % 8 == 0) ? 8 : (T % 8);
         const int xcd = bid % 8, loc = bid / 8;
         const int L = xcd < tall ? xcd * per + loc : tall * per + (xcd - tall) * (per - 1) + loc;
-        const int in_group = C::GROUP_M * g.tiles_n;
+        const int in_group = C::GROUP_M * tiles_n;
         const int grp = L / in_group;
         const int first_m = grp * C::GROUP_M;
-        const int gsz = min(g.tiles_m - first_m, C::GROUP_M);
+        const int gsz = min(tiles_m - first_m, C::GROUP_M);
         const int r = L % in_group;
         tile_m = first_m + r % gsz;
         tile_n = r / gsz;
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    // ---- epilogue operands: fetched once, long before they are needed ----------------------
-    if constexpr (OUT != OUT_I32) {
-        const float ws_one = g.ws ? (g.row_scale ? 0.0f : g.ws[0]) : g.ws_host;
-        for (int t = tid; t < BM; t += C::NT) s_xs[t] = (m0 + t < g.M) ? g.xs[m0 + t] : 0.0f;
-        for (int t = tid; t < BN; t += C::NT) {
-            const int n = n0 + t;
-            float wsv = ws_one, bv = 0.0f;
-            if (n < g.N) {
-                if (g.row_scale) wsv = g.ws[n];
-                if (g.bias) {
-                    if (g.bias_dtype == I8F_F32) bv = ((const float *)g.bias)[n];
-                    else if (g.bias_dtype == I8F_BF16) bv = bf16_bits_to_f32(((const uint16_t *)g.bias)[n]);
-                    else bv = f16_bits_to_f32(((const uint16_t *)g.bias)[n]);
-                }
-            }
-            s_ws[t] = wsv;
-            s_bias[t] = bv;
-        }
-    }
 
     // ---- global -> LDS plan ------------------------------------------------------------
     // One wave load moves 64 x 16 bytes into 1 KB of LDS (lane l lands at offset 16*l).  The lane
@@ -251,9 +236,9 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // offset of the K-tile travels in the scalar offset of the buffer instruction, so issuing a
     // load costs no vector arithmetic; rows beyond the matrix carry an out-of-range vector offset
     // and are zero-filled by the buffer bounds check (which looks at the vector offset only).
-    const int K = g.K;
-    const v4i rx = make_rsrc(g.x, (uint32_t)((int64_t)g.M * K));
-    const v4i rw = make_rsrc(g.w, (uint32_t)((int64_t)g.N * K));
+    const int K = gK;
+    const v4i rx = make_rsrc(gx, (uint32_t)((int64_t)gM * K));
+    const v4i rw = make_rsrc(gw, (uint32_t)((int64_t)gN * K));
     const uint32_t OOB = 0x7ffffff0u;
 
     uint32_t xoff[C::X_LOADS], woff[C::W_LOADS];  // byte offset of this lane's chunk at k-tile 0
@@ -264,7 +249,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         const int row = gidx / CPR, cl = gidx % CPR;
         xck[t] = (cl ^ swz<CPR>(row)) * 16;
         const int64_t grow = (int64_t)m0 + row;
-        xoff[t] = (row < BM && grow < g.M) ? (uint32_t)(grow * K + xck[t]) : OOB;
+        xoff[t] = (row < BM && grow < gM) ? (uint32_t)(grow * K + xck[t]) : OOB;
     }
 #pragma unroll
     for (int t = 0; t < C::W_LOADS; ++t) {
@@ -272,7 +257,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
         const int row = gidx / CPR, cl = gidx % CPR;
         wck[t] = (cl ^ swz<CPR>(row)) * 16;
         const int64_t grow = (int64_t)n0 + row;
-        woff[t] = (row < BN && grow < g.N) ? (uint32_t)(grow * K + wck[t]) : OOB;
+        woff[t] = (row < BN && grow < gN) ? (uint32_t)(grow * K + wck[t]) : OOB;
     }
 
     const int KT = (K + BK - 1) / BK;
@@ -354,8 +339,35 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
             issue(s, s < KT);
         }
     }
+    // ---- epilogue operands: requested behind the first tiles, parked in registers until the main loop
+    // is done.  Nothing looks at the results before the epilogue: indices are clamped instead of
+    // predicated and the conversion happens after the loop, so no instruction in between waits for
+    // them (the wait for tile 0 below counts them among the younger loads it may leave in flight, and
+    // so waits for up to three loads of tile 1 more than it has to).
+    constexpr int XS_PER = (BM + C::NT - 1) / C::NT, WS_PER = (BN + C::NT - 1) / C::NT;
+    float xs_r[XS_PER], ws_r[WS_PER];
+    uint32_t bias_r[WS_PER];
+    float ws_one = 0.0f;
+    const bool row_scale = flags & 1;
+    const int bias_dtype = flags >> 1;
+    if constexpr (OUT != OUT_I32) {
+        if (gws && !row_scale) ws_one = gws[0];
+#pragma unroll
+        for (int u = 0; u < XS_PER; ++u) xs_r[u] = gxs[min(m0 + tid + u * C::NT, gM - 1)];
+#pragma unroll
+        for (int u = 0; u < WS_PER; ++u) {
+            const int n = min(n0 + tid + u * C::NT, gN - 1);
+            ws_r[u] = row_scale ? gws[n] : 0.0f;
+            bias_r[u] = 0;
+            if (gbias) {
+                if (bias_dtype == I8F_F32) bias_r[u] = ((const uint32_t *)gbias)[n];
+                else bias_r[u] = ((const uint16_t *)gbias)[n];
+            }
+        }
+    }
+
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(SPREAD_DMA ? (PRE - 1) * C::LOADS : cut(1)));  // younger tiles may be in flight
-    __syncthreads();  // tile 0 and the staged epilogue operands are visible to everyone
+    __builtin_amdgcn_s_barrier();  // tile 0 is in LDS for everyone (no fence: nothing else has been written)
 
     // Fragments are double-buffered in registers: the LDS reads of k-step s+1 are issued before
     // the MFMAs of k-step s, so the matrix pipe does not wait for LDS.  There is one barrier per
@@ -415,7 +427,30 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     // The loads issued past the last tile move no data from memory but still zero-fill their LDS
     // destination: they must have landed before the stages are reused.
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-    __syncthreads();  // the stages are dead; reuse them as per-wave transpose buffers
+    if constexpr (OUT != OUT_I32) {
+        if (!gws) ws_one = g.ws_host;
+#pragma unroll
+        for (int u = 0; u < XS_PER; ++u) {
+            const int t = tid + u * C::NT;
+            if (t < BM) s_xs[t] = (m0 + t < gM) ? xs_r[u] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < WS_PER; ++u) {
+            const int t = tid + u * C::NT;
+            if (t < BN) {
+                const bool in = n0 + t < gN;
+                float bv = 0.0f;
+                if (gbias && in) {
+                    if (bias_dtype == I8F_F32) bv = __uint_as_float(bias_r[u]);
+                    else if (bias_dtype == I8F_BF16) bv = bf16_bits_to_f32(bias_r[u]);
+                    else bv = f16_bits_to_f32(bias_r[u]);
+                }
+                s_ws[t] = row_scale ? (in ? ws_r[u] : 0.0f) : ws_one;
+                s_bias[t] = bv;
+            }
+        }
+    }
+    __syncthreads();  // the stages are dead (reused as per-wave transpose buffers), the operands staged
     char *ebuf = smem + wave * WAVE_BYTES;
 
     // scale, bias, round: the flags are wave-uniform, so the variant is chosen once
@@ -439,7 +474,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
     using F_ = std::false_type;
     using O0 = std::integral_constant<int, I8F_EPI_TORCH>;
     using O1 = std::integral_constant<int, I8F_EPI_FUSED>;
-    const int variant = (g.order == I8F_EPI_FUSED ? 4 : 0) | (g.row_scale ? 2 : 0) | (g.bias ? 1 : 0);
+    const int variant = (g.order == I8F_EPI_FUSED ? 4 : 0) | (row_scale ? 2 : 0) | (gbias ? 1 : 0);
 
     // The whole epilogue is instantiated once per variant and the variant is chosen ONCE, so that
     // the instructions a wave executes are contiguous in memory (the epilogue runs once per wave,
@@ -514,9 +549,9 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const GemmArgs g) {
                 const uint4 val = *(const uint4 *)(ebuf + row * PITCH + cc * 16);
                 const int mm = m0 + wm * C::WTM + i0 * 32 + row;
                 const int nn = n0 + wn * C::WTN + cc * EPCO;
-                if (mm < g.M && nn < g.N)
+                if (mm < gM && nn < gN)
                 {
-                    const int64_t off = ((int64_t)mm * g.N + nn) * OB;
+                    const int64_t off = ((int64_t)mm * gN + nn) * OB;
                     uint4 v = val;
                     if (g.addend) v = add_rounded<OUT>(v, *(const uint4 *)((const char *)g.addend + off));
                     stream_store16((char *)g.out + off, v);
@@ -605,8 +640,13 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
     g.tiles_m = (g.M + C::BM - 1) / C::BM;
     g.tiles_n = (g.N + C::BN - 1) / C::BN;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    if (g.K % C::BK) hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g);
-    else hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g);
+    const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);  // what the prologue wants to know of the epilogue
+    if (g.K % C::BK)
+        hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
+                           g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
+    else
+        hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
+                           g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
     return check_launch();
 }
 
