@@ -508,6 +508,24 @@ def test_lora_merge_bit_exact(L, dev, N, K, r, row):
     assert np.array_equal(dq.cpu().numpy(), O.sr_delta(delta, ws.numpy(), noise.numpy()))
 
 
+@pytest.mark.parametrize("N,K,r", [(64, 256, 32), (96, 288, 16), (40, 100, 8)])
+def test_lora_merge_denormal_products_bit_exact(L, dev, N, K, r):
+    """Rank-r products and partial sums in the binary32 denormal range (|up*down| ~ 1e-40), with a weight
+    scale small enough that they still decide the rounded delta: the matrix-core form of the fused merge
+    (K % 32 == 0, ranks 4..32) and the vector form must both keep them as the oracle's fmaf chain does."""
+    w = i8(N, K)
+    up = torch.randn(N, r, generator=G) * 1e-20
+    down = torch.randn(r, K, generator=G) * 1e-20
+    noise = torch.rand(N, K, generator=G)
+    ws = float(np.float32(2e-40))                       # denormal scale: delta / scale is of order one
+    delta = O.lora_delta(up.numpy(), down.numpy(), 1.0)
+    assert (delta != 0).mean() > 0.9 and np.abs(delta).max() < 1.2e-38
+    want = O.lora_merge_sr(w.numpy(), np.asarray([ws], dtype=np.float32), noise.numpy(), up=up.numpy(), down=down.numpy(), lora_scale=1.0)
+    assert (want != w.numpy()).mean() > 0.2             # the denormal deltas do move the weights
+    fused = L.lora_merge_sr(w.to(dev), ws, noise.to(dev), up=up.to(dev), down=down.to(dev), lora_scale=1.0)
+    assert np.array_equal(fused.cpu().numpy(), want)
+
+
 def test_sr_special_noise_values(L, dev):
     x = torch.tensor([[0.5, 0.3, -0.3, 0.26, -0.26, 0.0, 40.0, -40.0]])
     for noise in (torch.zeros(1, 8), torch.full((1, 8), 1 - 2.0**-24), torch.tensor([[0.0, 0.2, 0.8, 0.04, 0.96, 0.5, 0.5, 0.5]])):
