@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libi8f_gfx950.so")
 BF16, F16, F32 = 0, 1, 2
 SCALE_TENSOR, SCALE_ROW = 0, 1
 EPI_TORCH, EPI_FUSED = 0, 1
+PRO_NONE, PRO_MODULATE, PRO_GELU_TANH = 0, 1, 2
 
 _DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
 
@@ -52,6 +53,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_last_hip_error.restype = i32
     L.i8f_quant_rowwise.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, vp]
     L.i8f_rotate128.argtypes = [vp, i32, i64, i64, i64, vp, vp]
+    L.i8f_quant_rowwise_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, i32, vp, vp, vp]
     L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
     L.i8f_quant_tensorwise_workspace_bytes.restype = i64
     L.i8f_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp, vp, i64, vp]
@@ -62,7 +64,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
+    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -71,7 +73,7 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
-    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static",
+    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue",
     "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
@@ -136,8 +138,11 @@ def _scale(ws, N: int, device):
 
 
 # --------------------------------------------------------------------------- entry points
-def quant_rowwise(x: torch.Tensor, rotate: bool = False):
-    """x [M,K] (bf16/fp16/fp32, cuda) -> (int8 [M,K], float32 [M,1]); rotate=True applies the 128-block Hadamard first."""
+def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NONE, mod_scale=None, mod_shift=None):
+    """x [M,K] (bf16/fp16/fp32, cuda) -> (int8 [M,K], float32 [M,1]); rotate=True applies the 128-block Hadamard first.
+    prologue applies an elementwise operation while the rows are read: PRO_GELU_TANH, or PRO_MODULATE with
+    mod_scale / mod_shift of x's dtype, [V,K] (or [K]): (1 + mod_scale) * x + mod_shift, M // V consecutive rows
+    to a vector."""
     _dev(x, "x")
     x = _rows(x, "x")
     M, K = x.shape
@@ -146,9 +151,31 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False):
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
     s = torch.empty((M, 1), dtype=torch.float32, device=x.device)
     ldx = x.stride(0) if M > 1 else K
+    rows_per_vec = 1
+    if prologue == PRO_MODULATE:
+        vecs = []
+        for name, v in (("mod_scale", mod_scale), ("mod_shift", mod_shift)):
+            _dev(v, name)
+            if v.dtype != x.dtype or v.device != x.device or v.numel() % max(K, 1) or v.shape[-1] != K:
+                raise ValueError(f"{name} must be [V,{K}] of {x.dtype} on {x.device}")
+            vecs.append(v.reshape(-1, K).contiguous())
+        mod_scale, mod_shift = vecs
+        V = mod_scale.shape[0]
+        if mod_shift.shape[0] != V or V == 0 or M % V:
+            raise ValueError(f"{M} rows do not split evenly over {V} modulation vectors")
+        rows_per_vec = max(1, M // V)
+    elif prologue not in (PRO_NONE, PRO_GELU_TANH):
+        raise ValueError(f"unknown prologue {prologue}")
+    else:
+        mod_scale = mod_shift = None
     with torch.cuda.device(x.device):
-        _check(lib().i8f_quant_rowwise(_ptr(x), dtype_code(x.dtype), M, K, ldx, 128 if rotate else 0, _ptr(q), _ptr(s),
-                                       _stream(x)), "i8f_quant_rowwise")
+        if prologue == PRO_NONE:
+            _check(lib().i8f_quant_rowwise(_ptr(x), dtype_code(x.dtype), M, K, ldx, 128 if rotate else 0, _ptr(q), _ptr(s),
+                                           _stream(x)), "i8f_quant_rowwise")
+        else:
+            _check(lib().i8f_quant_rowwise_prologue(_ptr(x), dtype_code(x.dtype), M, K, ldx, prologue, _ptr(mod_scale),
+                                                    _ptr(mod_shift), rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s),
+                                                    _stream(x)), "i8f_quant_rowwise_prologue")
     return q, s
 
 

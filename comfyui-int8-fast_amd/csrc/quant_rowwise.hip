@@ -32,6 +32,46 @@ struct Elem {
     static constexpr int LPB = 128 / EPC;                // lanes that share one 128-block
 };
 
+// ---- elementwise prologue --------------------------------------------------------------
+// What the model computes on the activations right in front of a quantised linear can be applied
+// while the row is read, which saves that operation's own pass over [M,K] (one write and one read):
+//   I8F_PRO_MODULATE   v = (1 + s[k]) * x + t[k]      adaLN modulation; s, t one vector per group of
+//                                                     rows_per_vec rows, in x's dtype.  Evaluated as
+//                                                     torch evaluates the three tensor operations in
+//                                                     x's dtype: each result rounded to that dtype.
+//   I8F_PRO_GELU_TANH  v = gelu(x), tanh form         0.5 x (1 + tanh(b (x + 0.044715 x^3))), b = sqrt(2/pi),
+//                                                     evaluated in binary32 and rounded once to x's dtype,
+//                                                     tanh(u) = 1 - 2 / (exp(2u) + 1) on the hardware's
+//                                                     exp2 and reciprocal (a few binary32 ulp).
+struct Prologue {
+    int kind;
+    const void *s, *t;       // modulation vectors (MODULATE)
+    int64_t rows_per_vec;    // rows that share one pair of vectors
+};
+
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+    const float kBeta = 0.7978845608028654f, kKappa = 0.044715f;
+    const float x3 = x * x * x;
+    const float inner = kBeta * (x + kKappa * x3);
+    // exp(2 inner) = exp2(2 log2(e) inner); an overflow to +inf gives tanh = 1, an underflow to 0 gives -1
+    const float e = __builtin_amdgcn_exp2f(inner * 2.885390081777927f);
+    const float th = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+    return 0.5f * x * (1.0f + th);
+}
+
+template <int DT, int PRO>
+__device__ __forceinline__ float apply_prologue(float x, float s, float t) {
+    if constexpr (PRO == I8F_PRO_MODULATE) {
+        const float a = round_to_dtype<DT>(1.0f + s);
+        const float b = round_to_dtype<DT>(a * x);
+        return round_to_dtype<DT>(b + t);
+    } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
+        return round_to_dtype<DT>(gelu_tanh_f32(x));
+    } else {
+        return x;
+    }
+}
+
 template <int DT>
 __device__ __forceinline__ void load_chunk(const void *p, float (&v)[Elem<DT>::EPC]) {
     const uint4 u = *(const uint4 *)p;
@@ -278,10 +318,10 @@ __device__ __forceinline__ uint32_t quant4_magic(float a, float b, float c, floa
 // fetches the next row while it reduces, scales and stores the current one: loads and stores of
 // different rows overlap inside a wave instead of every wave of the grid moving from a read phase
 // to a write phase in step.
-template <int DT, bool ROT, int WPR, int RUNS, int NROW>
+template <int DT, bool ROT, int WPR, int RUNS, int NROW, int PRO = I8F_PRO_NONE>
 __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x, int64_t M, int64_t K,
                                                        int64_t ldx_bytes, int8_t *__restrict__ q,
-                                                       float *__restrict__ scale) {
+                                                       float *__restrict__ scale, const Prologue pro) {
     static_assert(WPR == 1 || NROW == 1, "rows are walked only by single-wave rows");
     constexpr int TPR = 64 * WPR;
     constexpr int ROWS = 256 / TPR;  // the workgroup has ROWS * TPR threads: 256, or 192 with three waves to a row
@@ -322,6 +362,20 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
             expand16<DT>(raw[it & 1][r][0], raw[it & 1][r][1], v[r]);
+            if constexpr (PRO == I8F_PRO_MODULATE) {
+                // the vectors of this row's group, same 16 columns (they come from cache: every row of the group reads them)
+                const int R = r * TPR + p;
+                const int64_t vrow = (m < M ? m : 0) / pro.rows_per_vec;
+                const int64_t off = (vrow * K + (R < nruns ? R : 0) * 16) * 2;
+                float sv[16], tv[16];
+                expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), sv);
+                expand16<DT>(*(const uint4 *)((const char *)pro.t + off), *(const uint4 *)((const char *)pro.t + off + 16), tv);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v[r][j] = R < nruns ? apply_prologue<DT, PRO>(v[r][j], sv[j], tv[j]) : 0.0f;
+            } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v[r][j] = apply_prologue<DT, PRO>(v[r][j], 0.0f, 0.0f);
+            }
             if constexpr (ROT) rotate_run16<DT>(v[r], s0, s1, s2);
 #pragma unroll
             for (int j = 0; j < 16; j += 2) amax = max3_abs(amax, v[r][j], v[r][j + 1]);
@@ -359,24 +413,24 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
     }
 }
 
-template <int DT, bool ROT, int WPR, int RUNS>
-int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st) {
+template <int DT, bool ROT, int WPR, int RUNS, int PRO = I8F_PRO_NONE>
+int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st, const Prologue &pro = Prologue{}) {
     // One row per wave (NROW = 1): walking several rows per wave with the next row's loads in flight
     // measured slower at every size (fewer, longer-lived waves ramp up and drain more slowly).
     constexpr int ROWS = 256 / (64 * WPR);
     const int64_t blocks = (M + ROWS - 1) / ROWS;
-    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1>), dim3((unsigned)blocks), dim3(ROWS * 64 * WPR), 0, st, (const char *)x, M, K,
-                       ldx * 2, q, scale);
+    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1, PRO>), dim3((unsigned)blocks), dim3(ROWS * 64 * WPR), 0, st, (const char *)x, M, K,
+                       ldx * 2, q, scale, pro);
     return check_launch();
 }
 
-template <int DT, bool ROT, int WPR>
-int pick_runs16(int runs, const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st) {
+template <int DT, bool ROT, int WPR, int PRO = I8F_PRO_NONE>
+int pick_runs16(int runs, const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st, const Prologue &pro = Prologue{}) {
     switch (runs) {
-    case 1: return launch16<DT, ROT, WPR, 1>(x, M, K, ldx, q, scale, st);
-    case 2: return launch16<DT, ROT, WPR, 2>(x, M, K, ldx, q, scale, st);
-    case 3: return launch16<DT, ROT, WPR, 3>(x, M, K, ldx, q, scale, st);
-    default: return launch16<DT, ROT, WPR, 4>(x, M, K, ldx, q, scale, st);
+    case 1: return launch16<DT, ROT, WPR, 1, PRO>(x, M, K, ldx, q, scale, st, pro);
+    case 2: return launch16<DT, ROT, WPR, 2, PRO>(x, M, K, ldx, q, scale, st, pro);
+    case 3: return launch16<DT, ROT, WPR, 3, PRO>(x, M, K, ldx, q, scale, st, pro);
+    default: return launch16<DT, ROT, WPR, 4, PRO>(x, M, K, ldx, q, scale, st, pro);
     }
 }
 
@@ -401,28 +455,35 @@ __device__ __forceinline__ void rotate128_wave(float &e0, float &e1, int lane) {
     e1 = round_to_dtype<DT>(e1 * h);
 }
 
-template <int DT, bool ROT>
+template <int DT, bool ROT, int PRO = I8F_PRO_NONE>
 __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__restrict__ x, int64_t M,
                                                                   int64_t K, int64_t ldx,
                                                                   int8_t *__restrict__ q,
-                                                                  float *__restrict__ scale) {
+                                                                  float *__restrict__ scale, const Prologue pro) {
     const int64_t m = blockIdx.x;
     if (m >= M) return;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
     const int64_t base = m * ldx;
     __shared__ float red[4];
+    // element k of this row after the prologue
+    const int64_t vbase = PRO == I8F_PRO_MODULATE ? (m / pro.rows_per_vec) * K : 0;
+    auto element = [&](int64_t k) {
+        const float xv = load_as_f32<DT>(x, base + k);
+        if constexpr (PRO == I8F_PRO_MODULATE) return apply_prologue<DT, PRO>(xv, load_as_f32<DT>(pro.s, vbase + k), load_as_f32<DT>(pro.t, vbase + k));
+        else return apply_prologue<DT, PRO>(xv, 0.0f, 0.0f);
+    };
 
     float amax = 0.0f;
     if constexpr (ROT) {
         for (int64_t blk = wv; blk < K / 128; blk += 4) {
-            float e0 = load_as_f32<DT>(x, base + blk * 128 + lane);
-            float e1 = load_as_f32<DT>(x, base + blk * 128 + 64 + lane);
+            float e0 = element(blk * 128 + lane);
+            float e1 = element(blk * 128 + 64 + lane);
             rotate128_wave<DT>(e0, e1, lane);
             amax = fmaxf(amax, fmaxf(fabsf(e0), fabsf(e1)));
         }
     } else {
-        for (int64_t k = tid; k < K; k += 256) amax = fmaxf(amax, fabsf(load_as_f32<DT>(x, base + k)));
+        for (int64_t k = tid; k < K; k += 256) amax = fmaxf(amax, fabsf(element(k)));
     }
     amax = wave_max(amax);
     if (lane == 0) red[wv] = amax;
@@ -435,15 +496,14 @@ __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__r
     int8_t *qrow = q + m * K;
     if constexpr (ROT) {
         for (int64_t blk = wv; blk < K / 128; blk += 4) {
-            float e0 = load_as_f32<DT>(x, base + blk * 128 + lane);
-            float e1 = load_as_f32<DT>(x, base + blk * 128 + 64 + lane);
+            float e0 = element(blk * 128 + lane);
+            float e1 = element(blk * 128 + 64 + lane);
             rotate128_wave<DT>(e0, e1, lane);
             qrow[blk * 128 + lane] = (int8_t)quant_i8(e0 * inv);
             qrow[blk * 128 + 64 + lane] = (int8_t)quant_i8(e1 * inv);
         }
     } else {
-        for (int64_t k = tid; k < K; k += 256)
-            qrow[k] = (int8_t)quant_i8(load_as_f32<DT>(x, base + k) * inv);
+        for (int64_t k = tid; k < K; k += 256) qrow[k] = (int8_t)quant_i8(element(k) * inv);
     }
     if (tid == 0) scale[m] = s;
 }
@@ -538,34 +598,44 @@ int pick_nch(int per_thread, const void *x, int64_t M, int64_t K, int64_t ldx, i
     return launch_fast<DT, ROT, TPR, 8>(x, M, K, ldx, q, scale, st);
 }
 
-template <int DT, bool ROT>
-int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st) {
+template <int DT, bool ROT, int PRO = I8F_PRO_NONE>
+int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st, const Prologue &pro = Prologue{}) {
     constexpr int EPC = Elem<DT>::EPC;
     const size_t es = dtype_size(DT);
-    const bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) &&
-                         ((uintptr_t)q % 8 == 0);
+    bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) && ((uintptr_t)q % 8 == 0);
+    if constexpr (PRO == I8F_PRO_MODULATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0 && (uintptr_t)pro.t % 16 == 0;
     const int64_t nchunks = K / EPC;
     if constexpr (DT != I8F_F32) {
         const int64_t nruns = K / 16;
         if (aligned && K % 16 == 0 && (uintptr_t)q % 16 == 0 && nruns >= 1 && nruns <= 64 * 4 * 4) {
-            if (nruns <= 64 * 4) return pick_runs16<DT, ROT, 1>((int)((nruns + 63) / 64), x, M, K, ldx, q, scale, st);
-            return pick_runs16<DT, ROT, 4>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st);
+            if (nruns <= 64 * 4) return pick_runs16<DT, ROT, 1, PRO>((int)((nruns + 63) / 64), x, M, K, ldx, q, scale, st, pro);
+            return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
         }
     }
-    if (aligned && nchunks <= 1024 * 8) {
-        if (nchunks <= 64 * 8) return pick_nch<DT, ROT, 64>((int)((nchunks + 63) / 64), x, M, K, ldx, q, scale, st);
-        if (nchunks <= 256 * 8) return pick_nch<DT, ROT, 256>((int)((nchunks + 255) / 256), x, M, K, ldx, q, scale, st);
-        return pick_nch<DT, ROT, 1024>((int)((nchunks + 1023) / 1024), x, M, K, ldx, q, scale, st);
+    if constexpr (PRO == I8F_PRO_NONE) {  // the chunked kernels have no prologue form: such shapes take the generic kernel
+        if (aligned && nchunks <= 1024 * 8) {
+            if (nchunks <= 64 * 8) return pick_nch<DT, ROT, 64>((int)((nchunks + 63) / 64), x, M, K, ldx, q, scale, st);
+            if (nchunks <= 256 * 8) return pick_nch<DT, ROT, 256>((int)((nchunks + 255) / 256), x, M, K, ldx, q, scale, st);
+            return pick_nch<DT, ROT, 1024>((int)((nchunks + 1023) / 1024), x, M, K, ldx, q, scale, st);
+        }
     }
-    hipLaunchKernelGGL((quant_rows_generic_kernel<DT, ROT>), dim3((unsigned)M), dim3(256), 0, st, x, M, K, ldx,
-                       q, scale);
+    hipLaunchKernelGGL((quant_rows_generic_kernel<DT, ROT, PRO>), dim3((unsigned)M), dim3(256), 0, st, x, M, K, ldx,
+                       q, scale, pro);
     return check_launch();
 }
 
 template <int DT>
 int dispatch_rot(bool rot, const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale,
-                 hipStream_t st) {
-    return rot ? dispatch<DT, true>(x, M, K, ldx, q, scale, st) : dispatch<DT, false>(x, M, K, ldx, q, scale, st);
+                 hipStream_t st, const Prologue &pro = Prologue{}) {
+    switch (pro.kind) {
+    case I8F_PRO_MODULATE:
+        return rot ? dispatch<DT, true, I8F_PRO_MODULATE>(x, M, K, ldx, q, scale, st, pro)
+                   : dispatch<DT, false, I8F_PRO_MODULATE>(x, M, K, ldx, q, scale, st, pro);
+    case I8F_PRO_GELU_TANH:
+        return rot ? dispatch<DT, true, I8F_PRO_GELU_TANH>(x, M, K, ldx, q, scale, st, pro)
+                   : dispatch<DT, false, I8F_PRO_GELU_TANH>(x, M, K, ldx, q, scale, st, pro);
+    default: return rot ? dispatch<DT, true>(x, M, K, ldx, q, scale, st) : dispatch<DT, false>(x, M, K, ldx, q, scale, st);
+    }
 }
 
 }  // namespace
@@ -588,6 +658,31 @@ extern "C" int i8f_quant_rowwise(const void *x, int x_dtype, int64_t M, int64_t 
     case I8F_BF16: return dispatch_rot<I8F_BF16>(rot, x, M, K, ldx, q, scale, st);
     case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st);
     default: return dispatch_rot<I8F_F32>(rot, x, M, K, ldx, q, scale, st);
+    }
+}
+
+extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, int prologue,
+                                          const void *mod_scale, const void *mod_shift, int64_t rows_per_vec,
+                                          int rotate_block, int8_t *q, float *scale, void *stream) {
+    using namespace i8f;
+    if (prologue == I8F_PRO_NONE) return i8f_quant_rowwise(x, x_dtype, M, K, ldx, rotate_block, q, scale, stream);
+    if (prologue != I8F_PRO_MODULATE && prologue != I8F_PRO_GELU_TANH) return I8F_ERR_INVALID;
+    if (M < 0 || K < 0 || !valid_dtype(x_dtype)) return I8F_ERR_INVALID;
+    if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
+    if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
+    if (M == 0) return I8F_OK;
+    if (!scale || ldx < K) return I8F_ERR_INVALID;
+    if (K > 0 && (!x || !q)) return I8F_ERR_INVALID;
+    if (prologue == I8F_PRO_MODULATE && (rows_per_vec <= 0 || (K > 0 && (!mod_scale || !mod_shift)))) return I8F_ERR_INVALID;
+    if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
+    if (int rc = check_device()) return rc;
+    Prologue pro{prologue, mod_scale, mod_shift, rows_per_vec > 0 ? rows_per_vec : 1};
+    hipStream_t st = (hipStream_t)stream;
+    const bool rot = rotate_block != 0;
+    switch (x_dtype) {
+    case I8F_BF16: return dispatch_rot<I8F_BF16>(rot, x, M, K, ldx, q, scale, st, pro);
+    case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st, pro);
+    default: return dispatch_rot<I8F_F32>(rot, x, M, K, ldx, q, scale, st, pro);
     }
 }
 

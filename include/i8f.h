@@ -68,6 +68,17 @@ typedef enum i8f_scale_mode { I8F_SCALE_TENSOR = 0, I8F_SCALE_ROW = 1 } i8f_scal
  */
 typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
 
+/*
+ * Elementwise operation applied to the activations while the quantiser reads them
+ * (i8f_quant_rowwise_prologue).
+ *   I8F_PRO_NONE       none
+ *   I8F_PRO_MODULATE   (1 + s[k]) * x + t[k], the adaLN modulation in front of a DiT
+ *                      block's qkv and MLP projections; the three tensor operations
+ *                      are each rounded to x's dtype, as torch's eager kernels do
+ *   I8F_PRO_GELU_TANH  gelu(x, approximate="tanh") in binary32, rounded once to x's dtype
+ */
+typedef enum i8f_prologue { I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2 } i8f_prologue;
+
 /* Library version (I8F_VERSION of the build). */
 int i8f_version(void);
 
@@ -94,6 +105,25 @@ int i8f_last_hip_error(void);
  */
 int i8f_quant_rowwise(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                       int rotate_block, int8_t *q, float *scale, void *stream);
+
+/*
+ * i8f_quant_rowwise with the elementwise operation in front of the linear layer
+ * applied on the fly.  The reference gets this fusion from torch.compile, which
+ * fuses the producer of the activations into its traceable Triton quantiser
+ * (README.md:4,56; int8_fused_kernel.py:10-53); here it is an explicit variant of
+ * the quantiser, so the modulated / activated tensor is never written to memory.
+ *   prologue      i8f_prologue
+ *   mod_scale, mod_shift   I8F_PRO_MODULATE: [ceil(M / rows_per_vec), K] of x_dtype,
+ *                 contiguous; row m uses vector m / rows_per_vec (one pair of vectors
+ *                 per image of a batch); ignored otherwise
+ * I8F_PRO_MODULATE is bit-identical to torch's three eager operations followed by
+ * i8f_quant_rowwise; I8F_PRO_GELU_TANH agrees with torch's gelu to the last bits of
+ * binary32 before the rounding to x_dtype (tests state the tolerance).
+ */
+int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                               int prologue, const void *mod_scale, const void *mod_shift,
+                               int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale,
+                               void *stream);
 
 /*
  * One absmax scale for a whole tensor, then int8 quantisation with it.

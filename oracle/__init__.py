@@ -44,6 +44,7 @@ def lib() -> ctypes.CDLL:
         vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
         L.orc_quant_rowwise.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp]
         L.orc_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp]
+        L.orc_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, vp]
         L.orc_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp]
         L.orc_epilogue.argtypes = [vp, vp, vp, i32, vp, i32, vp, i32, i64, i64, i32]
         L.orc_linear_w8a8.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i32, vp, i32, vp, i32, i64, i32]
@@ -159,6 +160,23 @@ def quant_tensorwise(x, dtype_code):
     s = np.empty((1,), dtype=np.float32)
     _chk(lib().orc_quant_tensorwise(_p(x), dtype_code, x.size, _p(q), _p(s)), "quant_tensorwise")
     return q, s
+
+
+PRO_MODULATE, PRO_GELU_TANH = 1, 2
+
+
+def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
+    """The elementwise operation in front of a quantised linear (adaLN modulation or tanh-GELU), evaluated as
+    torch's eager kernels do; returns the storage array of dtype_code, shape of x."""
+    x = _arr(x, dtype_code)
+    M, K = x.shape
+    if kind == PRO_MODULATE:
+        s, t = _arr(s, dtype_code).reshape(-1, K), _arr(t, dtype_code).reshape(-1, K)
+        assert s.shape == t.shape and s.shape[0] * rows_per_vec >= M
+    out = np.empty((M, K), dtype=x.dtype)
+    _chk(lib().orc_prologue(_p(x), dtype_code, M, K, K, kind, _p(s) if s is not None else None,
+                            _p(t) if t is not None else None, rows_per_vec, _p(out)), "prologue")
+    return out
 
 
 def rotate(x, dtype_code, block=128):

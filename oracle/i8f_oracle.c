@@ -245,6 +245,46 @@ int orc_quant_rowwise(const void *x, int dtype, int64_t M, int64_t K, int64_t ld
 }
 
 /*
+ * The elementwise operation a model applies in front of a quantised linear, which
+ * the reference's torch.compile path fuses into its quantiser (README.md:4,56;
+ * the Triton quantiser int8_fused_kernel.py:10-53 is traceable).  Restated as
+ * torch's eager kernels evaluate it on a tensor of `dtype`:
+ *   kind 1  (1 + s[k]) * x + t[k]: three tensor operations, each computed in
+ *           binary32 and rounded to dtype; s, t are [ceil(M / rows_per_vec), K],
+ *           row m uses vector m / rows_per_vec
+ *   kind 2  gelu(x, approximate="tanh") = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+ *           in binary32, rounded once to dtype (the tanh is the C library's: a
+ *           tolerance reference in the last binary32 bits, not a bit pattern)
+ * out is [M,K] of dtype, contiguous.  Followed by orc_quant_rowwise it is the
+ * oracle of the fused quantiser.
+ */
+int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, int kind,
+                 const void *s, const void *t, int64_t rows_per_vec, void *out) {
+    if (M < 0 || K < 0 || ldx < K || (kind != 1 && kind != 2)) return -1;
+    if (kind == 1 && (rows_per_vec <= 0 || !s || !t)) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        for (int64_t k = 0; k < K; ++k) {
+            const float xv = load_as_f32(x, dtype, (size_t)(m * ldx + k));
+            float v;
+            if (kind == 1) {
+                const size_t vi = (size_t)((m / rows_per_vec) * K + k);
+                const float a = round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype);
+                const float b = round_to_dtype(a * xv, dtype);
+                v = b + load_as_f32(t, dtype, vi);
+            } else {
+                const float kBeta = 0.7978845608028654f, kKappa = 0.044715f;
+                const float x3 = xv * xv * xv;
+                const float inner = kBeta * (xv + kKappa * x3);
+                v = 0.5f * xv * (1.0f + tanhf(inner));
+            }
+            store_from_f32(out, dtype, (size_t)(m * K + k), v);
+        }
+    }
+    return 0;
+}
+
+/*
  * quantize_int8_tensorwise (int8_quant.py:23-26): one scale for the whole
  * tensor.  Used to prepare the tensorwise weights of BASELINE config 0.
  */

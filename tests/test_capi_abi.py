@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 14
+    assert len(names) == 15
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -52,6 +52,12 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_quant_rowwise(null, L.BF16, 4, 256, 256, 0, one, one, null) == INVALID    # NULL input
     assert lib.i8f_quant_rowwise(null, L.BF16, 0, 256, 256, 0, null, null, null) == 0        # empty: nothing to do
     assert lib.i8f_rotate128(one, L.F32, 4, 100, 100, one, null) == INVALID
+    # quantiser with a prologue: unknown operation, modulation without its vectors or with a bad group size
+    assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, 7, null, null, 1, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, L.PRO_MODULATE, null, one, 4, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, L.PRO_MODULATE, one, one, 0, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 200, 200, L.PRO_GELU_TANH, null, null, 1, 128, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_prologue(null, L.BF16, 0, 256, 256, L.PRO_GELU_TANH, null, null, 1, 0, null, null, null) == 0
     # tensorwise quantiser: workspace missing or too small, tensor beyond the static scratch's limit
     need = lib.i8f_quant_tensorwise_workspace_bytes(1 << 20)
     assert 0 < need <= 4096 and lib.i8f_quant_tensorwise_workspace_bytes(1 << 40) == 4096

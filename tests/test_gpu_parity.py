@@ -61,6 +61,49 @@ def test_quant_rowwise_bit_exact(L, dev, M, K, dt, rot):
     assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
 
 
+PROLOGUE_CASES = [
+    # M, K, dtype, rotate, vectors
+    (64, 3072, torch.bfloat16, False, 1), (48, 3072, torch.bfloat16, True, 2), (12, 12288, torch.bfloat16, False, 3),
+    (10, 1000, torch.bfloat16, False, 2), (6, 384, torch.float16, True, 1), (5, 77, torch.float32, False, 1), (8, 256, torch.float32, True, 4),
+]
+
+
+@pytest.mark.parametrize("M,K,dt,rot,V", PROLOGUE_CASES)
+def test_quant_rowwise_modulate_prologue_bit_exact(L, dev, M, K, dt, rot, V):
+    """adaLN modulation applied inside the quantiser == torch's three eager operations, then the quantiser."""
+    x = acts(M, K, dt)
+    sc, sh = (torch.randn(V, K, generator=G) * 0.3).to(dt), torch.randn(V, K, generator=G).to(dt)
+    xa, code = O.from_torch(x)
+    mod = O.prologue(xa, code, O.PRO_MODULATE, O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=M // V)
+    qo, so = O.quant_rowwise(mod, code, 128 if rot else 0)
+    q, s = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_MODULATE, mod_scale=sc.to(dev), mod_shift=sh.to(dev))
+    assert np.array_equal(q.cpu().numpy(), qo)
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+    # and against torch on the device followed by the plain quantiser
+    xd = x.to(dev)
+    t = ((1 + sc.to(dev)[:, None, :]) * xd.view(V, M // V, K) + sh.to(dev)[:, None, :]).reshape(M, K)
+    q2, s2 = L.quant_rowwise(t, rotate=rot)
+    assert torch.equal(q, q2) and torch.equal(s, s2)
+
+
+@pytest.mark.parametrize("M,K,dt,rot,V", PROLOGUE_CASES)
+def test_quant_rowwise_gelu_prologue_within_tolerance(L, dev, M, K, dt, rot, V):
+    """tanh-GELU inside the quantiser against the oracle (C tanhf) and against torch's gelu on the device followed
+    by the plain quantiser.  The activations agree to the last bits of binary32 before they are rounded to the
+    dtype, so: scales equal or one ulp of the dtype apart, int8 values at most 1 apart, at least 99.9 % equal
+    (un-rotated; a rotation spreads a one-ulp difference over its 128-block: 99 %)."""
+    x = (acts(M, K, dt).float() * 0.5).to(dt)
+    xa, code = O.from_torch(x)
+    qo, so = O.quant_rowwise(O.prologue(xa, code, O.PRO_GELU_TANH), code, 128 if rot else 0)
+    q, s = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_GELU_TANH)
+    q2, s2 = L.quant_rowwise(torch.nn.functional.gelu(x.to(dev), approximate="tanh"), rotate=rot)
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-22}[dt]
+    for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+        d = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() <= (1e-2 if rot else 1e-3)
+        assert (np.abs(s.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
+
+
 TENSORWISE_CASES = [
     # shape, dtype
     ((3072, 3072), torch.bfloat16), ((3072, 3072), torch.float32), ((1, 1), torch.float32), ((7,), torch.float16),

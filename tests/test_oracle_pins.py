@@ -398,3 +398,35 @@ def test_lora_merge_composes_the_three_steps():
     assert np.array_equal(O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), delta=delta), want)
     assert np.array_equal(O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), up=up.numpy(), down=down.numpy(), lora_scale=0.5), want)
     assert (want != w.numpy()).mean() > 0.5
+
+
+# ------------------------------------------------------------------ prologue in front of the quantiser
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+def test_prologue_modulate_equals_torch_eager_ops(dt):
+    """(1 + s) * x + t as three torch tensor operations in the tensor's dtype, bit for bit; two images of a
+    batch with their own vectors."""
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(2 * 6, 200, generator=g).to(dt)
+    sc, sh = (torch.randn(2, 200, generator=g) * 0.3).to(dt), torch.randn(2, 200, generator=g).to(dt)
+    want = ((1 + sc[:, None, :]) * x.view(2, 6, 200) + sh[:, None, :]).reshape(12, 200)
+    xa, code = O.from_torch(x)
+    got = O.prologue(xa, code, O.PRO_MODULATE, O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=6)
+    assert np.array_equal(got, O.from_torch(want)[0])
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+def test_prologue_gelu_tanh_agrees_with_torch(dt):
+    """torch's gelu(approximate="tanh") uses its own vectorised tanh: equal up to the last bits of binary32,
+    i.e. at most one unit in the last place of the storage dtype, and that only rarely."""
+    g = torch.Generator().manual_seed(32)
+    x = (torch.randn(64, 512, generator=g) * 3).to(dt)
+    x[0, :8] = torch.tensor([0.0, -0.0, 1e-6, -1e-6, 20.0, -20.0, 100.0, -100.0]).to(dt)
+    want = torch.nn.functional.gelu(x, approximate="tanh")
+    xa, code = O.from_torch(x)
+    got = O.to_f32(O.prologue(xa, code, O.PRO_GELU_TANH), code)
+    w = want.float().numpy()
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-22}[dt]
+    # far in the negative tail 1 + tanh cancels to the last bit of binary32: an absolute 2^-23 |x| on top
+    assert (np.abs(got - w) <= ulp * np.abs(w) + 2.0**-23 * np.abs(x.float().numpy())).all()
+    assert (got != w).mean() < (1e-2 if dt != torch.float32 else 0.5)
+    assert got[0, 4] == 20.0 and got[0, 5] == 0.0 and got[0, 0] == 0.0
