@@ -10,12 +10,22 @@ the namespace `i8f` with a shape-only ("fake") implementation:
     torch.ops.i8f.int8_linear           <- triton_int8_linear[_per_row]         (int8_fused_kernel.py:179-235, 330-372)
     torch.ops.i8f.linear_w8a16_small_m  <- the M <= 16 branch of Linear.forward (int8_quant.py:756-760)
     torch.ops.i8f.rotate128             <- rotate_activation                    (quarot.py:73-102)
+    torch.ops.i8f.int8_linear_prologue  <- int8_linear with the elementwise operation in front of the layer
+                                           (adaLN modulation, tanh-GELU) applied inside the quantiser: what
+                                           torch.compile's fusion into the Triton quantiser gives the reference
 
 `Int8TensorwiseOps.Linear.forward` switches to these operators while a graph is being traced
 (`torch.compiler.is_compiling()`); in eager mode it calls the library directly, which saves the
 dispatcher overhead per layer.  A weight scale is passed either as a tensor or, for the
 single-scale layout, as a float beside a `None` tensor.
+
+`fuse_prologues(graph_module)` rewrites a traced graph so that `gelu(x, approximate="tanh")` and
+`(1 + scale) * x + shift` feeding an `int8_linear` become its prologue, and `backend(inner)` is a
+torch.compile backend that applies the rewrite and hands the graph to `inner` ("inductor" by default):
+
+    model = torch.compile(model, backend=compile_ops.backend())
 """
+import operator
 from typing import Optional, Tuple
 
 import torch
@@ -96,7 +106,139 @@ def _(x, weight, weight_scale, weight_scale_value, bias, rotate):
     return x.new_empty((*x.shape[:-1], weight.shape[0]))
 
 
-OPS = ("quantize_rowwise", "rotate128", "linear_w8a8", "int8_linear", "linear_w8a16_small_m")
+@torch.library.custom_op(f"{NAMESPACE}::int8_linear_prologue", mutates_args=())
+def int8_linear_prologue(x: Tensor, prologue: int, mod_scale: Optional[Tensor], mod_shift: Optional[Tensor],
+                         weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
+                         bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int) -> Tensor:
+    """int8_linear on prologue(x): tanh-GELU, or (1 + mod_scale) * x + mod_shift with one pair of vectors per
+    group of consecutive rows; the transformed activations exist only inside the quantiser."""
+    lead = x.shape[:-1]
+    q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
+                              mod_shift=mod_shift)
+    y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order)
+    return y.reshape(*lead, weight.shape[0])
+
+
+@int8_linear_prologue.register_fake
+def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order):
+    return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
+
+
+OPS = ("quantize_rowwise", "rotate128", "linear_w8a8", "int8_linear", "linear_w8a16_small_m", "int8_linear_prologue")
+
+
+# --------------------------------------------------------------------------- graph rewrite
+_VIEW_METHODS = ("reshape", "view", "contiguous", "flatten")
+
+
+def _is_call(node, *targets):
+    return node.op == "call_function" and node.target in targets
+
+
+def _through_views(node):
+    """The producer of `node` behind shape-only steps that have no other user."""
+    while isinstance(node, torch.fx.Node) and len(node.users) == 1 and (
+            (node.op == "call_method" and node.target in _VIEW_METHODS)
+            or _is_call(node, torch.reshape, torch.flatten)):
+        node = node.args[0]
+    return node
+
+
+def _match_gelu(node):
+    if not (_is_call(node, torch.nn.functional.gelu, torch._C._nn.gelu) and len(node.users) == 1):
+        return None
+    approx = node.kwargs.get("approximate", node.args[1] if len(node.args) > 1 else "none")
+    return node.args[0] if approx == "tanh" else None
+
+
+def _match_modulate(node):
+    """(1 + scale) * x + shift in any operand order -> (x, scale, shift) nodes."""
+    if not (_is_call(node, operator.add, torch.add) and len(node.users) == 1 and len(node.args) == 2):
+        return None
+    for prod, shift in (node.args, node.args[::-1]):
+        if not (isinstance(prod, torch.fx.Node) and _is_call(prod, operator.mul, torch.mul) and len(prod.users) == 1):
+            continue
+        for gain, x in (prod.args, prod.args[::-1]):
+            if isinstance(gain, torch.fx.Node) and _is_call(gain, operator.add, torch.add) and len(gain.users) == 1 and len(gain.args) == 2:
+                for one, scale in (gain.args, gain.args[::-1]):
+                    if isinstance(one, (int, float)) and one == 1 and isinstance(scale, torch.fx.Node) \
+                            and isinstance(x, torch.fx.Node) and isinstance(shift, torch.fx.Node):
+                        return x, scale, shift
+    return None
+
+
+def _vectors_broadcast_over_tokens(x, scale, shift) -> bool:
+    """True if the traced shapes say scale/shift are [.., 1, K] (or [K]) against x [.., T, K]: one vector per
+    leading index, shared by the T rows that become consecutive rows of the flattened activations."""
+    def shape(n):
+        v = n.meta.get("example_value", n.meta.get("val"))
+        return None if v is None else tuple(v.shape)
+    xs, ss, ts = shape(x), shape(scale), shape(shift)
+    if xs is None or ss is None or ts is None or ss != ts or len(xs) < 2:
+        return False
+    if len(ss) == 1:
+        return ss[0] == xs[-1]
+    return len(ss) == len(xs) and ss[-1] == xs[-1] and ss[-2] == 1 and ss[:-2] == xs[:-2]
+
+
+def fuse_prologues(gm: torch.fx.GraphModule) -> int:
+    """Rewrite int8_linear(gelu_tanh(h)) and int8_linear((1 + s) * h + t) (no dynamic-LoRA addend, producer used
+    nowhere else) into int8_linear_prologue(h, ...).  Returns the number of layers rewritten."""
+    n_fused = 0
+    targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
+    for node in list(gm.graph.nodes):
+        if not _is_call(node, *targets):
+            continue
+        args = list(node.args) + [node.kwargs.get("addend")] * (9 - len(node.args))
+        x_in, weight, ws_t, ws_v, bias, cdt, rotate, order, addend = args[:9]
+        if addend is not None or not isinstance(x_in, torch.fx.Node):
+            continue
+        src = _through_views(x_in)
+        if not isinstance(src, torch.fx.Node):
+            continue
+        h = _match_gelu(src)
+        new_args = None
+        if h is not None:
+            new_args = (h, _lib.PRO_GELU_TANH, None, None)
+        else:
+            m = _match_modulate(src)
+            if m is not None and _vectors_broadcast_over_tokens(*m):
+                new_args = (m[0], _lib.PRO_MODULATE, m[1], m[2])
+        if new_args is None:
+            continue
+        with gm.graph.inserting_before(node):
+            fused = gm.graph.call_function(torch.ops.i8f.int8_linear_prologue,
+                                           (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order))
+            # the layer flattened its input to 2-D and restores the leading shape itself: so does the operator
+            restored = gm.graph.call_method("reshape", (fused, -1, _out_features(weight)))
+        node.replace_all_uses_with(restored)
+        gm.graph.erase_node(node)
+        n_fused += 1
+    if n_fused:
+        gm.graph.eliminate_dead_code()
+        gm.graph.lint()
+        gm.recompile()
+    return n_fused
+
+
+def _out_features(weight_node):
+    v = weight_node.meta.get("example_value", weight_node.meta.get("val"))
+    if v is None:
+        raise RuntimeError("the traced graph carries no shape for the weight")
+    return int(v.shape[0])
+
+
+def backend(inner="inductor"):
+    """A torch.compile backend: fuse_prologues, then `inner` (a registered backend name or a callable)."""
+    def compile_fn(gm, example_inputs):
+        fuse_prologues(gm)
+        fn = inner
+        if isinstance(inner, str):
+            from torch._dynamo.backends.registry import lookup_backend
+
+            fn = lookup_backend(inner)
+        return fn(gm, example_inputs)
+    return compile_fn
 
 
 def split_scale(weight_scale):

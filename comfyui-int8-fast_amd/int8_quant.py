@@ -79,16 +79,18 @@ def stochastic_round_int8_delta(x: Tensor, scale, seed: int = 0, noise: Tensor |
 # --------------------------------------------------------------------------- forward functions
 @torch.no_grad()
 def int8_forward_dynamic(x: Tensor, weight: Tensor, weight_scale, bias, compute_dtype: torch.dtype,
-                         rotate: bool = False, addend: Tensor | None = None) -> Tensor:
+                         rotate: bool = False, addend: Tensor | None = None, prologue=None) -> Tensor:
     """Dynamic per-token activation quantisation, ONE weight scale (int8_quant.py:68-88)."""
-    return hip_int8_linear(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend)
+    return hip_int8_linear(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=prologue)
 
 
 @torch.no_grad()
 def int8_forward_dynamic_per_row(x: Tensor, weight: Tensor, weight_scale: Tensor, bias,
-                                 compute_dtype: torch.dtype, rotate: bool = False, addend: Tensor | None = None) -> Tensor:
+                                 compute_dtype: torch.dtype, rotate: bool = False, addend: Tensor | None = None,
+                                 prologue=None) -> Tensor:
     """Dynamic per-token activation quantisation, per-row weight scales [N,1] (int8_quant.py:92-119)."""
-    return hip_int8_linear_per_row(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend)
+    return hip_int8_linear_per_row(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend,
+                                   prologue=prologue)
 
 
 # --------------------------------------------------------------------------- LoRA delta reconstruction
@@ -401,8 +403,21 @@ class Int8TensorwiseOps(manual_cast):
                 self.bias = nn.Parameter(out_bias, requires_grad=False)
 
         # -- forward ------------------------------------------------------------------------
-        def forward(self, x: Tensor) -> Tensor:
+        def forward(self, x: Tensor, prologue: int = _lib.PRO_NONE, mod_scale: Tensor | None = None,
+                    mod_shift: Tensor | None = None) -> Tensor:
+            """The reference's forward(x) (int8_quant.py:703-778).  The optional arguments name the elementwise
+            operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, or _lib.PRO_MODULATE with
+            (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension -- which the W8A8 path
+            then applies inside its quantiser instead of in a pass of its own (under torch.compile the graph
+            rewrite of compile_ops does this without the caller's help)."""
             managed = self.comfy_cast_weights or len(self.weight_function) > 0 or len(self.bias_function) > 0
+            if prologue != _lib.PRO_NONE:
+                rows = x.numel() // max(1, x.shape[-1])
+                fusable = (self._is_quantized and rows > SMALL_BATCH_ROWS and self.lora_A is None
+                           and not torch.compiler.is_compiling())
+                if not fusable:   # every other path takes the operation as torch would have applied it
+                    x = F.gelu(x, approximate="tanh") if prologue == _lib.PRO_GELU_TANH else (1 + mod_scale) * x + mod_shift
+                    prologue = _lib.PRO_NONE
 
             if not self._is_quantized:
                 if not managed:
@@ -456,7 +471,8 @@ class Int8TensorwiseOps(manual_cast):
                                                   int8_fused_kernel.DEFAULT_EPILOGUE, addend)
                 else:
                     fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
-                    y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend)
+                    pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift)
+                    y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=pro)
             else:
                 # W8A16: activations keep their dtype (rotated first when the weight is rotated)
                 if compiling:

@@ -1,7 +1,11 @@
 """torch.library registration of the forward path: schemas and shape-only implementations on the CPU,
-Dynamo tracing of Linear.forward without graph breaks, and (GPU) compiled == eager bit for bit."""
+Dynamo tracing of Linear.forward without graph breaks, the graph rewrite that moves the elementwise
+operation in front of a layer into its quantiser, and (GPU) the compiled forward (aot_eager and
+inductor) against eager and against the CPU oracle."""
+import numpy as np
 import pytest
 import torch
+import torch.nn.functional as F
 
 
 def _load(lin, sd, prefix="l."):
@@ -67,6 +71,119 @@ def test_forward_traces_into_one_operator_without_graph_breaks(pkg, rows, op):
     assert not any("rotate128" in t for t in targets)          # rotation is folded into the operator
     other = "linear_w8a16_small_m" if op == "int8_linear" else "int8_linear"
     assert not any(other in t for t in targets)
+
+
+class _ModulatedMlp(torch.nn.Module):
+    """The MLP branch of a DiT block: adaLN modulation -> up projection -> tanh-GELU -> down projection."""
+
+    def __init__(self, up, down):
+        super().__init__()
+        self.up, self.down = up, down
+
+    def forward(self, x, scale, shift):
+        h = (1 + scale) * x + shift
+        return self.down(F.gelu(self.up(h), approximate="tanh"))
+
+
+def _mlp(pkg, k=256, hidden=512):
+    g = torch.Generator().manual_seed(11)
+    layers = []
+    for n_out, k_in in ((hidden, k), (k, hidden)):
+        lin = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        _load(lin, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                    "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+        layers.append(lin)
+    return _ModulatedMlp(*layers)
+
+
+def test_graph_rewrite_moves_modulation_and_gelu_into_the_quantiser(pkg):
+    m = _mlp(pkg)
+    x, sc, sh = torch.randn(2, 24, 256).bfloat16(), torch.randn(2, 1, 256).bfloat16(), torch.randn(2, 1, 256).bfloat16()
+    gm = torch._dynamo.export(m)(x, sc, sh).graph_module
+    assert pkg.compile_ops.fuse_prologues(gm) == 2
+    calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+    fused = [n for n in calls if "int8_linear_prologue" in str(n.target)]
+    assert [n.args[1] for n in fused] == [pkg._lib.PRO_MODULATE, pkg._lib.PRO_GELU_TANH]
+    assert not any("gelu" in str(n.target) or n.target.__name__ in ("add", "mul") for n in calls if hasattr(n.target, "__name__"))
+    assert not any(str(n.target).endswith("int8_linear") for n in calls)
+
+
+def test_graph_rewrite_leaves_other_producers_alone(pkg):
+    m = _mlp(pkg)
+
+    class Other(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.m = m
+
+        def forward(self, x, scale, shift):
+            h = (1 + scale) * x + shift            # scale has one vector per TOKEN here: not the adaLN broadcast
+            g = F.gelu(self.m.up(h))               # exact (erf) GELU: not the tanh form
+            return self.m.down(g) + g.sum()        # and its result is used twice
+    x, sc, sh = torch.randn(2, 24, 256).bfloat16(), torch.randn(2, 24, 256).bfloat16(), torch.randn(2, 24, 256).bfloat16()
+    gm = torch._dynamo.export(Other())(x, sc, sh).graph_module
+    assert pkg.compile_ops.fuse_prologues(gm) == 0
+
+
+def _oracle_linear(O, x2d, lin):
+    xa, code = O.from_torch(x2d)
+    return O.linear_w8a8(xa, code, lin.weight.cpu().numpy(), lin.weight_scale.cpu().numpy().reshape(-1),
+                         O.from_torch(lin.bias.cpu())[0], O.BF16, O.BF16, 0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [48, 8])
+def test_inductor_compiled_forward_equals_the_oracle(pkg, dev, O, rows):
+    """Linear.forward under torch.compile(backend="inductor", fullgraph=True), plus an elementwise consumer that
+    inductor generates code for, against the CPU oracle (W8A8 rows bit for bit; the W8A16 rows within the bound
+    of that path)."""
+    m = _mlp(pkg).to(dev)
+    lin = m.up
+    x = torch.randn(rows, 256, generator=torch.Generator().manual_seed(5)).bfloat16()
+
+    def fn(t):
+        return lin(t) * 2
+
+    got = torch.compile(fn, backend="inductor", fullgraph=True)(x.to(dev))
+    if rows > 16:
+        want = O.to_f32(_oracle_linear(O, x, lin), O.BF16) * 2        # doubling a bf16 value is exact
+        assert np.array_equal(got.float().cpu().numpy(), want)
+    else:
+        xa, code = O.from_torch(x)
+        ref = O.to_f32(O.linear_w8a16(xa, code, lin.weight.cpu().numpy(), lin.weight_scale.cpu().numpy().reshape(-1),
+                                      O.from_torch(lin.bias.cpu())[0], code), code) * 2
+        assert (np.abs(got.float().cpu().numpy() - ref) <= 2.0**-7 * np.abs(ref) + 1e-3).all()
+
+
+@pytest.mark.gpu
+def test_compiled_mlp_with_fused_prologues_equals_the_oracle(pkg, dev, O):
+    """Modulation -> up -> GELU -> down compiled with the rewriting backend over inductor: the first layer is
+    bit-identical to the oracle (modulation restated operation for operation), the second, whose GELU differs from
+    the C library's in the last bits of binary32, within two bf16 ulps of the output scale."""
+    m = _mlp(pkg).to(dev)
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(2, 24, 256, generator=g).bfloat16()
+    sc, sh = (torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16(), torch.randn(2, 1, 256, generator=g).bfloat16()
+    seen = []
+
+    def counting(gm, inputs):
+        seen.append(sum("int8_linear_prologue" in str(n.target) for n in gm.graph.nodes))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x.to(dev), sc.to(dev), sh.to(dev))
+    assert seen == [2]
+    xa, code = O.from_torch(x.reshape(48, 256))
+    h = O.prologue(xa, code, O.PRO_MODULATE, O.from_torch(sc.reshape(2, 256))[0], O.from_torch(sh.reshape(2, 256))[0], rows_per_vec=24)
+    y1 = O.linear_w8a8(h, code, m.up.weight.cpu().numpy(), m.up.weight_scale.cpu().numpy().reshape(-1),
+                       O.from_torch(m.up.bias.cpu())[0], O.BF16, O.BF16, 0)
+    assert np.array_equal(O.from_torch(m.up((1 + sc.to(dev)) * x.to(dev) + sh.to(dev)).reshape(48, -1).cpu())[0], y1)   # eager == oracle
+    y2 = O.linear_w8a8(O.prologue(y1, code, O.PRO_GELU_TANH), code, m.down.weight.cpu().numpy(),
+                       m.down.weight_scale.cpu().numpy().reshape(-1), O.from_torch(m.down.bias.cpu())[0], O.BF16, O.BF16, 0)
+    want = O.to_f32(y2, O.BF16).reshape(2, 24, 256)
+    diff = np.abs(got.float().cpu().numpy() - want)
+    assert diff.max() <= 2.0**-7 * np.abs(want).max()
+    assert (diff != 0).mean() < 0.02
 
 
 @pytest.mark.gpu

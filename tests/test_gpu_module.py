@@ -253,3 +253,28 @@ def test_dynamic_lora_hook_drives_the_side_branch(pkg, dev):
     assert model.proj.lora_A.device.type == "cuda"
     assert torch.equal(got, base + side.to(base.dtype))
     assert torch.equal(model(x), base)                     # no entries in this call: the branch is gone again
+
+
+def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
+    """forward(x, prologue=...) against the same layer fed the tensor torch computes first: bit-identical for the
+    modulation, within one step of the output dtype for the GELU (whose last binary32 bits differ from torch's)."""
+    import torch.nn.functional as F
+    L = pkg._lib
+    g = torch.Generator().manual_seed(21)
+    lin = pkg.Int8TensorwiseOps.Linear(384, 96, bias=True)
+    lin._load_from_state_dict({"l.weight": torch.randint(-127, 128, (96, 384), dtype=torch.int8, generator=g),
+                               "l.weight_scale": torch.rand(96, 1, generator=g) * 0.002 + 1e-3,
+                               "l.bias": torch.randn(96, generator=g).bfloat16()}, "l.", {}, True, [], [], [])
+    lin = lin.to(dev)
+    x = torch.randn(2, 20, 384, generator=g).bfloat16().to(dev)
+    sc, sh = (torch.randn(2, 1, 384, generator=g) * 0.3).bfloat16().to(dev), torch.randn(2, 1, 384, generator=g).bfloat16().to(dev)
+    for quarot in (False, True):
+        lin._use_quarot = quarot
+        a = lin(x, prologue=L.PRO_MODULATE, mod_scale=sc, mod_shift=sh)
+        b = lin((1 + sc) * x + sh)
+        assert a.shape == (2, 20, 96) and torch.equal(a, b)
+        a = lin(x, prologue=L.PRO_GELU_TANH)
+        b = lin(F.gelu(x, approximate="tanh"))
+        assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
+    small = x[:1, :4]                     # four rows: the W8A16 path applies the operation in torch
+    assert torch.equal(lin(small, prologue=L.PRO_GELU_TANH), lin(F.gelu(small, approximate="tanh")))
