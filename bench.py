@@ -77,12 +77,37 @@ def make_config(i: int, rows: int | None = None) -> dict:
     raise ValueError(i)
 
 
-# HBM-side bytes per GEMM launch of config 1, from two rocprofv3 --pmc runs of
-# comfyui-int8-fast_amd/profiling/traffic_probe.py (summary in profiles/hbm_traffic_fetch_write_size.txt):
-# FETCH_SIZE 120105 KiB / WRITE_SIZE 110679 KiB for 4608x12288x3072 and 153807 / 27648 KiB for
-# 4608x3072x12288; a 256 MiB device copy reads 131084 / 262144 KiB on the same counters, so fetches
-# scale by 2.00 and writes by 1.00.  The mean of the two launches:
-GEMM_TRAFFIC_BYTES = int(((120105 * 2.0 + 110679) + (153807 * 2.0 + 27648)) / 2 * 1024)
+# HBM-side bytes per GEMM launch come from profiles/gemm_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# figures per shape and tile configuration, with the commands that produced them and the calibration of the
+# counters against a plain copy.  They are a property of (shape, tile configuration), not of this run: a row is
+# used only while the library still picks the tile configuration it was measured with.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_hbm_traffic.txt")
+
+
+def gemm_traffic(L, M, N, K):
+    """HBM-side bytes of one M x N x K GEMM launch from the profile, or None (with the reason)."""
+    tile = L.gemm_tile(M, N, K)
+    try:
+        lines = open(TRAFFIC_FILE).read().splitlines()
+    except OSError:
+        return None, "profiles/gemm_hbm_traffic.txt is missing"
+    f_fetch = f_write = None
+    row = None
+    for ln in lines:
+        t = ln.split()
+        if len(t) >= 5 and t[0] == "calibration":
+            f_fetch, f_write = float(t[2]), float(t[4])
+        if len(t) >= 8 and t[0] == "traffic" and t[1] == f"{M}x{N}x{K}":
+            row = (t[3], float(t[5]), float(t[7]))
+    if row is None or f_fetch is None:
+        return None, f"no row for {M}x{N}x{K} in profiles/gemm_hbm_traffic.txt"
+    if row[0] != f"{tile[0]}x{tile[1]}":
+        return None, f"the profile row was measured with tile {row[0]}, the library now picks {tile[0]}x{tile[1]}: not measured for this tile"
+    return int((row[1] * f_fetch + row[2] * f_write) * 1024), None
+
+
+def gemm_algorithmic_bytes(M, N, K, out_bytes=2, bias=True):
+    return M * K + N * K + out_bytes * M * N + 4 * M + 4 * N + (2 * N if bias else 0)
 
 
 # --------------------------------------------------------------------------- timing helpers
@@ -158,16 +183,29 @@ def extras(L, dev, quick=False):
     iters = 20 if quick else 100
     g = torch.Generator().manual_seed(99)
 
-    # north-star target shape: M=4608, K=N=3072, W8A8 rowwise
+    # north-star target shape: M=4608, K=N=3072, W8A8 rowwise.  Warm: the same 23.6 MB of operands in a loop (they
+    # sit in the 256 MB memory-side cache).  Cold: 12 operand sets in turn (283 MB of int8 operands + 340 MB of
+    # outputs), which is what a layer inside a model sees.
     M, N, K = 4608, 3072, 3072
     x = _acts(g, M, K, 0.01, 20.0).to(dev)
     wq, ws = L.quant_rowwise((torch.randn(N, K, generator=g) * 0.02).to(dev))
     q, s = L.quant_rowwise(x)
     y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     t = time_kernel(lambda i: L.linear_w8a8(q, s, wq, ws, None, torch.bfloat16, L.EPI_TORCH, y), max(10, iters // 4), burst=8)
-    tops = 2 * M * N * K / t["median_us"] / 1e6
+    nset = 12
+    cq = [q] + [L.quant_rowwise(_acts(g, M, K, 0.01, 20.0).to(dev)) [0] for _ in range(nset - 1)]
+    cw = [wq] + [L.quant_rowwise(torch.randn(N, K, device=dev) * 0.02)[0] for _ in range(nset - 1)]
+    cy = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nset)]
+    tc = time_kernel(lambda i: L.linear_w8a8(cq[i], s, cw[i], ws, None, torch.bfloat16, L.EPI_TORCH, cy[i]), max(10, iters // 4),
+                     sets=nset, burst=nset)
+    ops = 2 * M * N * K
+    tops, tops_c = ops / t["median_us"] / 1e6, ops / tc["median_us"] / 1e6
     out["target_gemm_4608x3072x3072"] = {"median_us": round(t["median_us"], 2), "min_us": round(t["min_us"], 2),
-                                          "tops": round(tops, 1), "frac_of_int8_peak": round(tops / PEAK_INT8_TOPS, 4)}
+                                          "tops": round(tops, 1), "frac_of_int8_peak": round(tops / PEAK_INT8_TOPS, 4),
+                                          "cold_operands_median_us": round(tc["median_us"], 2), "cold_operands_tops": round(tops_c, 1),
+                                          "cold_operands_frac_of_int8_peak": round(tops_c / PEAK_INT8_TOPS, 4),
+                                          "tile": "%dx%d" % L.gemm_tile(M, N, K)[:2]}
+    del cq, cw, cy
 
     # fused rotate + quant at the same shape, cycling 8 buffer sets (> 256 MB in total), bursts of 8
     # launches per event pair; a plain device copy of the same byte count is timed beside them
@@ -192,7 +230,41 @@ def extras(L, dev, quick=False):
     t = time_kernel(lambda i: dsts[i].copy_(srcs[i]), reps, sets=sets, burst=sets)
     out["device_copy_same_bytes"] = {"median_us": round(t["median_us"], 2), "gbs": round(2 * half / t["median_us"] / 1e3, 1),
                                      "note": "torch copy_ of 21.2 MB -> 21.2 MB over the same rotation of buffers, for comparison"}
-    del xs, qs, ss, srcs, dsts
+    # the quantiser with the elementwise operation in front of the layer applied on the fly, against the same
+    # operation as a torch kernel of its own followed by the plain quantiser
+    import torch.nn.functional as F
+    sc, sh = (torch.randn(1, K, device=dev) * 0.3).bfloat16(), torch.randn(1, K, device=dev).bfloat16()
+    def fused_call(i, kind, src, dq, ds, cols):
+        rc = lib.i8f_quant_rowwise_prologue(ptr(src[i]), L.BF16, M, cols, cols, kind, ptr(sc), ptr(sh), M, 0, ptr(dq[i]), ptr(ds[i]), stream)
+        assert rc == 0, rc
+
+    def plain_call(src, dq, ds, cols):
+        rc = lib.i8f_quant_rowwise(ptr(src), L.BF16, M, cols, cols, 0, ptr(dq), ptr(ds), stream)
+        assert rc == 0, rc
+
+    def mod_unfused(i):
+        plain_call((1 + sc) * xs[i] + sh, qs[i], ss[i], K)
+
+    t_f = time_kernel(lambda i: fused_call(i, L.PRO_MODULATE, xs, qs, ss, K), reps, sets=sets, burst=sets)
+    t_u = time_kernel(mod_unfused, reps, sets=sets, burst=sets)
+    out["modulate_quant_4608x3072"] = {"fused_median_us": round(t_f["median_us"], 2), "torch_ops_then_quant_median_us": round(t_u["median_us"], 2),
+                                       "fused_gbs": round(qbytes / t_f["median_us"] / 1e3, 1)}
+    hs = [torch.randn(M, 12288, device=dev).bfloat16() for _ in range(3)]
+    hq = [torch.empty(M, 12288, dtype=torch.int8, device=dev) for _ in range(3)]
+
+    def gelu_unfused(i):
+        plain_call(F.gelu(hs[i], approximate="tanh"), hq[i], ss[i], 12288)
+
+    t_p = time_kernel(lambda i: plain_call(hs[i], hq[i], ss[i], 12288), reps, sets=3, burst=3)
+    t_f = time_kernel(lambda i: fused_call(i, L.PRO_GELU_TANH, hs, hq, ss, 12288), reps, sets=3, burst=3)
+    t_u = time_kernel(gelu_unfused, reps, sets=3, burst=3)
+    hbytes = M * 12288 * 3 + 4 * M
+    out["gelu_quant_4608x12288"] = {"fused_median_us": round(t_f["median_us"], 2), "torch_gelu_then_quant_median_us": round(t_u["median_us"], 2),
+                                    "plain_quant_median_us": round(t_p["median_us"], 2), "fused_gbs": round(hbytes / t_f["median_us"] / 1e3, 1),
+                                    "plain_gbs": round(hbytes / t_p["median_us"] / 1e3, 1),
+                                    "note": "config 1's down-projection input: the fused form never writes the 113 MB activated tensor"}
+    del hq
+    del xs, qs, ss, srcs, dsts, hs
 
     # config 4: stochastic LoRA merge (rank 32 rebuilt in the kernel, float noise) and the skinny GEMM
     c = make_config(4)
@@ -356,6 +428,11 @@ def main():
     ms_per_step = wall / a.steps * 1e3
     value = 2 * step.gemm_ops / (ms_per_step * 1e-3) / 1e12
 
+    tr = [gemm_traffic(L, 4608, 12288, 3072), gemm_traffic(L, 4608, 3072, 12288)]
+    traffic = None if any(t[0] is None for t in tr) else (tr[0][0] + tr[1][0]) // 2
+    traffic_note = "; ".join(t[1] for t in tr if t[1]) or None
+    alg_bytes = (gemm_algorithmic_bytes(4608, 12288, 3072) + gemm_algorithmic_bytes(4608, 3072, 12288)) // 2
+
     line = {
         "metric": "INT8 GEMM TOPS (% of int8 MFMA peak) + ms per Flux-style DiT block, 1 GPU",
         "value": round(value, 1),
@@ -374,17 +451,41 @@ def main():
                                "quantise + GEMM for both projections, inputs resident in HBM"},
         "pct_of_int8_peak": round(100 * value / PEAK_INT8_TOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
-                     "traffic_unit": "bytes per launch beyond L2 (mean of the two GEMM launches; FETCH_SIZE x 2.00 + "
-                                     "WRITE_SIZE x 1.00, the factors a 256 MiB device copy gives)",
+                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": traffic,
+                     "traffic_unit": "bytes per launch beyond L2, mean of the two GEMM launches of the step, from "
+                                     "profiles/gemm_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a copy)",
+                     "algorithmic_bytes": alg_bytes,
+                     "traffic_over_algorithmic": None if traffic is None else round(traffic / alg_bytes, 2),
                      "kernel": "gemm_i8_kernel (int8 MFMA GEMM + dequant epilogue)",
+                     "tiles": {"4608x12288x3072": "%dx%d" % L.gemm_tile(4608, 12288, 3072)[:2],
+                               "4608x3072x12288": "%dx%d" % L.gemm_tile(4608, 3072, 12288)[:2]},
                      "ops_per_launch": step.gemm_ops, "avg_launch_us": round(avg_gemm_us, 2),
                      "launches_timed": len(gemm_us)},
     }
+    if traffic_note:
+        line["roofline"]["traffic_note"] = traffic_note
     extra = extras(L, dev, quick=a.quick) if not a.no_extras else None   # before the CPU leg: the GPU is still warm
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
     if extra is not None:
+        # the north-star shape as a roofline block of its own (the `roofline` block above is the step's GEMMs)
+        tg = extra["target_gemm_4608x3072x3072"]
+        t_traffic, t_note = gemm_traffic(L, 4608, 3072, 3072)
+        t_alg = gemm_algorithmic_bytes(4608, 3072, 3072, bias=False)
+        line["roofline_target"] = {"bound": "mfma", "shape": "M=4608, N=K=3072, W8A8 rowwise, bf16 out", "tile": tg["tile"],
+                                   "ops_per_launch": 2 * 4608 * 3072 * 3072, "avg_launch_us": tg["median_us"],
+                                   "achieved": tg["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": tg["frac_of_int8_peak"],
+                                   "operands": "the same operands in a loop (resident in the 256 MB memory-side cache)",
+                                   "cold_operands_avg_launch_us": tg["cold_operands_median_us"],
+                                   "cold_operands_frac": tg["cold_operands_frac_of_int8_peak"],
+                                   "traffic": t_traffic, "algorithmic_bytes": t_alg,
+                                   "traffic_over_algorithmic": None if t_traffic is None else round(t_traffic / t_alg, 2)}
+        if t_note:
+            line["roofline_target"]["traffic_note"] = t_note
+        rq = extra["rotate_quant_4608x3072"]
+        line["roofline_rotate_quant"] = {"bound": "hbm", "kernel": "quant16_kernel (rotate + absmax + int8, one pass)",
+                                         "bytes_per_launch": rq["bytes"], "avg_launch_us": rq["median_us"],
+                                         "achieved": rq["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": rq["frac_of_hbm_peak"]}
         line["extras"] = extra
         if "dit_block_linears" in extra:
             line["dit_block_ms"] = extra["dit_block_linears"]["ms"]

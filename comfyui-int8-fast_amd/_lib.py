@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
     L.i8f_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp, vp, i64, vp]
     L.i8f_quant_tensorwise_static.argtypes = [vp, i32, i64, vp, vp, vp]
     L.i8f_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp, vp]
+    L.i8f_gemm_tile.argtypes = [i64, i64, i64, ctypes.POINTER(i32), ctypes.POINTER(i32), ctypes.POINTER(i32)]
+    L.i8f_gemm_tile.restype = i32
     L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
@@ -74,7 +76,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue",
-    "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
 
@@ -223,6 +225,13 @@ def _i8_matrix(t: torch.Tensor, name: str) -> torch.Tensor:
     if t.dtype != torch.int8 or t.dim() != 2:
         raise TypeError(f"{name} must be a 2-D int8 tensor, got {t.dtype} {tuple(t.shape)}")
     return t if t.is_contiguous() else t.contiguous()
+
+
+def gemm_tile(M: int, N: int, K: int):
+    """(tile rows, tile columns, LDS stages) of the GEMM kernel variant an aligned M x N x K problem takes."""
+    bm, bn, st = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _check(lib().i8f_gemm_tile(M, N, K, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(st)), "i8f_gemm_tile")
+    return bm.value, bn.value, st.value
 
 
 def gemm_i32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

@@ -650,6 +650,84 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
     return check_launch();
 }
 
+enum Tile { TILE_BIG, TILE_B192, TILE_MID, TILE_TALL, TILE_WIDE, TILE_W96, TILE_MID_DEEP, TILE_M96_DEEP, TILE_S64_DEEP, TILE_T64_DEEP };
+
+// The tile configuration an M x N output takes (K does not enter).
+Tile choose_tile(int64_t M, int64_t N) {
+    // With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
+    // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
+    // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA) and the 288 x 256 tile of
+    // twelve waves, or 256 x 288, about 2 % (they pay where they save a round: 4608 x 12288 takes 768
+    // tiles of 288 x 256, three rounds, instead of 864 of 256 x 256, four; 4096 x 9216 takes 512 of
+    // 256 x 288, two rounds).  Outputs of fewer than 128
+    // such tiles take 128 x 128 tiles with two stages if that gives at least one workgroup per CU,
+    // else the four-stage configurations above.
+    const int64_t CUS = 256;
+    auto rounds_cost = [&](int bm, int bn, int per_op_cost) {
+        const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+        return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn * per_op_cost;
+    };
+    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    if (big_tiles < 128) {
+        const int64_t mid_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+        if (mid_tiles >= CUS) {
+            // Two 128 x 128 tiles to a CU fetch 2 x 256 rows per K-step, one 256 x 96 tile 352: the
+            // narrow tile wins where it still covers the output in one round (512 x 12288: 256 tiles).
+            const int64_t w96_tiles = (int64_t)((M + 255) / 256) * ((N + 95) / 96);
+            const int64_t f_w96 = ((w96_tiles + CUS - 1) / CUS) * (256 + 96);
+            const int64_t f_mid2 = ((mid_tiles + 2 * CUS - 1) / (2 * CUS)) * 2 * (128 + 128);
+            if (f_w96 < f_mid2) return TILE_W96;
+            return TILE_MID;
+        }
+        // Few tiles: the global->LDS path of a CU is what bounds these shapes, so a configuration costs
+        // the bytes its busiest CU has to fetch: (BM + BN) per K-step times the tiles that CU gets.
+        // Ties go to the larger tile (less traffic in total).
+        auto fetch_cost = [&](int bm, int bn) {
+            const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+            return ((tiles + CUS - 1) / CUS) * (bm + bn);
+        };
+        const int64_t f_mid = fetch_cost(128, 128), f_96 = fetch_cost(128, 96), f_s64 = fetch_cost(128, 64), f_t64 = fetch_cost(64, 64);
+        const int64_t f_min = std::min(std::min(f_mid, f_96), std::min(f_s64, f_t64));
+        if (f_mid == f_min) return TILE_MID_DEEP;
+        if (f_96 == f_min) return TILE_M96_DEEP;
+        if (f_s64 == f_min) return TILE_S64_DEEP;
+        return TILE_T64_DEEP;
+    }
+    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108);
+    const int64_t c_tall = rounds_cost(288, 256, 102), c_wide = rounds_cost(256, 288, 102);
+    // 128 x 128 tiles, two workgroups to a CU: 41 % dearer per operation, but nothing is wasted on a
+    // ragged M (640 x 12288: one round of 480 of them against 192 tiles of 256 x 192)
+    const int64_t mid_all = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+    const int64_t c_mid = ((mid_all + 2 * CUS - 1) / (2 * CUS)) * 2 * 128 * 128 * 141;
+    const int64_t c_min = std::min(std::min(std::min(c_big, c_192), std::min(c_tall, c_wide)), c_mid);
+    if (c_big == c_min) return TILE_BIG;
+    if (c_mid == c_min) return TILE_MID;
+    if (c_tall == c_min) return TILE_TALL;
+    if (c_wide == c_min) return TILE_WIDE;
+    return TILE_B192;
+}
+
+template <int OUT>
+int launch_tile(Tile t, GemmArgs &g, hipStream_t st) {
+    switch (t) {
+    case TILE_BIG: return launch_cfg<CfgBig, OUT>(g, st);
+    case TILE_B192: return launch_cfg<CfgB192, OUT>(g, st);
+    case TILE_MID: return launch_cfg<CfgMid, OUT>(g, st);
+    case TILE_TALL: return launch_cfg<CfgTall, OUT>(g, st);
+    case TILE_WIDE: return launch_cfg<CfgWide, OUT>(g, st);
+    case TILE_W96: return launch_cfg<CfgW96, OUT>(g, st);
+    case TILE_MID_DEEP: return launch_cfg<CfgMidDeep, OUT>(g, st);
+    case TILE_M96_DEEP: return launch_cfg<CfgM96Deep, OUT>(g, st);
+    case TILE_S64_DEEP: return launch_cfg<CfgS64Deep, OUT>(g, st);
+    default: return launch_cfg<CfgT64Deep, OUT>(g, st);
+    }
+}
+
+template <class C>
+void tile_dims(int *bm, int *bn, int *stages) {
+    *bm = C::BM, *bn = C::BN, *stages = C::STAGES;
+}
+
 template <int OUT>
 int launch(GemmArgs &g, hipStream_t st) {
     const int ob = OutElem<OUT>::BYTES;
@@ -677,57 +755,7 @@ int launch(GemmArgs &g, hipStream_t st) {
         hipLaunchKernelGGL((gemm_i8_generic_kernel<OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, g);
         return check_launch();
     }
-    // Tile choice.  With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
-    // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
-    // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA) and the 288 x 256 tile of
-    // twelve waves, or 256 x 288, about 2 % (they pay where they save a round: 4608 x 12288 takes 768
-    // tiles of 288 x 256, three rounds, instead of 864 of 256 x 256, four; 4096 x 9216 takes 512 of
-    // 256 x 288, two rounds).  Outputs of fewer than 128
-    // such tiles take 128 x 128 tiles with two stages if that gives at least one workgroup per CU,
-    // else the four-stage configurations above.
-    const int64_t CUS = 256;
-    auto rounds_cost = [&](int bm, int bn, int per_op_cost) {
-        const int64_t tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
-        return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn * per_op_cost;
-    };
-    const int64_t big_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    if (big_tiles < 128) {
-        const int64_t mid_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
-        if (mid_tiles >= CUS) {
-            // Two 128 x 128 tiles to a CU fetch 2 x 256 rows per K-step, one 256 x 96 tile 352: the
-            // narrow tile wins where it still covers the output in one round (512 x 12288: 256 tiles).
-            const int64_t w96_tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 95) / 96);
-            const int64_t f_w96 = ((w96_tiles + CUS - 1) / CUS) * (256 + 96);
-            const int64_t f_mid2 = ((mid_tiles + 2 * CUS - 1) / (2 * CUS)) * 2 * (128 + 128);
-            if (f_w96 < f_mid2) return launch_cfg<CfgW96, OUT>(g, st);
-            return launch_cfg<CfgMid, OUT>(g, st);
-        }
-        // Few tiles: the global->LDS path of a CU is what bounds these shapes, so a configuration costs
-        // the bytes its busiest CU has to fetch: (BM + BN) per K-step times the tiles that CU gets.
-        // Ties go to the larger tile (less traffic in total).
-        auto fetch_cost = [&](int bm, int bn) {
-            const int64_t tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
-            return ((tiles + CUS - 1) / CUS) * (bm + bn);
-        };
-        const int64_t f_mid = fetch_cost(128, 128), f_96 = fetch_cost(128, 96), f_s64 = fetch_cost(128, 64), f_t64 = fetch_cost(64, 64);
-        const int64_t f_min = std::min(std::min(f_mid, f_96), std::min(f_s64, f_t64));
-        if (f_mid == f_min) return launch_cfg<CfgMidDeep, OUT>(g, st);
-        if (f_96 == f_min) return launch_cfg<CfgM96Deep, OUT>(g, st);
-        if (f_s64 == f_min) return launch_cfg<CfgS64Deep, OUT>(g, st);
-        return launch_cfg<CfgT64Deep, OUT>(g, st);
-    }
-    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108);
-    const int64_t c_tall = rounds_cost(288, 256, 102), c_wide = rounds_cost(256, 288, 102);
-    // 128 x 128 tiles, two workgroups to a CU: 41 % dearer per operation, but nothing is wasted on a
-    // ragged M (640 x 12288: one round of 480 of them against 192 tiles of 256 x 192)
-    const int64_t mid_all = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
-    const int64_t c_mid = ((mid_all + 2 * CUS - 1) / (2 * CUS)) * 2 * 128 * 128 * 141;
-    const int64_t c_min = std::min(std::min(std::min(c_big, c_192), std::min(c_tall, c_wide)), c_mid);
-    if (c_big == c_min) return launch_cfg<CfgBig, OUT>(g, st);
-    if (c_mid == c_min) return launch_cfg<CfgMid, OUT>(g, st);
-    if (c_tall == c_min) return launch_cfg<CfgTall, OUT>(g, st);
-    if (c_wide == c_min) return launch_cfg<CfgWide, OUT>(g, st);
-    return launch_cfg<CfgB192, OUT>(g, st);
+    return launch_tile<OUT>(choose_tile(g.M, g.N), g, st);
 }
 
 int validate(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K, const void *out) {
@@ -784,4 +812,27 @@ extern "C" int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8
                                int out_dtype, int64_t M, int64_t N, int64_t K, int order, void *stream) {
     return i8f_linear_w8a8_add(a, a_scale, w, w_scale, w_scale_host, scale_mode, bias, bias_dtype, nullptr, out,
                                out_dtype, M, N, K, order, stream);
+}
+
+extern "C" int i8f_gemm_tile(int64_t M, int64_t N, int64_t K, int *bm, int *bn, int *stages) {
+    using namespace i8f;
+    if (M <= 0 || N <= 0 || K < 0 || !bm || !bn || !stages) return I8F_ERR_INVALID;
+    if (K % 16 || N % 8 || N * K >= (1ll << 31)) {  // such shapes take the one-thread-per-output kernel
+        *bm = *bn = 1, *stages = 0;
+        return I8F_OK;
+    }
+    if (M * K >= (1ll << 31)) M = (((1ll << 31) - 1) / K) / 256 * 256;  // launched in row blocks of this size
+    switch (choose_tile(M, N)) {
+    case TILE_BIG: tile_dims<CfgBig>(bm, bn, stages); break;
+    case TILE_B192: tile_dims<CfgB192>(bm, bn, stages); break;
+    case TILE_MID: tile_dims<CfgMid>(bm, bn, stages); break;
+    case TILE_TALL: tile_dims<CfgTall>(bm, bn, stages); break;
+    case TILE_WIDE: tile_dims<CfgWide>(bm, bn, stages); break;
+    case TILE_W96: tile_dims<CfgW96>(bm, bn, stages); break;
+    case TILE_MID_DEEP: tile_dims<CfgMidDeep>(bm, bn, stages); break;
+    case TILE_M96_DEEP: tile_dims<CfgM96Deep>(bm, bn, stages); break;
+    case TILE_S64_DEEP: tile_dims<CfgS64Deep>(bm, bn, stages); break;
+    default: tile_dims<CfgT64Deep>(bm, bn, stages); break;
+    }
+    return I8F_OK;
 }

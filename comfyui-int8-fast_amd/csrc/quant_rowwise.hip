@@ -359,13 +359,14 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
 
         float v[RUNS][16];
         float amax = 0.0f;
+        [[maybe_unused]] int64_t vrow = 0;  // the row's pair of modulation vectors (M < 2^31: a 32-bit division)
+        if constexpr (PRO == I8F_PRO_MODULATE) vrow = (uint32_t)(m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
             expand16<DT>(raw[it & 1][r][0], raw[it & 1][r][1], v[r]);
             if constexpr (PRO == I8F_PRO_MODULATE) {
                 // the vectors of this row's group, same 16 columns (they come from cache: every row of the group reads them)
                 const int R = r * TPR + p;
-                const int64_t vrow = (m < M ? m : 0) / pro.rows_per_vec;
                 const int64_t off = (vrow * K + (R < nruns ? R : 0) * 16) * 2;
                 float sv[16], tv[16];
                 expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), sv);
@@ -676,6 +677,7 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
     if (prologue == I8F_PRO_MODULATE && (rows_per_vec <= 0 || (K > 0 && (!mod_scale || !mod_shift)))) return I8F_ERR_INVALID;
     if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
     if (int rc = check_device()) return rc;
+    if (rows_per_vec > 0x7fffffff) rows_per_vec = 0x7fffffff;  // M itself is below 2^31
     Prologue pro{prologue, mod_scale, mod_shift, rows_per_vec > 0 ? rows_per_vec : 1};
     hipStream_t st = (hipStream_t)stream;
     const bool rot = rotate_block != 0;

@@ -178,6 +178,15 @@ int i8f_gemm_i32(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t
                  int32_t *acc, void *stream);
 
 /*
+ * The tile configuration i8f_gemm_i32 / i8f_linear_w8a8 use for an aligned M x N x K
+ * problem: rows and columns of the output tile one workgroup computes and the number
+ * of K-tile stages it keeps in LDS (1 x 1, 0 stages for shapes that take the
+ * one-thread-per-output kernel).  No counterpart in the reference; for benchmarks
+ * and profiles that have to name the kernel variant they measured.
+ */
+int i8f_gemm_tile(int64_t M, int64_t N, int64_t K, int *bm, int *bn, int *stages);
+
+/*
  * INT8 GEMM with the dequantisation epilogue fused in registers.
  * Replaces _int8_matmul_dequant_kernel and _int8_matmul_dequant_per_row_kernel
  * (int8_fused_kernel.py:91-173, 253-324) and the torch epilogue

@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 15
+    assert len(names) == 16
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -110,3 +110,13 @@ def test_product_code_never_imports_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
                 assert "_int_mm(" not in text, f"{f} calls torch._int_mm"
+
+
+def test_gemm_tile_reports_the_configuration_of_the_benchmark_shapes(L):
+    """Host-only: the tile choice is a function of the shape."""
+    assert L.gemm_tile(4608, 3072, 3072) == (256, 256, 2)
+    assert L.gemm_tile(4608, 12288, 3072) == (288, 256, 2)
+    assert L.gemm_tile(4608, 3072, 12288) == (256, 256, 2)
+    assert L.gemm_tile(512, 12288, 3072) == (256, 96, 3)
+    assert L.gemm_tile(33, 64, 77) == (1, 1, 0)           # K % 16 != 0: the generic kernel
+    assert L.lib().i8f_gemm_tile(0, 8, 16, None, None, None) == -1
