@@ -386,6 +386,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--quick", action="store_true", help="fewer iterations in the extra measurements")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="diagnostic: all-zero activations and weights (same instructions, no switching in the multipliers), "
+                         "to show what the power limit costs; the line says data = zeros and is not a benchmark result")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: the INT8 linear path has no multi-GPU part (run with --gpus 1)")
@@ -399,6 +402,9 @@ def main():
     torch.cuda.set_device(dev)
 
     step = MlpStep(L, dev)
+    if a.zero_operands:
+        for t in (step.x, step.h, step.wq_up, step.wq_dn):
+            t.zero_()
     # torch creates the HIP event behind an Event at its first record(): do that here, not inside
     # the timed region
     evs = [_events(4) for _ in range(a.steps)]
@@ -445,7 +451,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "int8",
-        "data": "synthetic",
+        "data": "zeros (power diagnostic, not a result)" if a.zero_operands else "synthetic",
         "clock_ramp_s": a.clock_ramp_s,
         "config": {"workload": "BASELINE config 1: Flux MLP W8A8 rowwise, M=4608, 3072->12288->3072, bf16 in/out, bias; "
                                "quantise + GEMM for both projections, inputs resident in HBM"},
