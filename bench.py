@@ -287,6 +287,31 @@ def extras(L, dev, quick=False):
                                          "tops": round(2 * 256 * Nw * Kw / t["median_us"] / 1e6, 1)}
     del noises, outs
 
+    # dynamic (unmerged) LoRA side branch, rank 32, on config 1's up-projection: the second rank-r product and the
+    # addition inside the GEMM epilogue, against torch's F.linear for the [M,N] side tensor + the addition in the epilogue
+    Mu, Nu, Ku, r = 4608, 12288, 3072, 32
+    xu = _acts(g, Mu, Ku, 0.01, 20.0).to(dev)
+    wqu, wsu = L.quant_rowwise(torch.randn(Nu, Ku, device=dev) * 0.02)
+    bu = (torch.randn(Nu, device=dev) * 0.01).bfloat16()
+    lA, lB = (torch.randn(r, Ku, device=dev) * 0.02).bfloat16(), (torch.randn(Nu, r, device=dev) * 0.02).bfloat16()
+    qu, su = L.quant_rowwise(xu)
+    yu = torch.empty(Mu, Nu, dtype=torch.bfloat16, device=dev)
+
+    def lora_fused(_i):
+        L.linear_w8a8_lora(qu, su, wqu, wsu, bu, F.linear(xu, lA), lB, None, torch.bfloat16, L.EPI_TORCH, yu)
+
+    def lora_side_tensor(_i):
+        L.linear_w8a8(qu, su, wqu, wsu, bu, torch.bfloat16, L.EPI_TORCH, yu, addend=F.linear(F.linear(xu, lA), lB))
+
+    t_plain = time_kernel(lambda i: L.linear_w8a8(qu, su, wqu, wsu, bu, torch.bfloat16, L.EPI_TORCH, yu), max(10, iters // 4))
+    t_f = time_kernel(lora_fused, max(10, iters // 4))
+    t_u = time_kernel(lora_side_tensor, max(10, iters // 4))
+    out["dynamic_lora_r32_4608x12288x3072"] = {"gemm_alone_median_us": round(t_plain["median_us"], 2),
+                                               "side_branch_in_epilogue_median_us": round(t_f["median_us"], 2),
+                                               "side_tensor_then_add_in_epilogue_median_us": round(t_u["median_us"], 2),
+                                               "note": "both include the first product x @ A.T in torch; the fused form takes 256x256 tiles"}
+    del xu, wqu, yu
+
     # config 2: QuaRot layer (width 3840, 2 % of the channels x50): time of the rotated path and what the
     # rotation buys in accuracy against the bf16 product
     c2 = make_config(2)

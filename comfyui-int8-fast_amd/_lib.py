@@ -63,10 +63,11 @@ def lib() -> ctypes.CDLL:
     L.i8f_gemm_tile.restype = i32
     L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
+    L.i8f_linear_w8a8_lora.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i64, i32, f32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add",
+    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -76,7 +77,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue",
-    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
 
@@ -289,6 +290,53 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
         _check(lib().i8f_linear_w8a8_add(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
                                          _ptr(addend), _ptr(out), dtype_code(out.dtype), M, N, K, order, _stream(a)),
                "i8f_linear_w8a8_add")
+    return out
+
+
+def lora_side_fusable(M: int, N: int, K: int, rank: int, out_dtype, side_dtype) -> bool:
+    """Whether linear_w8a8_lora takes this problem (else: a side tensor and linear_w8a8(addend=...))."""
+    return (out_dtype in (torch.bfloat16, torch.float16) and side_dtype == out_dtype and 0 < rank <= 64
+            and K % 128 == 0 and N % 8 == 0 and M > 0)
+
+
+def linear_w8a8_lora(a, a_scale, w, w_scale, bias, side_t, side_b, alpha=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None):
+    """linear_w8a8 plus the low-rank side branch side_t [M,r] @ side_b [N,r].T (both of out_dtype), formed inside the
+    GEMM epilogue: round(y + round(round(side) * alpha)).  A rank that is not a multiple of 16 is padded with zero
+    columns (they add exact zeros)."""
+    a, w = _i8_matrix(a, "a"), _i8_matrix(w, "w")
+    M, K = a.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise ValueError(f"K mismatch: a has {K}, w has {K2}")
+    for name, t, rows in (("side_t", side_t, M), ("side_b", side_b, N)):
+        _dev(t, name)
+        if t.dim() != 2 or t.shape[0] != rows or t.dtype != out_dtype or t.device != a.device:
+            raise ValueError(f"{name} must be [{rows}, rank] of {out_dtype} on {a.device}")
+    r = side_t.shape[1]
+    if side_b.shape[1] != r:
+        raise ValueError("side_t and side_b disagree on the rank")
+    if not lora_side_fusable(M, N, K, r, out_dtype, side_t.dtype):
+        raise ValueError("this problem has no fused side branch (see lora_side_fusable)")
+    if r % 16:
+        pad = 16 - r % 16
+        side_t = torch.nn.functional.pad(side_t, (0, pad))
+        side_b = torch.nn.functional.pad(side_b, (0, pad))
+        r += pad
+    side_t, side_b = side_t.contiguous(), side_b.contiguous()
+    a_scale = a_scale.reshape(-1).contiguous()
+    if a_scale.numel() != M or a_scale.dtype != torch.float32:
+        raise ValueError("a_scale must be float32 with M elements")
+    ws, ws_host, mode = _scale(w_scale, N, a.device)
+    bias, bcode = _bias_arg(bias, N, a.device)
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    elif tuple(out.shape) != (M, N) or not out.is_contiguous() or out.dtype != out_dtype or out.device != a.device:
+        raise ValueError(f"out must be a contiguous [{M},{N}] tensor of {out_dtype} on {a.device}")
+    with torch.cuda.device(a.device):
+        _check(lib().i8f_linear_w8a8_lora(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
+                                          _ptr(side_t), _ptr(side_b), r, 0 if alpha is None else 1,
+                                          0.0 if alpha is None else float(alpha), _ptr(out), dtype_code(out_dtype), M, N, K, order,
+                                          _stream(a)), "i8f_linear_w8a8_lora")
     return out
 
 

@@ -35,6 +35,19 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum { OUT_BF16 = 0, OUT_F16 = 1, OUT_F32 = 2, OUT_I32 = 3 };
 
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+
+// 32 x 32 x 16 product of two 16-bit fragments (8 values per lane each) into a binary32 block
+template <int OUT>
+__device__ __forceinline__ v16f side_mfma(v4i a, v4i b, v16f c) {
+    if constexpr (OUT == OUT_BF16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf_t, a), __builtin_bit_cast(v8bf_t, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, a), __builtin_bit_cast(v8h_t, b), c, 0, 0, 0);
+}
+
 struct GemmArgs {
     const int8_t *x;
     const int8_t *w;
@@ -47,6 +60,11 @@ struct GemmArgs {
     int bias_dtype;
     int order;
     const void *addend;  // nullptr or [M,N] of the output dtype, added to the rounded result
+    // low-rank side branch, side[m,n] = sum_j side_t[m,j] * side_b[n,j] (operands of the output dtype, rank % 16 == 0),
+    // rounded to that dtype, times side_alpha if side_has_alpha (rounded again), added to the rounded result
+    const void *side_t, *side_b;
+    int side_rank, side_has_alpha;
+    float side_alpha;
     void *out;
     int tiles_m, tiles_n;
 };
@@ -114,9 +132,9 @@ struct OutElem {
 
 // One 4-element group of the epilogue, with the operation order, the scale mode and the bias
 // fixed at compile time (a run-time test per value costs more than the arithmetic).
-template <int OUT, int ORDER, bool ROW, bool BIAS>
+template <int OUT, int ORDER, bool ROW, bool BIAS, bool SIDE = false>
 __device__ __forceinline__ void epilogue_quad(const int (&a4)[4], float xs, const float4 w4, const float4 b4,
-                                              char *dst) {
+                                              char *dst, const float *side4 = nullptr) {
     constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : (OUT == OUT_F16 ? I8F_F16 : I8F_F32);
     const float wsv[4] = {w4.x, w4.y, w4.z, w4.w};
     const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
@@ -140,6 +158,8 @@ __device__ __forceinline__ void epilogue_quad(const int (&a4)[4], float xs, cons
             t = a * sc;
             if constexpr (BIAS) t = t + bv[e];
         }
+        // the side branch is added to the ROUNDED result, as a tensor addition would (y + side.to(y.dtype))
+        if constexpr (SIDE) t = round_to_dtype<DT>(t) + side4[e];
         y[e] = t;
     }
     if constexpr (OUT == OUT_BF16) {
@@ -185,7 +205,7 @@ __device__ __forceinline__ uint4 add_rounded(uint4 y, uint4 s) {
 // What the prologue needs (operand pointers, sizes, tile counts) comes first in the argument list: the
 // first 16 dwords of the kernel arguments are preloaded into SGPRs at wave launch, the rest (epilogue
 // operands) is fetched by scalar loads that have the whole main loop to land.
-template <class C, int OUT, bool KTAIL>
+template <class C, int OUT, bool KTAIL, bool SIDE = false>
 __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
                                                         const float *gxs, const float *gws, const void *gbias, int flags,
                                                         const GemmArgs g) {
@@ -482,7 +502,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // With more than 8 waves a wave has fewer registers than the accumulators plus the operands of
     // all its columns need: the column operands are then fetched per 32-column block, and a block is
     // converted for all staged strips before the next one is fetched.
-    constexpr bool PRELOAD_ALL = C::NT <= 512;
+    // (the variant with a low-rank side branch needs registers for its operands: per-block fetches as well)
+    constexpr bool PRELOAD_ALL = C::NT <= 512 && !SIDE;
     auto run_epilogue = [&](auto ORDER, auto ROW, auto BIAS) {
         constexpr int NPRE = PRELOAD_ALL ? NI : 1;
         float4 wr[NPRE][4], br[NPRE][4];
@@ -523,16 +544,49 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
 #pragma unroll
                 for (int j = 0; j < NI; ++j) {
                     fetch_cols(j, wr[0], br[0]);
+                    // side branch: the rank-r product of this 32 x 32 block on the matrix cores, with the same
+                    // operand roles as the main product (rows n from side_b, columns m from side_t), so that
+                    // the result has the accumulators' layout
+                    constexpr int RMAX = 64;
+                    [[maybe_unused]] v4i bfr[RMAX / 16];
+                    if constexpr (SIDE) {
+                        const int n = min(n0 + wn * C::WTN + j * 32 + l32, gN - 1);
+#pragma unroll
+                        for (int ks = 0; ks < RMAX / 16; ++ks)
+                            if (ks * 16 < g.side_rank)
+                                bfr[ks] = *(const v4i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lhalf * 8) * 2);
+                    }
 #pragma unroll
                     for (int is = 0; is < EPI_STRIPS; ++is) {
                         const int i = i0 + is;
                         const float xs = s_xs[wm * C::WTM + i * 32 + l32];
+                        [[maybe_unused]] float sd[16];
+                        if constexpr (SIDE) {
+                            const int m = min(m0 + wm * C::WTM + i * 32 + l32, gM - 1);
+                            v16f sacc;
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
+#pragma unroll
+                            for (int ks = 0; ks < RMAX / 16; ++ks) {
+                                if (ks * 16 < g.side_rank) {
+                                    const v4i tfr = *(const v4i *)((const char *)g.side_t + ((int64_t)m * g.side_rank + ks * 16 + lhalf * 8) * 2);
+                                    sacc = side_mfma<OUT>(bfr[ks], tfr, sacc);
+                                }
+                            }
+                            constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : I8F_F16;
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                float v = round_to_dtype<DT>(sacc[r]);
+                                if (g.side_has_alpha) v = round_to_dtype<DT>(v * g.side_alpha);
+                                sd[r] = v;
+                            }
+                        }
 #pragma unroll
                         for (int qd = 0; qd < 4; ++qd) {
                             const int nl = j * 32 + qd * 8 + lhalf * 4;
                             const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-                            epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value>(
-                                a4, xs, wr[0][qd], br[0][qd], ebuf + (is * 32 + l32) * PITCH + nl * OB);
+                            epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value, SIDE>(
+                                a4, xs, wr[0][qd], br[0][qd], ebuf + (is * 32 + l32) * PITCH + nl * OB, SIDE ? &sd[4 * qd] : nullptr);
                         }
                     }
                 }
@@ -641,6 +695,13 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
     g.tiles_n = (g.N + C::BN - 1) / C::BN;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
     const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);  // what the prologue wants to know of the epilogue
+    if constexpr ((OUT == OUT_BF16 || OUT == OUT_F16) && C::NT <= 512) {  // (twelve-wave tiles have no registers to spare for it)
+        if (g.side_t) {  // validated by the entry point: K % BK == 0 here
+            hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N,
+                               g.K, g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
+            return check_launch();
+        }
+    }
     if (g.K % C::BK)
         hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
                            g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
@@ -745,17 +806,21 @@ int launch(GemmArgs &g, hipStream_t st) {
             if (g.xs) sub.xs = g.xs + m0;
             sub.out = (char *)g.out + m0 * g.N * ob;
             if (g.addend) sub.addend = (const char *)g.addend + m0 * g.N * ob;
+            if (g.side_t) sub.side_t = (const char *)g.side_t + m0 * g.side_rank * 2;
             if (int rc = launch<OUT>(sub, st)) return rc;
         }
         return I8F_OK;
     }
     const bool fast = aligned && ((int64_t)g.M * g.K < (1ll << 31));
+    if (g.side_t && (!fast || g.K % 128 || (uintptr_t)g.side_t % 16 || (uintptr_t)g.side_b % 16)) return I8F_ERR_UNSUPPORTED;
     if (!fast) {
         const int64_t total = (int64_t)g.M * g.N;
         hipLaunchKernelGGL((gemm_i8_generic_kernel<OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, g);
         return check_launch();
     }
-    return launch_tile<OUT>(choose_tile(g.M, g.N), g, st);
+    Tile t = choose_tile(g.M, g.N);
+    if (g.side_t && (t == TILE_TALL || t == TILE_WIDE)) t = TILE_BIG;  // the side branch exists for the eight-wave tiles
+    return launch_tile<OUT>(t, g, st);
 }
 
 int validate(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K, const void *out) {
@@ -805,6 +870,31 @@ extern "C" int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const 
     case I8F_F16: return launch<OUT_F16>(g, st);
     default: return launch<OUT_F32>(g, st);
     }
+}
+
+extern "C" int i8f_linear_w8a8_lora(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                                    float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                                    const void *side_t, const void *side_b, int64_t rank, int has_alpha, float alpha,
+                                    void *out, int out_dtype, int64_t M, int64_t N, int64_t K, int order, void *stream) {
+    using namespace i8f;
+    if (int rc = validate(a, w, M, N, K, out)) return rc;
+    if (!valid_dtype(out_dtype) || (bias && !valid_dtype(bias_dtype))) return I8F_ERR_INVALID;
+    if (scale_mode != I8F_SCALE_TENSOR && scale_mode != I8F_SCALE_ROW) return I8F_ERR_INVALID;
+    if (order != I8F_EPI_TORCH && order != I8F_EPI_FUSED) return I8F_ERR_INVALID;
+    if (rank <= 0 || !side_t || !side_b) return I8F_ERR_INVALID;
+    if (M == 0 || N == 0) return I8F_OK;
+    if (!a_scale) return I8F_ERR_INVALID;
+    if (scale_mode == I8F_SCALE_ROW && !w_scale) return I8F_ERR_INVALID;
+    // the matrix-core side product: 16-bit operands of the output dtype, rank a multiple of 16 up to 64
+    if (out_dtype == I8F_F32 || rank % 16 || rank > 64 || K == 0) return I8F_ERR_UNSUPPORTED;
+    if (int rc = check_device()) return rc;
+    GemmArgs g{};
+    g.x = a, g.w = w, g.M = (int)M, g.N = (int)N, g.K = (int)K, g.out = out;
+    g.xs = a_scale, g.ws = w_scale, g.ws_host = w_scale_host, g.row_scale = scale_mode == I8F_SCALE_ROW;
+    g.bias = bias, g.bias_dtype = bias_dtype, g.order = order, g.addend = nullptr;
+    g.side_t = side_t, g.side_b = side_b, g.side_rank = (int)rank, g.side_has_alpha = has_alpha != 0, g.side_alpha = alpha;
+    hipStream_t st = (hipStream_t)stream;
+    return out_dtype == I8F_BF16 ? launch<OUT_BF16>(g, st) : launch<OUT_F16>(g, st);
 }
 
 extern "C" int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,

@@ -79,18 +79,19 @@ def stochastic_round_int8_delta(x: Tensor, scale, seed: int = 0, noise: Tensor |
 # --------------------------------------------------------------------------- forward functions
 @torch.no_grad()
 def int8_forward_dynamic(x: Tensor, weight: Tensor, weight_scale, bias, compute_dtype: torch.dtype,
-                         rotate: bool = False, addend: Tensor | None = None, prologue=None) -> Tensor:
+                         rotate: bool = False, addend: Tensor | None = None, prologue=None, side=None) -> Tensor:
     """Dynamic per-token activation quantisation, ONE weight scale (int8_quant.py:68-88)."""
-    return hip_int8_linear(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=prologue)
+    return hip_int8_linear(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=prologue,
+                           side=side)
 
 
 @torch.no_grad()
 def int8_forward_dynamic_per_row(x: Tensor, weight: Tensor, weight_scale: Tensor, bias,
                                  compute_dtype: torch.dtype, rotate: bool = False, addend: Tensor | None = None,
-                                 prologue=None) -> Tensor:
+                                 prologue=None, side=None) -> Tensor:
     """Dynamic per-token activation quantisation, per-row weight scales [N,1] (int8_quant.py:92-119)."""
     return hip_int8_linear_per_row(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend,
-                                   prologue=prologue)
+                                   prologue=prologue, side=side)
 
 
 # --------------------------------------------------------------------------- LoRA delta reconstruction
@@ -445,10 +446,13 @@ class Int8TensorwiseOps(manual_cast):
             rotate = bool(getattr(self, "_use_quarot", False))
 
             # Dynamic (unmerged) LoRA side branch, float; it is fed the rotated activations when QuaRot
-            # is on, as in the reference (int8_quant.py:741-744,768).  On the W8A8 path its sum with the
-            # main result happens inside the GEMM epilogue (same rounding as the reference's
+            # is on, as in the reference (int8_quant.py:741-744,768).  On the W8A8 path its second product
+            # and its sum with the main result happen inside the GEMM epilogue when the factors have the
+            # compute dtype and a rank up to 64 (no [M,N] side tensor at all); otherwise the side tensor is
+            # formed by torch and only added inside the epilogue (same rounding as the reference's
             # `y + lora_out.to(y.dtype)`, one pass over [M,N] less).
             side = None
+            side_factors = None   # (lora_x, lB, alpha): the second product happens inside the GEMM epilogue
             compiling = torch.compiler.is_compiling()
             if self.lora_A is not None and self.lora_B is not None:
                 lA = self.lora_A.to(x.device, non_blocking=True)
@@ -459,9 +463,15 @@ class Int8TensorwiseOps(manual_cast):
                     x_side = torch.ops.i8f.rotate128(x_2d)
                 else:
                     x_side = _lib.rotate128(x_2d)
-                side = F.linear(F.linear(x_side.to(lA.dtype), lA), lB)
-                if self.lora_alpha is not None:
-                    side = side * self.lora_alpha
+                lora_x = F.linear(x_side.to(lA.dtype), lA)
+                rows = x_2d.shape[0]
+                if (not compiling and rows > SMALL_BATCH_ROWS and lB.dtype == lA.dtype
+                        and _lib.lora_side_fusable(rows, weight.shape[0], weight.shape[1], lA.shape[0], compute_dtype, lA.dtype)):
+                    side_factors = (lora_x, lB, self.lora_alpha)
+                else:
+                    side = F.linear(lora_x, lB)
+                    if self.lora_alpha is not None:
+                        side = side * self.lora_alpha
 
             if x_2d.shape[0] > SMALL_BATCH_ROWS:
                 addend = None if side is None else side.to(compute_dtype)
@@ -472,7 +482,8 @@ class Int8TensorwiseOps(manual_cast):
                 else:
                     fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
                     pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift)
-                    y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=pro)
+                    y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=pro,
+                            side=side_factors)
             else:
                 # W8A16: activations keep their dtype (rotated first when the weight is rotated)
                 if compiling:

@@ -221,6 +221,28 @@ int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const int8_t *w, 
                         int order, void *stream);
 
 /*
+ * i8f_linear_w8a8 with the second product of the dynamic (unmerged) LoRA side branch
+ * computed inside the epilogue on the matrix cores:
+ *   out[m,n] = round( i8f_linear_w8a8(...)[m,n] + side[m,n] )
+ *   side     = round( round( sum_j side_t[m,j] * side_b[n,j] ) * alpha )   (the multiplication
+ *              by alpha and its rounding only if has_alpha)
+ * Replaces lora_y = F.linear(lora_x, lB); lora_y * alpha; y + lora_y.to(y.dtype) of Linear.forward
+ * (int8_quant.py:768-774): no [M,N] side tensor is written or read.  side_t = lora_x [M,rank]
+ * (the caller's first product F.linear(x, lA)), side_b = lB [N,rank], both of out_dtype and
+ * contiguous; all roundings are to out_dtype.  The sum over j is accumulated in binary32 by the
+ * matrix core; the reference's order is its BLAS library's, so results agree to the rounding of
+ * that sum (tests state the tolerance).
+ * I8F_ERR_UNSUPPORTED unless out_dtype is I8F_BF16 or I8F_F16, rank is a multiple of 16 up to 64,
+ * K is a multiple of 128 and the operands are 16-byte aligned (N % 8 == 0, K % 16 == 0): such
+ * callers use i8f_linear_w8a8_add with a side tensor instead.
+ */
+int i8f_linear_w8a8_lora(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                         float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                         const void *side_t, const void *side_b, int64_t rank, int has_alpha, float alpha,
+                         void *out, int out_dtype, int64_t M, int64_t N, int64_t K, int order,
+                         void *stream);
+
+/*
  * Small-batch W8A16 path, M <= 16: activations stay in their dtype, the int8
  * weight is dequantised on the fly.  Replaces the "small batch fallback" of
  * Linear.forward (int8_quant.py:756-760):

@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 16
+    assert len(names) == 17
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -73,6 +73,11 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_linear_w8a8(one, one, one, null, 1.0, L.SCALE_ROW, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID  # row scales missing
     assert lib.i8f_linear_w8a8(one, one, one, one, 1.0, 5, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID             # bad scale mode
     assert lib.i8f_linear_w8a8(one, one, one, one, 1.0, 0, null, 0, one, L.BF16, 4, 4, 4, 9, null) == INVALID             # bad epilogue order
+    # side branch in the epilogue: operands missing, binary32 output, rank not a multiple of 16 or above 64
+    assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, null, one, 16, 0, 0.0, one, L.BF16, 32, 32, 128, 0, null) == INVALID
+    assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 16, 0, 0.0, one, L.F32, 32, 32, 128, 0, null) == UNSUPPORTED
+    assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 24, 0, 0.0, one, L.BF16, 32, 32, 128, 0, null) == UNSUPPORTED
+    assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 80, 0, 0.0, one, L.BF16, 32, 32, 128, 0, null) == UNSUPPORTED
     assert lib.i8f_linear_w8a8(one, null, one, one, 1.0, 0, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID            # activation scales missing
     assert lib.i8f_linear_w8a8_add(one, one, one, one, 1.0, 0, null, 0, one, null, L.BF16, 4, 4, 4, 0, null) == INVALID   # no output
     assert lib.i8f_linear_w8a8_add(one, one, one, one, 1.0, 0, null, 0, one, one, 9, 4, 4, 4, 0, null) == INVALID         # bad output dtype

@@ -509,6 +509,47 @@ def test_config4_fused_merge_against_library_product_delta(L, dev):
     assert diff.max().item() <= 1 and frac <= 1e-6, f"{frac:.2e} of the merged bytes differ"
 
 
+# ------------------------------------------------------------------ dynamic LoRA side branch in the epilogue (f4)
+@pytest.mark.parametrize("M,N,K,r,dt,alpha,row", [
+    (300, 512, 256, 32, torch.bfloat16, None, True), (1000, 264, 384, 16, torch.float16, 0.5, True),
+    (4608, 3072, 3072, 32, torch.bfloat16, None, True), (512, 12288, 3072, 64, torch.bfloat16, 1.25, True),
+    (4608, 12288, 3072, 32, torch.bfloat16, None, True), (130, 96, 128, 24, torch.bfloat16, None, False),
+    (257, 3080, 640, 8, torch.float16, 2.0, True),
+])
+def test_linear_w8a8_lora_side_branch(L, dev, M, N, K, r, dt, alpha, row):
+    """out = round(y + round(round(t @ B.T) * alpha)) with the rank-r product formed inside the GEMM epilogue, against
+    (1) the same arithmetic with the product taken in float64 on the oracle's bit-exact y and (2) the unfused path
+    (torch F.linear on the device, added by i8f_linear_w8a8_add).  The matrix core accumulates the r products in binary32
+    in its own order, so a side value may round the other way now and then: results at most one ulp of the dtype
+    apart, at least 99 % identical."""
+    x = acts(M, K, dt)
+    w = i8(N, K)
+    ws = torch.rand(N if row else 1, generator=G) * 0.002 + 0.0005
+    bias = (torch.randn(N, generator=G) * 0.1).to(dt)
+    t = (torch.randn(M, r, generator=G) * 0.5).to(dt)
+    B = (torch.randn(N, r, generator=G) * 0.2).to(dt)
+    q, s = L.quant_rowwise(x.to(dev))
+    ws_arg = ws.to(dev) if row else float(ws[0])
+    got = L.linear_w8a8_lora(q, s, w.to(dev), ws_arg, bias.to(dev), t.to(dev), B.to(dev), alpha, dt)
+    side = torch.nn.functional.linear(t.to(dev), B.to(dev))
+    if alpha is not None:
+        side = side * alpha
+    unfused = L.linear_w8a8(q, s, w.to(dev), ws_arg, bias.to(dev), dt, L.EPI_TORCH, addend=side)
+    xa, code = O.from_torch(x)
+    y = O.to_f32(O.linear_w8a8(xa, code, w.numpy(), ws.numpy(), O.from_torch(bias)[0], code, code), code)
+    sd = torch.from_numpy(t.double().numpy() @ B.double().numpy().T).to(dt)
+    if alpha is not None:
+        sd = (sd.float() * alpha).to(dt)
+    want = (torch.from_numpy(y) + sd.float()).to(dt)
+    ulp = ULP[dt]
+    for ref in (want, unfused.cpu()):
+        d = (got.cpu().float() - ref.float()).abs()
+        # one ulp of the side value (it may round the other way, twice with alpha) plus one of the sum
+        bound = 2 * ulp * (2 * sd.float().abs() + ref.float().abs()) + 1e-6   # (the spacing of the dtype is up to 2 ulp * |v|)
+        assert (d <= bound).all(), f"max excess {(d - bound).max().item()} at {(d - bound).argmax().item()}"
+        assert (d != 0).float().mean().item() <= 0.01
+
+
 # ------------------------------------------------------------------ small batch W8A16 (a8)
 ULP = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-23}
 
