@@ -440,6 +440,10 @@ class Int8TensorwiseOps(manual_cast):
             w_scale = self._get_weight_scale()
             if isinstance(w_scale, Tensor) and w_scale.device != x.device:
                 w_scale = w_scale.to(x.device, non_blocking=True)
+            if isinstance(w_scale, Tensor) and not self._is_per_row and w_scale.numel() != 1:
+                # a one-scale layer whose scale tensor has several elements: element 0 counts, in eager mode and
+                # under torch.compile alike (the reference's kernel reads b_scale_ptr[0], int8_fused_kernel.py:153)
+                w_scale = w_scale.reshape(-1)[:1]
 
             compute_dtype = x.dtype if x.dtype in (torch.float16, torch.bfloat16) else torch.bfloat16
             x_2d = x.reshape(-1, x.shape[-1])

@@ -265,6 +265,10 @@ int i8f_linear_w8a16_small_m(const void *x, int x_dtype, int64_t M, int64_t K, i
  * reproduce, so the caller passes the [N,K] float noise in [0,1).
  *   dq[n,k] = int8(clamp(noise < frac(x/scale) ? floor(x/scale)+1 : floor(x/scale)))
  *   x, noise [N,K] float; scale as w_scale above; dq [N,K] int8.
+ * x / scale is a correctly rounded binary32 division, which is what torch computes for a tensor
+ * scale on any device and for a Python-float scale on the CPU; for a Python-float scale on a GPU
+ * torch multiplies by the rounded reciprocal instead, which can differ in the last bit: bit-for-bit
+ * parity is with the CPU chain.
  */
 int i8f_sr_quant_delta(const float *x, const float *scale, float scale_host, int scale_mode,
                        const float *noise, int64_t N, int64_t K, int8_t *dq, void *stream);
