@@ -170,11 +170,16 @@ def _match_modulate(node):
 def _vectors_broadcast_over_tokens(x, scale, shift) -> bool:
     """True if the traced shapes say scale/shift are [.., 1, K] (or [K]) against x [.., T, K]: one vector per
     leading index, shared by the T rows that become consecutive rows of the flattened activations."""
+    def meta(n):
+        return n.meta.get("example_value", n.meta.get("val"))
+
     def shape(n):
-        v = n.meta.get("example_value", n.meta.get("val"))
+        v = meta(n)
         return None if v is None else tuple(v.shape)
     xs, ss, ts = shape(x), shape(scale), shape(shift)
     if xs is None or ss is None or ts is None or ss != ts or len(xs) < 2:
+        return False
+    if not (meta(x).dtype == meta(scale).dtype == meta(shift).dtype):   # mixed dtypes promote in torch: leave them to it
         return False
     if len(ss) == 1:
         return ss[0] == xs[-1]
