@@ -1,844 +1,20 @@
-// int8 x int8 -> int32 "NT" GEMM on the gfx950 matrix cores with the
-// dequantisation epilogue fused in registers.
-//
-//   acc[m,n] = sum_k X[m,k] * W[n,k]         X [M,K] int8, W [N,K] int8 (K contiguous)
-//   out[m,n] = epilogue(acc, xs[m], ws[n], bias[n])
-//
-// Structure of one workgroup (a BM x BN tile of the output):
-//   * global -> LDS with buffer_load_dwordx4 ... lds (16 bytes per lane, no
-//     VGPR round trip), STAGES tiles of BK bytes in flight; rows and K-tails
-//     outside the matrices are zero-filled by the buffer bounds check.
-//   * LDS rows keep the K-contiguous layout of the operands; the 16-byte chunk
-//     index is XOR-swizzled with the row so that the 32 lanes reading one K
-//     chunk of 32 different rows hit different banks.
-//   * v_mfma_i32_32x32x32_i8, W fragments as the A operand and X fragments as
-//     the B operand, so that a lane ends up with 4 consecutive n of one m:
-//     integer sums do not depend on the order of k, so any k permutation that
-//     is the same for both operands is allowed and none has to be undone.
-//   * epilogue: scale/bias/round in registers, then a per-wave transpose
-//     through LDS so that every global store is 16 bytes per lane and covers
-//     whole 128-byte lines.
-//   * workgroup id -> tile: consecutive ids go to different XCDs (hardware
-//     round-robin), so ids are first regrouped per XCD and then walked in
-//     GROUP_M-row panels, which keeps the X and W panels a single XCD touches
-//     small enough for its own L2.
-#include <type_traits>
-
-#include "i8f_common.hpp"
-#include <algorithm>
+// Entry points of the int8 GEMM (include/i8f.h) and the instantiations for bfloat16 outputs; the other
+// output types are instantiated in gemm_i8_f16.hip and gemm_i8_wide.hip.
+#include "gemm_i8_impl.hpp"
 
 namespace i8f {
-namespace {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-enum { OUT_BF16 = 0, OUT_F16 = 1, OUT_F32 = 2, OUT_I32 = 3 };
-
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
-typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
-
-// 32 x 32 x 16 product of two 16-bit fragments (8 values per lane each) into a binary32 block
-template <int OUT>
-__device__ __forceinline__ v16f side_mfma(v4i a, v4i b, v16f c) {
-    if constexpr (OUT == OUT_BF16)
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf_t, a), __builtin_bit_cast(v8bf_t, b), c, 0, 0, 0);
-    else
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, a), __builtin_bit_cast(v8h_t, b), c, 0, 0, 0);
-}
-
-struct GemmArgs {
-    const int8_t *x;
-    const int8_t *w;
-    int M, N, K;
-    const float *xs;
-    const float *ws;
-    float ws_host;
-    int row_scale;  // 1: ws[n]; 0: one scale (ws[0] or ws_host when ws == nullptr)
-    const void *bias;
-    int bias_dtype;
-    int order;
-    const void *addend;  // nullptr or [M,N] of the output dtype, added to the rounded result
-    // low-rank side branch, side[m,n] = sum_j side_t[m,j] * side_b[n,j] (operands of the output dtype, rank % 16 == 0),
-    // rounded to that dtype, times side_alpha if side_has_alpha (rounded again), added to the rounded result
-    const void *side_t, *side_b;
-    int side_rank, side_has_alpha;
-    float side_alpha;
-    void *out;
-    int tiles_m, tiles_n;
-};
-
-// SPLIT_ (two-stage configurations): how a wave's loads of one K-tile are dealt over the phases that
-// follow the barrier which frees their stage, one hex digit per phase, first phase in the top digit
-// (0 = all of them in the first phase).
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_, int SPLIT_ = 0>
-struct Cfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_, GROUP_M = GROUP_M_;
-    static constexpr int SPLIT = SPLIT_;
-    static constexpr int NW = WM * WN;
-    static constexpr int NT = NW * 64;
-    static constexpr int WTM = BM / WM, WTN = BN / WN;  // per-wave tile
-    static constexpr int MI = WTM / 32, NI = WTN / 32;  // 32x32 MFMA blocks per wave
-    static constexpr int CPR = BK / 16;                 // 16-byte chunks per LDS row
-    static constexpr int X_BYTES = BM * BK, W_BYTES = BN * BK;
-    // every wave issues the same number of 1 KB loads per tile; a tile that does not split evenly
-    // over the waves is rounded up, and the surplus loads are out of range (they move nothing)
-    static constexpr int X_LOADS = (X_BYTES / 1024 + NW - 1) / NW, W_LOADS = (W_BYTES / 1024 + NW - 1) / NW;
-    static constexpr int X_ALLOC = X_LOADS * NW * 1024, W_ALLOC = W_LOADS * NW * 1024;
-    static constexpr int STAGE_BYTES = X_ALLOC + W_ALLOC;
-    static constexpr int LOADS = X_LOADS + W_LOADS;
-    static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
-    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
-    static_assert(X_BYTES % 1024 == 0 && W_BYTES % 1024 == 0, "tile must split into whole wave loads");
-    static_assert(BK == 64 || BK == 128, "BK");
-};
-
-// chunk swizzle: a function of the low 5 bits of the row only
-template <int CPR>
-__device__ __forceinline__ int swz(int r) {
-    if constexpr (CPR == 4) return ((r >> 1) & 3) ^ ((r >> 3) & 1);
-    else return (r ^ ((r >> 3) & 3)) & 7;
-}
-
-__device__ __forceinline__ constexpr int waitcnt_vm(int n) {
-    // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]; others left at "no wait"
-    return (n & 0xf) | (0x7 << 4) | (0xf << 8) | (((n >> 4) & 0x3) << 14);
-}
-
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-
-// One wave-wide global -> LDS load of 16 bytes per lane (lane l lands at lds_base + 16 l), issued
-// from inline assembly on purpose: the compiler knows nothing of an LDS write in flight, so it does
-// not put a full vmcnt(0) wait in front of every later LDS read (it cannot prove that the reads
-// touch another stage).  The waits for these loads are the explicit s_waitcnt of the main loop.
-__device__ __forceinline__ void dma16(v4i rsrc, uint32_t lds_base, uint32_t voffset, int soffset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
-                 : "memory", "m0");
-}
-
-__device__ __forceinline__ v4i make_rsrc(const void *p, uint32_t bytes) {
-    const uint64_t a = (uint64_t)p;
-    v4i r = {(int)(uint32_t)a, (int)((uint32_t)(a >> 32) & 0xffffu), (int)bytes, 0x00020000};
-    return r;
-}
-
-template <int OUT>
-struct OutElem {
-    static constexpr int BYTES = (OUT == OUT_BF16 || OUT == OUT_F16) ? 2 : 4;
-};
-
-// One 4-element group of the epilogue, with the operation order, the scale mode and the bias
-// fixed at compile time (a run-time test per value costs more than the arithmetic).
-template <int OUT, int ORDER, bool ROW, bool BIAS, bool SIDE = false>
-__device__ __forceinline__ void epilogue_quad(const int (&a4)[4], float xs, const float4 w4, const float4 b4,
-                                              char *dst, const float *side4 = nullptr) {
-    constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : (OUT == OUT_F16 ? I8F_F16 : I8F_F32);
-    const float wsv[4] = {w4.x, w4.y, w4.z, w4.w};
-    const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
-    float y[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const float a = (float)a4[e];
-        float t;
-        if constexpr (ORDER == I8F_EPI_TORCH) {
-            if constexpr (ROW) {
-                t = a * xs;
-                t = t * wsv[e];
-            } else {
-                const float sc = wsv[e] * xs;
-                t = a * sc;
-            }
-            t = round_to_dtype<DT>(t);
-            if constexpr (BIAS) t = t + round_to_dtype<DT>(bv[e]);
-        } else {
-            const float sc = xs * wsv[e];
-            t = a * sc;
-            if constexpr (BIAS) t = t + bv[e];
-        }
-        // the side branch is added to the ROUNDED result, as a tensor addition would (y + side.to(y.dtype))
-        if constexpr (SIDE) t = round_to_dtype<DT>(t) + side4[e];
-        y[e] = t;
-    }
-    if constexpr (OUT == OUT_BF16) {
-        *(uint2 *)dst = make_uint2(f32x2_to_bf16x2_bits(y[0], y[1]), f32x2_to_bf16x2_bits(y[2], y[3]));
-    } else if constexpr (OUT == OUT_F16) {
-        *(uint2 *)dst = make_uint2(f32x2_to_f16x2_bits(y[0], y[1]), f32x2_to_f16x2_bits(y[2], y[3]));
-    } else {
-        *(float4 *)dst = make_float4(y[0], y[1], y[2], y[3]);
-    }
-}
-
-// Eight (or four) outputs of one 16-byte piece plus the addend's, rounded once more to the output
-// dtype: what the reference's `y + side.to(y.dtype)` computes on its rounded tensors.
-template <int OUT>
-__device__ __forceinline__ uint4 add_rounded(uint4 y, uint4 s) {
-    if constexpr (OUT == OUT_F32) {
-        return make_uint4(__float_as_uint(__uint_as_float(y.x) + __uint_as_float(s.x)),
-                          __float_as_uint(__uint_as_float(y.y) + __uint_as_float(s.y)),
-                          __float_as_uint(__uint_as_float(y.z) + __uint_as_float(s.z)),
-                          __float_as_uint(__uint_as_float(y.w) + __uint_as_float(s.w)));
-    } else if constexpr (OUT == OUT_I32) {
-        return y;
-    } else {
-        const uint32_t yv[4] = {y.x, y.y, y.z, y.w}, sv[4] = {s.x, s.y, s.z, s.w};
-        uint32_t o[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            if constexpr (OUT == OUT_BF16) {
-                const float lo = bf16_bits_to_f32(yv[e] & 0xffffu) + bf16_bits_to_f32(sv[e] & 0xffffu);
-                const float hi = bf16_bits_to_f32(yv[e] >> 16) + bf16_bits_to_f32(sv[e] >> 16);
-                o[e] = f32x2_to_bf16x2_bits(lo, hi);
-            } else {
-                const float lo = f16_bits_to_f32(yv[e] & 0xffffu) + f16_bits_to_f32(sv[e] & 0xffffu);
-                const float hi = f16_bits_to_f32(yv[e] >> 16) + f16_bits_to_f32(sv[e] >> 16);
-                o[e] = f32x2_to_f16x2_bits(lo, hi);
-            }
-        }
-        return make_uint4(o[0], o[1], o[2], o[3]);
-    }
-}
-
-// KTAIL: K is not a multiple of BK (the last tile is ragged); the common case is the other kernel.
-// What the prologue needs (operand pointers, sizes, tile counts) comes first in the argument list: the
-// first 16 dwords of the kernel arguments are preloaded into SGPRs at wave launch, the rest (epilogue
-// operands) is fetched by scalar loads that have the whole main loop to land.
-template <class C, int OUT, bool KTAIL, bool SIDE = false>
-__global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
-                                                        const float *gxs, const float *gws, const void *gbias, int flags,
-                                                        const GemmArgs g) {
-    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NI = C::NI, CPR = C::CPR;
-    constexpr int S = C::STAGES;
-    constexpr int OB = OutElem<OUT>::BYTES;
-    constexpr int KS = BK / 32;  // MFMA k-steps per tile
-    static_assert(KS % 2 == 0, "fragment double-buffering alternates over an even number of k-steps");
-    // The epilogue stages EPI_STRIPS 32-row strips of a wave's tile at once (all of it for 2-byte
-    // outputs), padded so that the transposing writes do not collide on banks.
-    constexpr int ROW_BYTES = C::WTN * OB;
-    constexpr int PITCH = ROW_BYTES + (OB == 2 ? 8 : 16);
-    constexpr int EPI_STRIPS = (OB == 2 || MI == 1) ? MI : MI / 2;
-    constexpr int WAVE_BYTES = EPI_STRIPS * 32 * PITCH;
-    constexpr int SMEM_BYTES = C::LDS_BYTES > WAVE_BYTES * NW ? C::LDS_BYTES : WAVE_BYTES * NW;
-    static_assert(SMEM_BYTES + 4 * (BM + 2 * BN) <= 160 * 1024, "LDS");
-    __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
-    __shared__ float s_xs[BM], s_ws[BN], s_bias[BN];  // epilogue operands of this tile
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: lets LDS bases live in SGPRs
-    const int wm = wave / C::WN, wn = wave % C::WN;
-    const int l32 = lane & 31, lhalf = lane >> 5;
-
-    // ---- workgroup id -> output tile -------------------------------------------------
-    int tile_m, tile_n;
-    {
-        const int T = tiles_m * tiles_n;
-        const int bid = blockIdx.x;
-        const int per = (T + 7) / 8;
-        const int tall = (T % 8 == 0) ? 8 : (T % 8);
-        const int xcd = bid % 8, loc = bid / 8;
-        const int L = xcd < tall ? xcd * per + loc : tall * per + (xcd - tall) * (per - 1) + loc;
-        const int in_group = C::GROUP_M * tiles_n;
-        const int grp = L / in_group;
-        const int first_m = grp * C::GROUP_M;
-        const int gsz = min(tiles_m - first_m, C::GROUP_M);
-        const int r = L % in_group;
-        tile_m = first_m + r % gsz;
-        tile_n = r / gsz;
-    }
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    // ---- global -> LDS plan ------------------------------------------------------------
-    // One wave load moves 64 x 16 bytes into 1 KB of LDS (lane l lands at offset 16*l).  The lane
-    // decides WHICH global chunk it fetches, which is where the swizzle is applied.  The byte
-    // offset of the K-tile travels in the scalar offset of the buffer instruction, so issuing a
-    // load costs no vector arithmetic; rows beyond the matrix carry an out-of-range vector offset
-    // and are zero-filled by the buffer bounds check (which looks at the vector offset only).
-    const int K = gK;
-    const v4i rx = make_rsrc(gx, (uint32_t)((int64_t)gM * K));
-    const v4i rw = make_rsrc(gw, (uint32_t)((int64_t)gN * K));
-    const uint32_t OOB = 0x7ffffff0u;
-
-    uint32_t xoff[C::X_LOADS], woff[C::W_LOADS];  // byte offset of this lane's chunk at k-tile 0
-    int xck[C::X_LOADS], wck[C::W_LOADS];         // byte position of that chunk inside a k-tile
-#pragma unroll
-    for (int t = 0; t < C::X_LOADS; ++t) {
-        const int gidx = (t * NW + wave) * 64 + lane;
-        const int row = gidx / CPR, cl = gidx % CPR;
-        xck[t] = (cl ^ swz<CPR>(row)) * 16;
-        const int64_t grow = (int64_t)m0 + row;
-        xoff[t] = (row < BM && grow < gM) ? (uint32_t)(grow * K + xck[t]) : OOB;
-    }
-#pragma unroll
-    for (int t = 0; t < C::W_LOADS; ++t) {
-        const int gidx = (t * NW + wave) * 64 + lane;
-        const int row = gidx / CPR, cl = gidx % CPR;
-        wck[t] = (cl ^ swz<CPR>(row)) * 16;
-        const int64_t grow = (int64_t)n0 + row;
-        woff[t] = (row < BN && grow < gN) ? (uint32_t)(grow * K + wck[t]) : OOB;
-    }
-
-    const int KT = (K + BK - 1) / BK;
-
-    // `live` false (a tile index past the end, at the tail of the loop) turns every lane's offset
-    // out of range: the instruction is still issued, which keeps the loop body free of branches,
-    // but moves no data.
-    // load r of tile kt: r < X_LOADS fetches a piece of the X tile, the others a piece of the W tile
-    const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
-    auto issue_one = [&](int kt, bool live, int r) {
-        const uint32_t st = smem_base + (kt % S) * C::STAGE_BYTES + wave * 1024;
-        const int kb = kt * BK;
-        const bool is_x = r < C::X_LOADS;
-        const int t = is_x ? r : r - C::X_LOADS;
-        uint32_t vo = live ? (is_x ? xoff[t] : woff[t]) : OOB;
-        int so = kb;
-        if constexpr (KTAIL) {  // chunks past K are forced out of range per lane
-            vo = (kb + (is_x ? xck[t] : wck[t]) < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
-            so = 0;
-        }
-        dma16(is_x ? rx : rw, st + (is_x ? 0 : C::X_ALLOC) + t * NW * 1024, vo, so);
-    };
-    auto issue = [&](int kt, bool live) {
-#pragma unroll
-        for (int r = 0; r < C::LOADS; ++r) issue_one(kt, live, r);
-    };
-
-    // ---- LDS -> register plan ----------------------------------------------------------
-    const int sw = swz<CPR>(l32);
-    int koff[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) koff[ks] = ((ks * 2 + lhalf) ^ sw) * 16;
-    const int xrow_off = (wm * C::WTM + l32) * BK;
-    const int wrow_off = C::X_ALLOC + (wn * C::WTN + l32) * BK;
-
-    v16i acc[MI][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-    auto load_frags = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI]) {
-#pragma unroll
-        for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ks]);
-#pragma unroll
-        for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
-    };
-    auto mma_one = [&](const v4i (&xf)[MI], const v4i (&wf)[NI], int r) {
-        const int i = r / NI, j = r % NI;
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
-    };
-
-    // ---- prologue: S tiles in flight, fragments of the first k-step in registers --------------
-    // Two ways to keep the stages full.  With two stages a stage is refilled right after the barrier
-    // that frees it (tile kt+S from the last phase of iteration kt on), in one burst or, by the SPLIT
-    // of the configuration, over that phase and the following ones of iteration kt+1.  With three
-    // or more the refill of the stage freed by the PREVIOUS iteration is dealt out over the whole of
-    // iteration kt (tile kt+S-1): a wave that issues many loads at once blocks on the load queue, and
-    // while it is blocked it issues no MFMAs either.  Loads past the last tile are issued all the
-    // same (they move nothing), so the number of loads in flight at any point is a constant.
-    constexpr bool SPREAD_DMA = S >= 3;
-    constexpr int PRE = SPREAD_DMA ? S - 1 : S;  // tiles issued before the loop
-    // two stages: loads [cut(p), cut(p+1)) of a tile go out in the p-th phase after the barrier
-    auto cut = [](int p) constexpr {
-        if (C::SPLIT == 0) return p <= 0 ? 0 : C::LOADS;
-        int c = 0;
-        for (int q = 0; q < p && q < KS; ++q) c += (C::SPLIT >> (4 * (KS - 1 - q))) & 0xf;
-        return c;
-    };
-    static_assert(SPREAD_DMA || cut(KS) == C::LOADS, "the split has to cover every load of a tile");
-#pragma unroll
-    for (int s = 0; s < PRE; ++s) {
-        if (!SPREAD_DMA && s == PRE - 1) {
-#pragma unroll
-            for (int r = 0; r < cut(1); ++r) issue_one(s, s < KT, r);  // the rest follows inside the loop
-        } else {
-            issue(s, s < KT);
-        }
-    }
-    // ---- epilogue operands: requested behind the first tiles, parked in registers until the main loop
-    // is done.  Nothing looks at the results before the epilogue: indices are clamped instead of
-    // predicated and the conversion happens after the loop, so no instruction in between waits for
-    // them (the wait for tile 0 below counts them among the younger loads it may leave in flight, and
-    // so waits for up to three loads of tile 1 more than it has to).
-    constexpr int XS_PER = (BM + C::NT - 1) / C::NT, WS_PER = (BN + C::NT - 1) / C::NT;
-    float xs_r[XS_PER], ws_r[WS_PER];
-    uint32_t bias_r[WS_PER];
-    float ws_one = 0.0f;
-    const bool row_scale = flags & 1;
-    const int bias_dtype = flags >> 1;
-    if constexpr (OUT != OUT_I32) {
-        if (gws && !row_scale) ws_one = gws[0];
-#pragma unroll
-        for (int u = 0; u < XS_PER; ++u) xs_r[u] = gxs[min(m0 + tid + u * C::NT, gM - 1)];
-#pragma unroll
-        for (int u = 0; u < WS_PER; ++u) {
-            const int n = min(n0 + tid + u * C::NT, gN - 1);
-            ws_r[u] = row_scale ? gws[n] : 0.0f;
-            bias_r[u] = 0;
-            if (gbias) {
-                if (bias_dtype == I8F_F32) bias_r[u] = ((const uint32_t *)gbias)[n];
-                else bias_r[u] = ((const uint16_t *)gbias)[n];
-            }
-        }
-    }
-
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(SPREAD_DMA ? (PRE - 1) * C::LOADS : cut(1)));  // younger tiles may be in flight
-    __builtin_amdgcn_s_barrier();  // tile 0 is in LDS for everyone (no fence: nothing else has been written)
-
-    // Fragments are double-buffered in registers: the LDS reads of k-step s+1 are issued before
-    // the MFMAs of k-step s, so the matrix pipe does not wait for LDS.  There is one barrier per
-    // K-tile, in front of its last MFMA group: by then every wave has finished reading tile kt
-    // (its last fragments are in registers), so the stage of tile kt is refilled with tile kt+S
-    // right away, and tile kt+1 is known to have landed, so its first fragments can be fetched.
-    v4i xa[MI] = {}, wa[NI] = {}, xb[MI] = {}, wb[NI] = {};
-    if (KT > 0) load_frags(smem, 0, xa, wa);
-    // Drain scalar loads (kernel arguments) here: a scalar load still pending at the loop header
-    // would turn every LDS wait inside the loop into a full lgkmcnt(0).
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-
-    for (int kt = 0; kt < KT; ++kt) {
-        const char *st = smem + (kt % S) * C::STAGE_BYTES;
-        const char *nx = smem + ((kt + 1) % S) * C::STAGE_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const bool last = ks == KS - 1;
-            constexpr int MN = MI * NI;
-            if (last) {
-                // my part of tile kt+1 has landed and my LDS reads of tile kt have returned; what may
-                // still be in flight are the younger tiles (and, spread, the part of the newest one
-                // that the earlier phases of this iteration have issued)
-                constexpr int YOUNGER = SPREAD_DMA ? (S - 3) * C::LOADS + (KS - 1) * C::LOADS / KS : 0;
-                __builtin_amdgcn_s_waitcnt(waitcnt_vm(YOUNGER) & 0xF0FF);
-                __builtin_amdgcn_s_barrier();
-            }
-            v4i(&xc)[MI] = (ks & 1) ? xb : xa;
-            v4i(&wc)[NI] = (ks & 1) ? wb : wa;
-            v4i(&xn)[MI] = (ks & 1) ? xa : xb;
-            v4i(&wn_)[NI] = (ks & 1) ? wa : wb;
-            // past the last tile the next-fragment reads fetch stale LDS that nobody uses
-            const char *fsrc = last ? nx : st;
-            const int fks = last ? 0 : ks + 1;
-            load_frags(fsrc, fks, xn, wn_);
-            __builtin_amdgcn_sched_barrier(0);
-            // the tile being fetched: two stages refill the stage that this iteration's barrier frees
-            // (tile kt+2) from the last phase on and finish in the following phases of the next iteration
-            const int ft = SPREAD_DMA ? kt + S - 1 : (last ? kt + S : kt + S - 1);
-            const bool live = ft < KT;
-            (void)live;
-            // this phase's share of its loads
-            const int la = SPREAD_DMA ? ks * C::LOADS / KS : (last ? 0 : cut(ks + 1));
-            const int lb = SPREAD_DMA ? (ks + 1) * C::LOADS / KS : (last ? cut(1) : cut(ks + 2));
-#pragma unroll
-            for (int r = 0; r < MN; ++r) {
-                mma_one(xc, wc, r);
-#pragma unroll
-                for (int l = la + r * (lb - la) / MN; l < la + (r + 1) * (lb - la) / MN; ++l) issue_one(ft, live, l);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-
-    // ---- epilogue ----------------------------------------------------------------------
-    // The loads issued past the last tile move no data from memory but still zero-fill their LDS
-    // destination: they must have landed before the stages are reused.
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-    if constexpr (OUT != OUT_I32) {
-        if (!gws) ws_one = g.ws_host;
-#pragma unroll
-        for (int u = 0; u < XS_PER; ++u) {
-            const int t = tid + u * C::NT;
-            if (t < BM) s_xs[t] = (m0 + t < gM) ? xs_r[u] : 0.0f;
-        }
-#pragma unroll
-        for (int u = 0; u < WS_PER; ++u) {
-            const int t = tid + u * C::NT;
-            if (t < BN) {
-                const bool in = n0 + t < gN;
-                float bv = 0.0f;
-                if (gbias && in) {
-                    if (bias_dtype == I8F_F32) bv = __uint_as_float(bias_r[u]);
-                    else if (bias_dtype == I8F_BF16) bv = bf16_bits_to_f32(bias_r[u]);
-                    else bv = f16_bits_to_f32(bias_r[u]);
-                }
-                s_ws[t] = row_scale ? (in ? ws_r[u] : 0.0f) : ws_one;
-                s_bias[t] = bv;
-            }
-        }
-    }
-    __syncthreads();  // the stages are dead (reused as per-wave transpose buffers), the operands staged
-    char *ebuf = smem + wave * WAVE_BYTES;
-
-    // scale, bias, round: the flags are wave-uniform, so the variant is chosen once
-    // scale, bias, round.  The per-column operands (4 consecutive n per lane and MFMA block) are
-    // fetched from LDS into registers once, in front of the strips: fetched inside, every group of
-    // four values would wait for an LDS round trip.
-    auto convert_strip = [&](int i, char *dst_rows, const auto &wr, const auto &br, auto ORDER, auto ROW, auto BIAS) {
-        const float xs = s_xs[wm * C::WTM + i * 32 + l32];
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int nl = j * 32 + qd * 8 + lhalf * 4;  // first of 4 consecutive n held by this lane
-                const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-                epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value>(
-                    a4, xs, wr[j][qd], br[j][qd], dst_rows + l32 * PITCH + nl * OB);
-            }
-        }
-    };
-    using T_ = std::true_type;
-    using F_ = std::false_type;
-    using O0 = std::integral_constant<int, I8F_EPI_TORCH>;
-    using O1 = std::integral_constant<int, I8F_EPI_FUSED>;
-    const int variant = (g.order == I8F_EPI_FUSED ? 4 : 0) | (row_scale ? 2 : 0) | (gbias ? 1 : 0);
-
-    // The whole epilogue is instantiated once per variant and the variant is chosen ONCE, so that
-    // the instructions a wave executes are contiguous in memory (the epilogue runs once per wave,
-    // straight from a cold instruction cache).
-    // With more than 8 waves a wave has fewer registers than the accumulators plus the operands of
-    // all its columns need: the column operands are then fetched per 32-column block, and a block is
-    // converted for all staged strips before the next one is fetched.
-    // (the variant with a low-rank side branch needs registers for its operands: per-block fetches as well)
-    constexpr bool PRELOAD_ALL = C::NT <= 512 && !SIDE;
-    auto run_epilogue = [&](auto ORDER, auto ROW, auto BIAS) {
-        constexpr int NPRE = PRELOAD_ALL ? NI : 1;
-        float4 wr[NPRE][4], br[NPRE][4];
-        auto fetch_cols = [&](int j, float4 (&wj)[4], float4 (&bj)[4]) __attribute__((always_inline)) {
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int nl = wn * C::WTN + j * 32 + qd * 8 + lhalf * 4;
-                if constexpr (decltype(ROW)::value) wj[qd] = *(const float4 *)&s_ws[nl];
-                else wj[qd] = make_float4(s_ws[0], s_ws[0], s_ws[0], s_ws[0]);
-                if constexpr (decltype(BIAS)::value) bj[qd] = *(const float4 *)&s_bias[nl];
-                else bj[qd] = make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-        };
-        if constexpr (OUT != OUT_I32 && PRELOAD_ALL) {
-#pragma unroll
-            for (int j = 0; j < NI; ++j) fetch_cols(j, wr[j], br[j]);
-        }
-#pragma unroll
-        for (int i0 = 0; i0 < MI; i0 += EPI_STRIPS) {
-#pragma unroll
-            for (int is = 0; is < EPI_STRIPS; ++is) {
-                const int i = i0 + is;
-                char *rows = ebuf + is * 32 * PITCH;
-                if constexpr (OUT == OUT_I32) {
-#pragma unroll
-                    for (int j = 0; j < NI; ++j)
-#pragma unroll
-                        for (int qd = 0; qd < 4; ++qd) {
-                            const int nl = j * 32 + qd * 8 + lhalf * 4;
-                            v4i o = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-                            *(v4i *)(rows + l32 * PITCH + nl * 4) = o;
-                        }
-                } else if constexpr (PRELOAD_ALL) {
-                    convert_strip(i, rows, wr, br, ORDER, ROW, BIAS);
-                }
-            }
-            if constexpr (OUT != OUT_I32 && !PRELOAD_ALL) {
-#pragma unroll
-                for (int j = 0; j < NI; ++j) {
-                    fetch_cols(j, wr[0], br[0]);
-                    // side branch: the rank-r product of this 32 x 32 block on the matrix cores, with the same
-                    // operand roles as the main product (rows n from side_b, columns m from side_t), so that
-                    // the result has the accumulators' layout
-                    constexpr int RMAX = 64;
-                    [[maybe_unused]] v4i bfr[RMAX / 16];
-                    if constexpr (SIDE) {
-                        const int n = min(n0 + wn * C::WTN + j * 32 + l32, gN - 1);
-#pragma unroll
-                        for (int ks = 0; ks < RMAX / 16; ++ks)
-                            if (ks * 16 < g.side_rank)
-                                bfr[ks] = *(const v4i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lhalf * 8) * 2);
-                    }
-#pragma unroll
-                    for (int is = 0; is < EPI_STRIPS; ++is) {
-                        const int i = i0 + is;
-                        const float xs = s_xs[wm * C::WTM + i * 32 + l32];
-                        [[maybe_unused]] float sd[16];
-                        if constexpr (SIDE) {
-                            const int m = min(m0 + wm * C::WTM + i * 32 + l32, gM - 1);
-                            v16f sacc;
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
-#pragma unroll
-                            for (int ks = 0; ks < RMAX / 16; ++ks) {
-                                if (ks * 16 < g.side_rank) {
-                                    const v4i tfr = *(const v4i *)((const char *)g.side_t + ((int64_t)m * g.side_rank + ks * 16 + lhalf * 8) * 2);
-                                    sacc = side_mfma<OUT>(bfr[ks], tfr, sacc);
-                                }
-                            }
-                            constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : I8F_F16;
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) {
-                                float v = round_to_dtype<DT>(sacc[r]);
-                                if (g.side_has_alpha) v = round_to_dtype<DT>(v * g.side_alpha);
-                                sd[r] = v;
-                            }
-                        }
-#pragma unroll
-                        for (int qd = 0; qd < 4; ++qd) {
-                            const int nl = j * 32 + qd * 8 + lhalf * 4;
-                            const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-                            epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value, SIDE>(
-                                a4, xs, wr[0][qd], br[0][qd], ebuf + (is * 32 + l32) * PITCH + nl * OB, SIDE ? &sd[4 * qd] : nullptr);
-                        }
-                    }
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
-            // read the staged rows back row-contiguously and store 16 bytes per lane
-            constexpr int CPO = ROW_BYTES / 16;      // chunks per output row
-            constexpr int EPCO = 16 / OB;            // output elements per chunk
-            constexpr int PASSES = EPI_STRIPS * 32 * CPO / 64;
-#pragma unroll
-            for (int p = 0; p < PASSES; ++p) {
-                const int id = p * 64 + lane;
-                const int row = id / CPO, cc = id % CPO;
-                const uint4 val = *(const uint4 *)(ebuf + row * PITCH + cc * 16);
-                const int mm = m0 + wm * C::WTM + i0 * 32 + row;
-                const int nn = n0 + wn * C::WTN + cc * EPCO;
-                if (mm < gM && nn < gN)
-                {
-                    const int64_t off = ((int64_t)mm * gN + nn) * OB;
-                    uint4 v = val;
-                    if (g.addend) v = add_rounded<OUT>(v, *(const uint4 *)((const char *)g.addend + off));
-                    stream_store16((char *)g.out + off, v);
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
-        }
-    };
-    if constexpr (OUT == OUT_I32) {
-        run_epilogue(O0{}, F_{}, F_{});
-    } else {
-        switch (variant) {
-        case 0: run_epilogue(O0{}, F_{}, F_{}); break;
-        case 1: run_epilogue(O0{}, F_{}, T_{}); break;
-        case 2: run_epilogue(O0{}, T_{}, F_{}); break;
-        case 3: run_epilogue(O0{}, T_{}, T_{}); break;
-        case 4: run_epilogue(O1{}, F_{}, F_{}); break;
-        case 5: run_epilogue(O1{}, F_{}, T_{}); break;
-        case 6: run_epilogue(O1{}, T_{}, F_{}); break;
-        default: run_epilogue(O1{}, T_{}, T_{}); break;
-        }
-    }
-}
-
-// ---- slow but shape-agnostic kernel: one thread per output -----------------------------
-template <int OUT>
-__global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (int64_t)g.M * g.N) return;
-    const int m = (int)(idx / g.N), n = (int)(idx % g.N);
-    const int8_t *xr = g.x + (int64_t)m * g.K;
-    const int8_t *wr = g.w + (int64_t)n * g.K;
-    int acc = 0;
-    for (int k = 0; k < g.K; ++k) acc += (int)xr[k] * (int)wr[k];
-    if constexpr (OUT == OUT_I32) {
-        ((int *)g.out)[idx] = acc;
-    } else {
-        constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : (OUT == OUT_F16 ? I8F_F16 : I8F_F32);
-        const float xs = g.xs[m];
-        const float ws = g.ws ? g.ws[g.row_scale ? n : 0] : g.ws_host;
-        const float a = (float)acc;
-        float b = 0.0f;
-        if (g.bias) {
-            if (g.bias_dtype == I8F_F32) b = ((const float *)g.bias)[n];
-            else if (g.bias_dtype == I8F_BF16) b = bf16_bits_to_f32(((const uint16_t *)g.bias)[n]);
-            else b = f16_bits_to_f32(((const uint16_t *)g.bias)[n]);
-        }
-        float t;
-        if (g.order == I8F_EPI_TORCH) {
-            if (g.row_scale) {
-                t = a * xs;
-                t = t * ws;
-            } else {
-                const float sc = ws * xs;
-                t = a * sc;
-            }
-            t = round_to_dtype<DT>(t);
-            if (g.bias) t = t + round_to_dtype<DT>(b);
-        } else {
-            const float sc = xs * ws;
-            t = a * sc;
-            if (g.bias) t = t + b;
-        }
-        if (g.addend) t = round_to_dtype<DT>(t) + load_as_f32<DT>(g.addend, idx);
-        store_from_f32<DT>(g.out, idx, t);
-    }
-}
-
-// tile configurations
-using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400>;  // 8 waves, 2 x 64 KB stages, one workgroup per CU; refill in two halves (2-3 % faster than one burst)
-using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
-using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
-using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8>;  // 12 waves of 96 x 64, 2 x 72 KB stages
-using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8>;  // 12 waves of 64 x 96, the same transposed
-// Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
-// loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
-// flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
-using CfgW96 = Cfg<256, 96, 128, 8, 1, 3, 8>;      // 8 waves of 32 x 96, 3 x 44 KB stages
-using CfgMidDeep = Cfg<128, 128, 128, 2, 2, 4, 8>;
-using CfgM96Deep = Cfg<128, 96, 128, 4, 1, 4, 8>;
-using CfgS64Deep = Cfg<128, 64, 128, 2, 2, 4, 8>;
-using CfgT64Deep = Cfg<64, 64, 128, 2, 2, 4, 8>;
-
-template <class C, int OUT>
-int launch_cfg(GemmArgs &g, hipStream_t st) {
-    g.tiles_m = (g.M + C::BM - 1) / C::BM;
-    g.tiles_n = (g.N + C::BN - 1) / C::BN;
-    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);  // what the prologue wants to know of the epilogue
-    if constexpr ((OUT == OUT_BF16 || OUT == OUT_F16) && C::NT <= 512) {  // (twelve-wave tiles have no registers to spare for it)
-        if (g.side_t) {  // validated by the entry point: K % BK == 0 here
-            hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N,
-                               g.K, g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
-            return check_launch();
-        }
-    }
-    if (g.K % C::BK)
-        hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
-                           g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
-    else
-        hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
-                           g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
-    return check_launch();
-}
-
-enum Tile { TILE_BIG, TILE_B192, TILE_MID, TILE_TALL, TILE_WIDE, TILE_W96, TILE_MID_DEEP, TILE_M96_DEEP, TILE_S64_DEEP, TILE_T64_DEEP };
-
-// The tile configuration an M x N output takes (K does not enter).
-Tile choose_tile(int64_t M, int64_t N) {
-    // With 256-row tiles a CU holds one workgroup at a time, so a launch costs about
-    // ceil(tiles / 256 CUs) rounds of one tile's work; per operation the 256 x 192 tile is about 8 %
-    // dearer than 256 x 256 (more LDS and global->LDS traffic per MFMA) and the 288 x 256 tile of
-    // twelve waves, or 256 x 288, about 2 % (they pay where they save a round: 4608 x 12288 takes 768
-    // tiles of 288 x 256, three rounds, instead of 864 of 256 x 256, four; 4096 x 9216 takes 512 of
-    // 256 x 288, two rounds).  Outputs of fewer than 128
-    // such tiles take 128 x 128 tiles with two stages if that gives at least one workgroup per CU,
-    // else the four-stage configurations above.
-    const int64_t CUS = 256;
-    auto rounds_cost = [&](int bm, int bn, int per_op_cost) {
-        const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-        return ((tiles + CUS - 1) / CUS) * (int64_t)bm * bn * per_op_cost;
-    };
-    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-    if (big_tiles < 128) {
-        const int64_t mid_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
-        if (mid_tiles >= CUS) {
-            // Two 128 x 128 tiles to a CU fetch 2 x 256 rows per K-step, one 256 x 96 tile 352: the
-            // narrow tile wins where it still covers the output in one round (512 x 12288: 256 tiles).
-            const int64_t w96_tiles = (int64_t)((M + 255) / 256) * ((N + 95) / 96);
-            const int64_t f_w96 = ((w96_tiles + CUS - 1) / CUS) * (256 + 96);
-            const int64_t f_mid2 = ((mid_tiles + 2 * CUS - 1) / (2 * CUS)) * 2 * (128 + 128);
-            if (f_w96 < f_mid2) return TILE_W96;
-            return TILE_MID;
-        }
-        // Few tiles: the global->LDS path of a CU is what bounds these shapes, so a configuration costs
-        // the bytes its busiest CU has to fetch: (BM + BN) per K-step times the tiles that CU gets.
-        // Ties go to the larger tile (less traffic in total).
-        auto fetch_cost = [&](int bm, int bn) {
-            const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-            return ((tiles + CUS - 1) / CUS) * (bm + bn);
-        };
-        const int64_t f_mid = fetch_cost(128, 128), f_96 = fetch_cost(128, 96), f_s64 = fetch_cost(128, 64), f_t64 = fetch_cost(64, 64);
-        const int64_t f_min = std::min(std::min(f_mid, f_96), std::min(f_s64, f_t64));
-        if (f_mid == f_min) return TILE_MID_DEEP;
-        if (f_96 == f_min) return TILE_M96_DEEP;
-        if (f_s64 == f_min) return TILE_S64_DEEP;
-        return TILE_T64_DEEP;
-    }
-    const int64_t c_big = rounds_cost(256, 256, 100), c_192 = rounds_cost(256, 192, 108);
-    const int64_t c_tall = rounds_cost(288, 256, 102), c_wide = rounds_cost(256, 288, 102);
-    // 128 x 128 tiles, two workgroups to a CU: 41 % dearer per operation, but nothing is wasted on a
-    // ragged M (640 x 12288: one round of 480 of them against 192 tiles of 256 x 192)
-    const int64_t mid_all = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
-    const int64_t c_mid = ((mid_all + 2 * CUS - 1) / (2 * CUS)) * 2 * 128 * 128 * 141;
-    const int64_t c_min = std::min(std::min(std::min(c_big, c_192), std::min(c_tall, c_wide)), c_mid);
-    if (c_big == c_min) return TILE_BIG;
-    if (c_mid == c_min) return TILE_MID;
-    if (c_tall == c_min) return TILE_TALL;
-    if (c_wide == c_min) return TILE_WIDE;
-    return TILE_B192;
-}
-
-template <int OUT>
-int launch_tile(Tile t, GemmArgs &g, hipStream_t st) {
-    switch (t) {
-    case TILE_BIG: return launch_cfg<CfgBig, OUT>(g, st);
-    case TILE_B192: return launch_cfg<CfgB192, OUT>(g, st);
-    case TILE_MID: return launch_cfg<CfgMid, OUT>(g, st);
-    case TILE_TALL: return launch_cfg<CfgTall, OUT>(g, st);
-    case TILE_WIDE: return launch_cfg<CfgWide, OUT>(g, st);
-    case TILE_W96: return launch_cfg<CfgW96, OUT>(g, st);
-    case TILE_MID_DEEP: return launch_cfg<CfgMidDeep, OUT>(g, st);
-    case TILE_M96_DEEP: return launch_cfg<CfgM96Deep, OUT>(g, st);
-    case TILE_S64_DEEP: return launch_cfg<CfgS64Deep, OUT>(g, st);
-    default: return launch_cfg<CfgT64Deep, OUT>(g, st);
-    }
-}
-
-template <class C>
-void tile_dims(int *bm, int *bn, int *stages) {
-    *bm = C::BM, *bn = C::BN, *stages = C::STAGES;
-}
-
-template <int OUT>
-int launch(GemmArgs &g, hipStream_t st) {
-    const int ob = OutElem<OUT>::BYTES;
-    const bool aligned = (g.K % 16 == 0) && (g.N % 8 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
-                         ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.N * g.K < (1ll << 31)) &&
-                         (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) &&
-                         (!g.bias || (uintptr_t)g.bias % 16 == 0) && (!g.addend || (uintptr_t)g.addend % 16 == 0);
-    // The buffer descriptors address 2^31 bytes: more activations than that go in row blocks.
-    if (aligned && (int64_t)g.M * g.K >= (1ll << 31) && (int64_t)256 * g.K < (1ll << 31)) {
-        const int rows_per = (int)((((1ll << 31) - 1) / g.K) / 256 * 256);
-        for (int64_t m0 = 0; m0 < g.M; m0 += rows_per) {
-            GemmArgs sub = g;
-            sub.M = (int)(g.M - m0 < rows_per ? g.M - m0 : rows_per);
-            sub.x = g.x + m0 * g.K;
-            if (g.xs) sub.xs = g.xs + m0;
-            sub.out = (char *)g.out + m0 * g.N * ob;
-            if (g.addend) sub.addend = (const char *)g.addend + m0 * g.N * ob;
-            if (g.side_t) sub.side_t = (const char *)g.side_t + m0 * g.side_rank * 2;
-            if (int rc = launch<OUT>(sub, st)) return rc;
-        }
-        return I8F_OK;
-    }
-    const bool fast = aligned && ((int64_t)g.M * g.K < (1ll << 31));
-    if (g.side_t && (!fast || g.K % 128 || (uintptr_t)g.side_t % 16 || (uintptr_t)g.side_b % 16)) return I8F_ERR_UNSUPPORTED;
-    if (!fast) {
-        const int64_t total = (int64_t)g.M * g.N;
-        hipLaunchKernelGGL((gemm_i8_generic_kernel<OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, g);
-        return check_launch();
-    }
-    Tile t = choose_tile(g.M, g.N);
-    if (g.side_t && (t == TILE_TALL || t == TILE_WIDE)) t = TILE_BIG;  // the side branch exists for the eight-wave tiles
-    return launch_tile<OUT>(t, g, st);
-}
-
-int validate(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K, const void *out) {
-    if (M < 0 || N < 0 || K < 0) return I8F_ERR_INVALID;
-    if (M == 0 || N == 0) return I8F_OK;
-    if (!out) return I8F_ERR_INVALID;
-    if (K > 0 && (!a || !w)) return I8F_ERR_INVALID;
-    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
-    if (M * N >= (1ll << 40)) return I8F_ERR_UNSUPPORTED;
-    return I8F_OK;
-}
-
-}  // namespace
+namespace gemm {
+template int launch<OUT_BF16>(GemmArgs &, hipStream_t);
+extern template int launch<OUT_F16>(GemmArgs &, hipStream_t);
+extern template int launch<OUT_F32>(GemmArgs &, hipStream_t);
+extern template int launch<OUT_I32>(GemmArgs &, hipStream_t);
+}  // namespace gemm
 }  // namespace i8f
 
 extern "C" int i8f_gemm_i32(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K, int32_t *acc,
                             void *stream) {
     using namespace i8f;
+    using namespace i8f::gemm;
     if (int rc = validate(a, w, M, N, K, acc)) return rc;
     if (M == 0 || N == 0) return I8F_OK;
     if (int rc = check_device()) return rc;
@@ -852,6 +28,7 @@ extern "C" int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const 
                                    const void *addend, void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
                                    int order, void *stream) {
     using namespace i8f;
+    using namespace i8f::gemm;
     if (int rc = validate(a, w, M, N, K, out)) return rc;
     if (!valid_dtype(out_dtype) || (bias && !valid_dtype(bias_dtype))) return I8F_ERR_INVALID;
     if (scale_mode != I8F_SCALE_TENSOR && scale_mode != I8F_SCALE_ROW) return I8F_ERR_INVALID;
@@ -877,6 +54,7 @@ extern "C" int i8f_linear_w8a8_lora(const int8_t *a, const float *a_scale, const
                                     const void *side_t, const void *side_b, int64_t rank, int has_alpha, float alpha,
                                     void *out, int out_dtype, int64_t M, int64_t N, int64_t K, int order, void *stream) {
     using namespace i8f;
+    using namespace i8f::gemm;
     if (int rc = validate(a, w, M, N, K, out)) return rc;
     if (!valid_dtype(out_dtype) || (bias && !valid_dtype(bias_dtype))) return I8F_ERR_INVALID;
     if (scale_mode != I8F_SCALE_TENSOR && scale_mode != I8F_SCALE_ROW) return I8F_ERR_INVALID;
@@ -906,6 +84,7 @@ extern "C" int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8
 
 extern "C" int i8f_gemm_tile(int64_t M, int64_t N, int64_t K, int *bm, int *bn, int *stages) {
     using namespace i8f;
+    using namespace i8f::gemm;
     if (M <= 0 || N <= 0 || K < 0 || !bm || !bn || !stages) return I8F_ERR_INVALID;
     if (K % 16 || N % 8 || N * K >= (1ll << 31)) {  // such shapes take the one-thread-per-output kernel
         *bm = *bn = 1, *stages = 0;
