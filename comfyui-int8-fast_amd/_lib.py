@@ -95,6 +95,24 @@ def _dev(t: torch.Tensor, name: str) -> None:
         raise RuntimeError(f"{name} is on {t.device}: the INT8 engine runs on a gfx950 GPU only (no CPU path)")
 
 
+class _Nop:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NOP = _Nop()
+
+
+def _on(device):
+    """Context that makes `device` current for the call: nothing to do (and nothing to pay) when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NOP
+    return torch.cuda.device(device)
+
+
 def _ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
@@ -171,7 +189,7 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
         raise ValueError(f"unknown prologue {prologue}")
     else:
         mod_scale = mod_shift = None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         if prologue == PRO_NONE:
             _check(lib().i8f_quant_rowwise(_ptr(x), dtype_code(x.dtype), M, K, ldx, 128 if rotate else 0, _ptr(q), _ptr(s),
                                            _stream(x)), "i8f_quant_rowwise")
@@ -193,7 +211,7 @@ def quant_tensorwise(x: torch.Tensor, static_scratch: bool = False):
     n = xc.numel()
     q = torch.empty(xc.shape, dtype=torch.int8, device=x.device)
     s = torch.empty((), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         if static_scratch:
             _check(lib().i8f_quant_tensorwise_static(_ptr(xc), dtype_code(x.dtype), n, _ptr(q), _ptr(s), _stream(x)),
                    "i8f_quant_tensorwise_static")
@@ -216,7 +234,7 @@ def rotate128(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     elif out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous() or out.device != x.device:
         raise ValueError("out must be a contiguous tensor like x")
     ldx = x.stride(0) if M > 1 else K
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _check(lib().i8f_rotate128(_ptr(x), dtype_code(x.dtype), M, K, ldx, _ptr(out), _stream(x)), "i8f_rotate128")
     return out
 
@@ -243,7 +261,7 @@ def gemm_i32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     if K != K2:
         raise ValueError(f"K mismatch: a has {K}, w has {K2}")
     acc = torch.empty((M, N), dtype=torch.int32, device=a.device)
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         _check(lib().i8f_gemm_i32(_ptr(a), _ptr(w), M, N, K, _ptr(acc), _stream(a)), "i8f_gemm_i32")
     return acc
 
@@ -286,7 +304,7 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
         if addend.numel() != M * N or addend.dtype != out.dtype:
             raise ValueError(f"addend must have {M * N} elements of {out.dtype}")
         addend = addend.reshape(M, N).contiguous()
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         _check(lib().i8f_linear_w8a8_add(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
                                          _ptr(addend), _ptr(out), dtype_code(out.dtype), M, N, K, order, _stream(a)),
                "i8f_linear_w8a8_add")
@@ -332,7 +350,7 @@ def linear_w8a8_lora(a, a_scale, w, w_scale, bias, side_t, side_b, alpha=None, o
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     elif tuple(out.shape) != (M, N) or not out.is_contiguous() or out.dtype != out_dtype or out.device != a.device:
         raise ValueError(f"out must be a contiguous [{M},{N}] tensor of {out_dtype} on {a.device}")
-    with torch.cuda.device(a.device):
+    with _on(a.device):
         _check(lib().i8f_linear_w8a8_lora(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
                                           _ptr(side_t), _ptr(side_b), r, 0 if alpha is None else 1,
                                           0.0 if alpha is None else float(alpha), _ptr(out), dtype_code(out_dtype), M, N, K, order,
@@ -353,7 +371,7 @@ def linear_w8a16_small_m(x, w, w_scale, bias=None):
     bias, bcode = _bias_arg(bias, N, x.device)
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     ldx = x.stride(0) if M > 1 else K
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _check(lib().i8f_linear_w8a16_small_m(_ptr(x), dtype_code(x.dtype), M, K, ldx, _ptr(w), _ptr(ws), ws_host, mode,
                                               _ptr(bias), bcode, _ptr(out), N, _stream(x)), "i8f_linear_w8a16_small_m")
     return out
@@ -379,7 +397,7 @@ def sr_quant_delta(x, scale, noise):
     N, K = x.shape
     ws, ws_host, mode = _scale(scale, N, x.device)
     dq = torch.empty((N, K), dtype=torch.int8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _check(lib().i8f_sr_quant_delta(_ptr(x), _ptr(ws), ws_host, mode, _ptr(noise), N, K, _ptr(dq), _stream(x)),
                "i8f_sr_quant_delta")
     return dq
@@ -410,7 +428,7 @@ def lora_merge_sr(w, w_scale, noise, delta=None, up=None, down=None, lora_scale=
         out = torch.empty_like(w)
     elif out.shape != w.shape or out.dtype != torch.int8 or not out.is_contiguous():
         raise ValueError("out must be a contiguous int8 tensor like w")
-    with torch.cuda.device(w.device):
+    with _on(w.device):
         _check(lib().i8f_lora_merge_sr(_ptr(w), _ptr(ws), ws_host, mode, _ptr(delta), _ptr(up), _ptr(down), rank,
                                        float(lora_scale), _ptr(noise), N, K, _ptr(out), _stream(w)), "i8f_lora_merge_sr")
     return out
