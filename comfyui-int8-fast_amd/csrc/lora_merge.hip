@@ -1,6 +1,6 @@
 // Stochastic-rounding LoRA merge into int8 weights, one pass over HBM.
 //
-//   xs  = delta_f / w_scale                 correctly rounded division
+//   xs  = delta_f / w_scale                 correctly rounded division (sr_row: how it is obtained)
 //   f   = floor(xs);  frac = xs - f
 //   dq  = sat8(noise < frac ? f + 1 : f)    strict compare, noise supplied
 //   w'  = sat8(w + dq)
@@ -33,16 +33,92 @@ struct MergeArgs {
     int8_t *out;
 };
 
-__device__ __forceinline__ int sr_one(float delta, float sc, float noise) {
-    const float xs = delta / sc;
+// A weight row's scale with what the fast quotient below needs.
+struct RowScale {
+    float sc, rcp;
+    bool fast;
+};
+
+__device__ __forceinline__ RowScale row_scale(float sc) {
+    RowScale r;
+    r.sc = sc;
+    r.rcp = 1.0f / sc;                              // correctly rounded
+    r.fast = sc >= 0x1p-20f && sc <= 0x1p+20f;      // false for NaN
+    return r;
+}
+
+// Stochastic rounding of NE elements of one weight row: r[e] = sat8(noise < frac ? floor + 1 : floor) as a float.
+//
+// The quotient delta / sc is the correctly rounded one.  With y = RN(1/sc) computed once per row, q = delta * y followed by
+// two corrections q += RN(delta - sc q) * y (each an fma pair) gives it in five instructions instead of the division's
+// eleven: after the first correction q is within one ulp of the quotient, the remainder delta - sc q is then exact, and a
+// correction of such a q with a correctly rounded reciprocal rounds correctly (Markstein's theorem) as long as nothing
+// overflows or underflows: 2^-20 <= sc <= 2^20 and 2^-102 <= |delta| <= 2^80 make every intermediate a normal number.
+// A zero delta gives a zero quotient on either route.  A smaller non-zero delta has |quotient| < 2^-82; whatever the
+// corrections make of it (same sign or a zero of either sign, still tiny), floor and compare give the same result as
+// for the true quotient when 2^-82 <= noise < 1, which is tested on the noise's bit pattern (so NaN and negative noise
+// fail).  A NaN delta gives NaN on either route.  Lanes that fail a test redo their elements with the division.
+struct SrGuard {
+    float dmax = 0.0f;
+    uint32_t nmin = 0xffffffffu, nmax = 0u;
+    template <int NE>
+    __device__ __forceinline__ void add(const float (&delta)[NE], const float (&noise)[NE]) {
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            dmax = fmaxf(dmax, fabsf(delta[e]));
+            const uint32_t nb = __float_as_uint(noise[e]);
+            nmin = min(nmin, nb), nmax = max(nmax, nb);
+        }
+    }
+    __device__ __forceinline__ bool fast(const RowScale &rs) const {
+        return rs.fast && dmax <= 0x1p+80f && nmin >= 0x16800000u /* 2^-82 */ && nmax < 0x3f800000u /* 1 */;
+    }
+};
+
+__device__ __forceinline__ float fast_quotient(float delta, const RowScale &rs) {
+    float q = delta * rs.rcp;
+    float t = __builtin_fmaf(-rs.sc, q, delta);
+    q = __builtin_fmaf(t, rs.rcp, q);
+    t = __builtin_fmaf(-rs.sc, q, delta);
+    return __builtin_fmaf(t, rs.rcp, q);
+}
+
+__device__ __forceinline__ float sr_round(float xs, float noise) {
     const float f = floorf(xs);
     const float frac = xs - f;
-    float r = noise < frac ? f + 1.0f : f;
-    r = fminf(fmaxf(r, -128.0f), 127.0f);
-    return (int)r;
+    const float v = noise < frac ? f + 1.0f : f;
+    return fminf(fmaxf(v, -128.0f), 127.0f);  // NaN becomes -128
+}
+
+template <int NE>
+__device__ __forceinline__ void sr_row(const float (&delta)[NE], const float (&noise)[NE], const RowScale &rs, float (&r)[NE]) {
+    float xs[NE];
+    SrGuard g;
+    g.add(delta, noise);
+#pragma unroll
+    for (int e = 0; e < NE; ++e) xs[e] = fast_quotient(delta[e], rs);
+    if (__builtin_expect(!g.fast(rs), 0)) {
+#pragma unroll
+        for (int e = 0; e < NE; ++e) xs[e] = delta[e] / rs.sc;
+    }
+#pragma unroll
+    for (int e = 0; e < NE; ++e) r[e] = sr_round(xs[e], noise[e]);
 }
 
 __device__ __forceinline__ int sat8(int v) { return min(max(v, -128), 127); }
+
+// sat8(w + r) for four int8 weights packed in wp and four integer-valued r in [-128, 127], packed again.  With both
+// moved up by 128 the sum is a float in [0, 510] minus 128 and the saturating float-to-byte conversion does the clamp.
+__device__ __forceinline__ uint32_t add_sat8_pack(uint32_t wp, const float (&r)[4]) {
+    const uint32_t u = wp ^ 0x80808080u;
+    uint32_t o = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float t = (float)((u >> (8 * e)) & 0xffu) + r[e];
+        o = __builtin_amdgcn_cvt_pk_u8_f32(t, e, o);  // v_cvt_pk_u8_f32 clamps to 0..255
+    }
+    return o ^ 0x80808080u;
+}
 
 // VEC: 4 elements per thread with 16-byte loads when K % 4 == 0 and pointers are aligned, else 1
 template <int VEC, bool FUSED>
@@ -88,23 +164,13 @@ __global__ __launch_bounds__(256) void lora_merge_kernel(const MergeArgs a) {
         nz[0] = a.noise[base];
     }
 
-    int q[VEC];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) q[e] = sr_one(d[e], sc, nz[e]);
+    float r[VEC];
+    sr_row<VEC>(d, nz, row_scale(sc), r);
 
     if constexpr (VEC == 4) {
-        if (a.w) {
-            const uint32_t wp = *(const uint32_t *)(a.w + base);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) q[e] = sat8((int)(int8_t)(wp >> (8 * e)) + q[e]);
-        }
-        uint32_t o = 0;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o |= ((uint32_t)q[e] & 0xffu) << (8 * e);
-        stream_store4(a.out + base, o);
+        stream_store4(a.out + base, add_sat8_pack(a.w ? *(const uint32_t *)(a.w + base) : 0u, r));
     } else {
-        if (a.w) q[0] = sat8((int)a.w[base] + q[0]);
-        a.out[base] = (int8_t)q[0];
+        a.out[base] = (int8_t)sat8((a.w ? (int)a.w[base] : 0) + (int)r[0]);
     }
 }
 
@@ -150,14 +216,11 @@ __global__ __launch_bounds__(256) void lora_merge_band_kernel(const MergeArgs a,
             acc[3] = fmaf(u, dn[j].w, acc[3]);
         }
         const float nzv[4] = {nz_cur.x, nz_cur.y, nz_cur.z, nz_cur.w};
-        uint32_t o = 0;
+        float d[4], r[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int dq = sr_one(acc[e] * a.lora_scale, sc, nzv[e]);
-            const int wv = (int)(int8_t)(wp_cur >> (8 * e));
-            o |= ((uint32_t)sat8(wv + dq) & 0xffu) << (8 * e);
-        }
-        stream_store4(a.out + n * a.K + k0, o);
+        for (int e = 0; e < 4; ++e) d[e] = acc[e] * a.lora_scale;
+        sr_row<4>(d, nzv, row_scale(sc), r);
+        stream_store4(a.out + n * a.K + k0, add_sat8_pack(wp_cur, r));
     }
 }
 
@@ -168,14 +231,19 @@ __global__ __launch_bounds__(256) void lora_merge_band_kernel(const MergeArgs a,
 // D[k][n] = sum_j down[j][k] * up[n][j]: a lane then holds, for ONE weight row n, four groups of
 // four consecutive k, so the rounding step works on 16-byte noise and 4-byte weight pieces.
 //
-// A workgroup of 8 waves owns 256 columns and walks a band of rows in blocks of 32.  Its threads
-// fetch a block row by row (one wave instruction = 1 KB of one noise row) into an LDS tile, from
-// which every wave takes the 32 x 32 piece of its own 32 columns in the layout above; results go
-// back through the tile so that they leave in 256-byte runs.  Each wave keeps its slice of `down`
-// in RANK/2 registers; `up` is fetched once per block for all eight waves.  The operands of the
-// next block are in flight while this one is computed.
+// A workgroup of 8 waves owns 256 columns and walks a band of rows in blocks of 32.  The noise of a
+// block goes from global memory straight into one of two LDS tiles (buffer_load ... lds: a wave
+// instruction moves 1 KB of one noise row, no registers involved) while the block before it is
+// worked on; weights and `up` travel through registers.  Every wave takes the 32 x 32 piece of its
+// own 32 columns from the tiles in the layout above; results go back through the weight tile so that
+// they leave in 256-byte runs.  Each wave keeps its slice of `down` in RANK/2 registers.
+//
+// The product of block i+1 is computed while block i is rounded: the matrix instructions (64 cycles
+// each, one dependent chain) are dealt out between the vector instructions of the rounding, so a
+// wave keeps both units busy instead of using them in turn.
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef int v4i_t __attribute__((ext_vector_type(4)));
 
 template <int RANK>
 struct MfmaMergeLds {
@@ -183,105 +251,206 @@ struct MfmaMergeLds {
     static constexpr int NZ_PITCH = COLS * 4 + 16;   // 260 words: the column reads of 16 rows hit 16 different bank groups
     static constexpr int UP_PITCH = RANK * 4 + 4;
     static constexpr int WB_PITCH = COLS + 16;
-    static constexpr int NZ = 0, UP = NZ + 32 * NZ_PITCH, WB = UP + ((32 * UP_PITCH + 15) / 16) * 16;
+    static constexpr int NZ_BYTES = 32 * NZ_PITCH;
+    static constexpr int NZ = 0, UP = 2 * NZ_BYTES, WB = UP + ((32 * UP_PITCH + 15) / 16) * 16;
     static constexpr int BYTES = WB + 32 * WB_PITCH;
 };
 
+// Workgroup barrier for data exchanged through LDS only: waits for this wave's LDS operations and leaves its global
+// loads and stores in flight (__syncthreads() would wait for those as well).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// One wave-wide load of 16 bytes per lane from a buffer straight into LDS: lane l lands at lds_base + 16 l.  Bytes
+// beyond the buffer's size arrive as zeros.  The compiler does not see this load: what waits for it is an explicit
+// s_waitcnt vmcnt in the caller.
+__device__ __forceinline__ void buffer_to_lds16(v4i_t rsrc, uint32_t lds_base, uint32_t voffset, uint32_t soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory", "m0");
+}
+
+// p and bytes are the same in every lane; readfirstlane tells the compiler so (64-bit address arithmetic runs on the
+// vector ALUs and would otherwise leave the descriptor in vector registers, where a buffer instruction cannot take it).
+__device__ __forceinline__ v4i_t buffer_resource(const void *p, uint32_t bytes) {
+    const uint64_t a = (uint64_t)p;
+    v4i_t r = {__builtin_amdgcn_readfirstlane((int)(uint32_t)a), __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+               __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+    return r;
+}
+
 template <int RANK>
-__global__ __launch_bounds__(512) void lora_merge_mfma_kernel(const MergeArgs a, int blocks_per_band) {
+__global__ __launch_bounds__(512, 4) void lora_merge_mfma_kernel(const MergeArgs a, int bands) {
     using T = MfmaMergeLds<RANK>;
+    constexpr int NT = 512, P = RANK / 2;
     __shared__ __attribute__((aligned(16))) char lds[T::BYTES];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
-    const int64_t k0 = (int64_t)blockIdx.x * T::COLS;     // first column of the workgroup (K % 32 == 0 here)
-    const int64_t kbase = k0 + wave * 32;                  // first column of this wave
-    const bool wave_live = kbase < a.K;
-    float da[RANK / 2];
-#pragma unroll
-    for (int p = 0; p < RANK / 2; ++p) da[p] = wave_live ? a.down[(int64_t)(2 * p + half) * a.K + kbase + l32] : 0.0f;
-
+    // Workgroup (band, column block) takes the row blocks band, band + bands, band + 2 bands, ... of its 256 columns,
+    // so that the workgroups running at the same time read neighbouring rows.
     const int64_t nblocks = (a.N + 31) / 32;
-    const int64_t nb_begin = (int64_t)blockIdx.y * blocks_per_band;
-    const int64_t nb_end = nb_begin + blocks_per_band < nblocks ? nb_begin + blocks_per_band : nblocks;
+    const int band = blockIdx.y;
+    const int count = (int)((nblocks - band + bands - 1) / bands);
+    if (count <= 0) return;
+    auto block_of = [&](int it) { return band + (int64_t)it * bands; };
 
-    // what a thread fetches of a block: 4 pieces of noise (piece c = tid + 512 i: row c / 64, 16-byte
-    // column c % 64), one 16-byte piece of weight (row tid / 16, column tid % 16) and, threads below
-    // 8 RANK, one 16-byte piece of the contiguous 32 x RANK block of `up`
-    constexpr int UP_THREADS = 32 * RANK / 4;
-    const bool nz_col_ok = k0 + (tid & 63) * 4 < a.K, wb_col_ok = k0 + (tid & 15) * 16 < a.K;
-    auto clampn = [&](int64_t n) { return n < a.N ? n : a.N - 1; };  // rows past the end repeat the last one, unstored
-    auto fetch = [&](int64_t nb, v4f (&nz)[4], v4f &up, v4u_t &wb, float &sc) __attribute__((always_inline)) {
-        const int64_t n0 = nb * 32;
+    const int64_t k0 = (int64_t)blockIdx.x * T::COLS;      // first column of the workgroup (K % 32 == 0 here)
+    const int64_t kbase = k0 + wave * 32;                  // first column of this wave
+    float da[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) da[p] = kbase < a.K ? a.down[(int64_t)(2 * p + half) * a.K + kbase + l32] : 0.0f;
+
+    // Noise: wave w moves rows w, w + 8, w + 16, w + 24 of a block, lane l the 16 bytes at column 4 l.  The buffer
+    // starts at the block's first row and the workgroup's first column and ends with the array, so rows past N
+    // read as zeros (their results are not stored).
+    const uint32_t row_bytes = (uint32_t)a.K * 4u;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+    auto fetch_noise = [&](int64_t nb, int buf) __attribute__((always_inline)) {
+        const int64_t first = nb * 32 * a.K + k0;
+        const int64_t left = (a.N * a.K - first) * 4;
+        const v4i_t rsrc = buffer_resource(a.noise + first, left < 0xffffffffll ? (uint32_t)left : 0xffffffffu);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            if (nz_col_ok) nz[i] = *(const v4f *)(a.noise + clampn(n0 + (tid >> 6) + 8 * i) * a.K + k0 + (tid & 63) * 4);
-        if (tid < UP_THREADS) up = *(const v4f *)(a.up + clampn(n0 + tid * 4 / RANK) * RANK + (tid * 4) % RANK);
-        if (wb_col_ok) wb = *(const v4u_t *)(a.w + clampn(n0 + (tid >> 4)) * a.K + k0 + (tid & 15) * 16);
-        sc = a.ws ? a.ws[a.row_scale ? clampn(n0 + l32) : 0] : a.ws_host;
+            buffer_to_lds16(rsrc, lds_base + T::NZ + buf * T::NZ_BYTES + (wave + 8 * i) * T::NZ_PITCH, (uint32_t)lane * 16u,
+                            (uint32_t)(wave + 8 * i) * row_bytes);
     };
-
-    v4f nz_r[4] = {}, up_r = {};
-    v4u_t wb_r = {};
-    float sc_r = 1.0f;
-    if (nb_begin < nb_end) fetch(nb_begin, nz_r, up_r, wb_r, sc_r);
-    for (int64_t nb = nb_begin; nb < nb_end; ++nb) {
-        // registers -> LDS tile; the same registers then receive the next block
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *(v4f *)(lds + T::NZ + ((tid >> 6) + 8 * i) * T::NZ_PITCH + (tid & 63) * 16) = nz_r[i];
+    // Weights (one 16-byte piece per thread: row tid / 16, column 16 (tid % 16)), the row scale and, threads below
+    // 8 RANK, one 16-byte piece of the contiguous 32 x RANK block of `up`, through registers.
+    constexpr int UP_THREADS = 32 * RANK / 4;
+    static_assert(UP_THREADS <= NT, "one piece of the up block per thread");
+    const int wb_row = tid >> 4, wb_col = tid & 15;
+    const bool wb_col_ok = k0 + wb_col * 16 < a.K;
+    auto clampn = [&](int64_t n) { return n < a.N ? n : a.N - 1; };  // rows past the end repeat the last one, unstored
+    auto fetch_weights = [&](int64_t nb, v4u_t &wb, float &sc) __attribute__((always_inline)) {
+        if (wb_col_ok) wb = *(const v4u_t *)(a.w + clampn(nb * 32 + wb_row) * a.K + k0 + wb_col * 16);
+        sc = a.ws ? a.ws[a.row_scale ? clampn(nb * 32 + l32) : 0] : a.ws_host;
+    };
+    auto fetch_up = [&](int64_t nb, v4f &up) __attribute__((always_inline)) {
+        if (tid < UP_THREADS) up = *(const v4f *)(a.up + clampn(nb * 32 + tid * 4 / RANK) * RANK + (tid * 4) % RANK);
+    };
+    auto park_up = [&](const v4f &up) __attribute__((always_inline)) {
         if (tid < UP_THREADS) {
             float *dst = (float *)(lds + T::UP + (tid * 4 / RANK) * T::UP_PITCH + ((tid * 4) % RANK) * 4);
-            dst[0] = up_r.x, dst[1] = up_r.y, dst[2] = up_r.z, dst[3] = up_r.w;
+            dst[0] = up.x, dst[1] = up.y, dst[2] = up.z, dst[3] = up.w;
         }
-        *(v4u_t *)(lds + T::WB + (tid >> 4) * T::WB_PITCH + (tid & 15) * 16) = wb_r;
-        const float sc = sc_r;
-        __syncthreads();
-        if (nb + 1 < nb_end) fetch(nb + 1, nz_r, up_r, wb_r, sc_r);
+    };
+    auto up_operand = [&](int p) __attribute__((always_inline)) {
+        return *(const float *)(lds + T::UP + l32 * T::UP_PITCH + (2 * p + half) * 4);
+    };
 
-        v16f acc;
+    v4f up_r = {};
+    v4u_t wb_r = {};
+    float sc_r = 1.0f;
+    v16f acc_cur, acc_next;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int i = 0; i < 16; ++i) acc_cur[i] = 0.0f;
+    // the first block's product; every later one is computed beside the rounding of its predecessor
+    fetch_up(block_of(0), up_r);
+    fetch_noise(block_of(0), 0);
+    fetch_weights(block_of(0), wb_r, sc_r);
+    park_up(up_r);
+    fetch_up(block_of(1), up_r);
+    lds_barrier();
 #pragma unroll
-        for (int p = 0; p < RANK / 2; ++p) {
-            const float u = *(const float *)(lds + T::UP + l32 * T::UP_PITCH + (2 * p + half) * 4);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(da[p], u, acc, 0, 0, 0);
+    for (int p = 0; p < P; ++p) acc_cur = __builtin_amdgcn_mfma_f32_32x32x2f32(da[p], up_operand(p), acc_cur, 0, 0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the first block's noise is in its tile
+    lds_barrier();
+
+    for (int it = 0; it < count; ++it) {
+        const int64_t nb = block_of(it);
+        const int buf = it & 1;
+        const char *nz_tile = lds + T::NZ + buf * T::NZ_BYTES;
+        park_up(up_r);  // of the next block
+        *(v4u_t *)(lds + T::WB + wb_row * T::WB_PITCH + wb_col * 16) = wb_r;
+        const RowScale rs = row_scale(sc_r);
+        lds_barrier();  // this block's noise landed before the last barrier of the block before (or of the prologue)
+        if (it + 1 < count) {
+            fetch_noise(block_of(it + 1), buf ^ 1);
+            fetch_weights(block_of(it + 1), wb_r, sc_r);
         }
+        if (it + 2 < count) fetch_up(block_of(it + 2), up_r);
+
+        float d[16];
         uint32_t o[4];
+        SrGuard guard;
+        auto noise_quad = [&](int q, float (&nzv)[4]) __attribute__((always_inline)) {
+            const v4f nz = *(const v4f *)(nz_tile + l32 * T::NZ_PITCH + wave * 128 + (2 * q + half) * 16);
+            nzv[0] = nz.x, nzv[1] = nz.y, nzv[2] = nz.z, nzv[3] = nz.w;
+        };
+        auto weight_quad = [&](int q) __attribute__((always_inline)) {
+            return *(const uint32_t *)(lds + T::WB + l32 * T::WB_PITCH + wave * 32 + 8 * q + 4 * half);
+        };
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const v4f nz = *(const v4f *)(lds + T::NZ + l32 * T::NZ_PITCH + wave * 128 + (2 * q + half) * 16);
-            const uint32_t wp = *(const uint32_t *)(lds + T::WB + l32 * T::WB_PITCH + wave * 32 + 8 * q + 4 * half);
-            const float nzv[4] = {nz.x, nz.y, nz.z, nz.w};
-            o[q] = 0;
+        for (int q = 0; q < 4; ++q) {  // the noise is read again where it is used: sixteen registers fewer across the block
+            float nzv[4], dq[4];
+            noise_quad(q, nzv);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int dq = sr_one(acc[4 * q + e] * a.lora_scale, sc, nzv[e]);
-                const int wv = (int)(int8_t)(wp >> (8 * e));
-                o[q] |= ((uint32_t)sat8(wv + dq) & 0xffu) << (8 * e);
+            for (int e = 0; e < 4; ++e) dq[e] = d[4 * q + e] = acc_cur[4 * q + e] * a.lora_scale;
+            guard.add(dq, nzv);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc_next[i] = 0.0f;
+        if (__builtin_amdgcn_ballot_w64(!guard.fast(rs)) == 0) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int p = q * P / 4; p < (q + 1) * P / 4; ++p)
+                    acc_next = __builtin_amdgcn_mfma_f32_32x32x2f32(da[p], up_operand(p), acc_next, 0, 0, 0);
+                float r[4], nzv[4];
+                noise_quad(q, nzv);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[e] = sr_round(fast_quotient(d[4 * q + e], rs), nzv[e]);
+                o[q] = add_sat8_pack(weight_quad(q), r);
+            }
+#pragma unroll
+            for (int i = 0; i < P; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        // one matrix instruction
+                __builtin_amdgcn_sched_group_barrier(0x002, 224 / P, 0);  // its share of the vector work
+            }
+        } else {  // some lane needs the division: every lane takes it
+#pragma unroll
+            for (int p = 0; p < P; ++p) acc_next = __builtin_amdgcn_mfma_f32_32x32x2f32(da[p], up_operand(p), acc_next, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float r[4], nzv[4];
+                noise_quad(q, nzv);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[e] = sr_round(d[4 * q + e] / rs.sc, nzv[e]);
+                o[q] = add_sat8_pack(weight_quad(q), r);
             }
         }
+        acc_cur = acc_next;
         // results: back through the weight tile (each lane overwrites exactly the bytes it read),
         // then one 16-byte store per thread
 #pragma unroll
         for (int q = 0; q < 4; ++q) *(uint32_t *)(lds + T::WB + l32 * T::WB_PITCH + wave * 32 + 8 * q + 4 * half) = o[q];
-        __syncthreads();
-        const v4u_t obv = *(const v4u_t *)(lds + T::WB + (tid >> 4) * T::WB_PITCH + (tid & 15) * 16);
-        const int64_t nrow = nb * 32 + (tid >> 4);
-        if (nrow < a.N && wb_col_ok) stream_store16(a.out + nrow * a.K + k0 + (tid & 15) * 16, make_uint4(obv.x, obv.y, obv.z, obv.w));
-        __syncthreads();  // the tile is free for the next block
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next block's noise is in its tile (and this wave's last store is out)
+        lds_barrier();
+        const v4u_t obv = *(const v4u_t *)(lds + T::WB + wb_row * T::WB_PITCH + wb_col * 16);
+        const int64_t nrow = nb * 32 + wb_row;
+        if (nrow < a.N && wb_col_ok) stream_store16(a.out + nrow * a.K + k0 + wb_col * 16, make_uint4(obv.x, obv.y, obv.z, obv.w));
+        lds_barrier();  // the weight and `up` tiles are free for the next block
     }
 }
 
 template <int RANK>
 int launch_mfma(const MergeArgs &a, hipStream_t st) {
-    const unsigned col_blocks = (unsigned)((a.K + 255) / 256);
-    const int64_t nblocks = (a.N + 31) / 32;
-    const int64_t target_wgs = 256 * 12;  // short bands: several workgroups per CU take turns at the barriers
-    int64_t bands = (target_wgs + col_blocks - 1) / col_blocks;
-    int64_t per = (nblocks + bands - 1) / bands;
-    if (per < 2) per = 2;
-    bands = (nblocks + per - 1) / per;
-    if (bands > 65535) return I8F_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((lora_merge_mfma_kernel<RANK>), dim3(col_blocks, (unsigned)bands), dim3(512), 0, st, a, (int)per);
+    const int64_t col_blocks = (a.K + 255) / 256, nblocks = (a.N + 31) / 32;
+    if (col_blocks > 0x7fffffffll) return I8F_ERR_UNSUPPORTED;
+    // Two workgroups fit a CU (LDS), so 512 run at a time.  Bands are chosen for the fewest block steps on the busiest
+    // CU: rounds of 512 workgroups times the blocks of a band, plus half a step for a workgroup's start (its first
+    // product is not overlapped with anything); the smaller count wins a tie.
+    constexpr int64_t SLOTS = 512;
+    int64_t max_bands = 4 * SLOTS / col_blocks + 1;
+    if (max_bands > nblocks) max_bands = nblocks;
+    if (max_bands > 65535) max_bands = 65535;
+    int64_t bands = 1, best = -1;
+    for (int64_t b = 1; b <= max_bands; ++b) {
+        const int64_t rounds = (col_blocks * b + SLOTS - 1) / SLOTS, steps2 = 2 * ((nblocks + b - 1) / b) + 1;
+        if (best < 0 || rounds * steps2 < best) best = rounds * steps2, bands = b;
+    }
+    hipLaunchKernelGGL((lora_merge_mfma_kernel<RANK>), dim3((unsigned)col_blocks, (unsigned)bands), dim3(512), 0, st, a, (int)bands);
     return check_launch();
 }
 

@@ -268,7 +268,9 @@ int i8f_linear_w8a16_small_m(const void *x, int x_dtype, int64_t M, int64_t K, i
  * x / scale is a correctly rounded binary32 division, which is what torch computes for a tensor
  * scale on any device and for a Python-float scale on the CPU; for a Python-float scale on a GPU
  * torch multiplies by the rounded reciprocal instead, which can differ in the last bit: bit-for-bit
- * parity is with the CPU chain.
+ * parity is with the CPU chain.  (The kernels obtain the same quotient from a correctly rounded
+ * reciprocal and two fma corrections where that is exact, and divide elsewhere.)  A NaN quotient
+ * (NaN input, 0/0, inf/inf) gives -128 here; the reference converts a NaN to int8, which is undefined.
  */
 int i8f_sr_quant_delta(const float *x, const float *scale, float scale_host, int scale_mode,
                        const float *noise, int64_t N, int64_t K, int8_t *dq, void *stream);

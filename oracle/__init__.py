@@ -51,6 +51,8 @@ def lib() -> ctypes.CDLL:
         L.orc_linear_w8a16.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i64]
         L.orc_sr_delta.argtypes = [vp, vp, i32, vp, i64, i64, vp]
         L.orc_merge_i8.argtypes = [vp, vp, i64, vp]
+        L.orc_quotient_by_reciprocal_mismatches.argtypes = [vp, vp, i64, vp]
+        L.orc_quotient_by_reciprocal_mismatches.restype = i64
         L.orc_lora_delta.argtypes = [vp, vp, i64, i64, i64, f32, vp]
         L.orc_lora_merge_sr.argtypes = [vp, vp, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp]
         L.orc_fwht_f32.argtypes = [vp, i32]
@@ -276,6 +278,15 @@ def sr_delta(x, scale, noise):
     dq = np.empty((N, K), dtype=np.int8)
     _chk(lib().orc_sr_delta(_p(x), _p(scale), mode, _p(noise), N, K, _p(dq)), "sr_delta")
     return dq
+
+
+def quotient_by_reciprocal_mismatches(a, b):
+    """How many pairs the reciprocal-and-two-corrections quotient gets differently from a / b, and the first index."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    first = ctypes.c_int64(-1)
+    n = lib().orc_quotient_by_reciprocal_mismatches(_p(a), _p(b), a.size, ctypes.byref(first))
+    return int(n), int(first.value)
 
 
 def merge_i8(w, dq):

@@ -494,6 +494,30 @@ int orc_sr_delta(const float *x, const float *scale, int scale_mode, const float
 }
 
 /*
+ * Check of an arithmetic identity that the HIP merge kernels rely on (no counterpart in the reference, which
+ * divides): with y = 1/b correctly rounded, q = a*y followed by two corrections q = fma(fma(-b, q, a), y, q)
+ * is the correctly rounded a/b as long as nothing over- or underflows.  Returns how many of the n pairs
+ * disagree with the division (bit patterns compared) and stores the index of the first in *first_bad.
+ */
+int64_t orc_quotient_by_reciprocal_mismatches(const float *a, const float *b, int64_t n, int64_t *first_bad) {
+    int64_t bad = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        const float y = 1.0f / b[i];
+        float q = a[i] * y;
+        float r = fmaf(-b[i], q, a[i]);
+        q = fmaf(r, y, q);
+        r = fmaf(-b[i], q, a[i]);
+        q = fmaf(r, y, q);
+        const float t = a[i] / b[i];
+        if (memcmp(&q, &t, 4) != 0) {
+            if (bad == 0 && first_bad) *first_bad = i;
+            ++bad;
+        }
+    }
+    return bad;
+}
+
+/*
  * int8-space merge (int8_quant.py:313-316 and :399-402):
  *   w' = int8(clamp(int32(w) + int32(dq), -128, 127))
  */

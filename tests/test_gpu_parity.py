@@ -639,6 +639,51 @@ def test_lora_merge_denormal_products_bit_exact(L, dev, N, K, r):
     assert np.array_equal(fused.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("K", [256, 100, 37])
+def test_sr_quotient_shortcut_and_division_agree_on_awkward_inputs(L, dev, K):
+    """The merge kernels take delta / scale from a reciprocal and two fma corrections where that is provably the
+    correctly rounded quotient, and from the division elsewhere.  Rows of tiny, zero, huge and infinite deltas,
+    noise that is zero, denormal, negative, >= 1 or NaN, and scales outside the shortcut's range must all come out
+    as the oracle's division gives them, in the matrix-core form (K = 256), the vector form (K = 100), the
+    per-element form (K = 37) and the form that reads a given delta; weights at both ends of the int8 range
+    exercise the saturating conversion that packs the result."""
+    small = [0.0, -0.0, 1e-45, -3e-42, 1e-36, -2e-33, 7e-31, 3e-7, -0.01, 0.37, -1.5, 90.0, -200.0]
+    large = [3e20, -5e25, 1e38, float("inf"), float("-inf")]  # no NaN: the reference's conversion of a NaN to int8 is undefined
+    near, far = [1e-3, 2.5e-3, 0.25, 1.0], [3e-7, 1e-12, 2e-40, 4e6, 1e30]
+    # 64 rows that qualify for the shortcut (a wave of the matrix-core form decides for 32 rows at once), then the rest
+    rows = [(m, sc) for m in small for sc in near] + [(m, near[0]) for m in small[:12]]
+    rows += [(m, sc) for m in small for sc in far] + [(m, sc) for m in large for sc in near + far]
+    N = len(rows)
+    u = torch.tensor([r[0] for r in rows], dtype=torch.float32)
+    ws = torch.tensor([r[1] for r in rows], dtype=torch.float32)
+    v = torch.tensor([1.0, -1.0, 0.5, 3.0, 1e-3, -7.0, 0.125, 1.0 + 2.0**-23] * ((K + 7) // 8), dtype=torch.float32)[:K]
+    special = [0.0, 1e-45, 1e-30, 2.0**-82, 2.0**-83, 1 - 2.0**-24, 1.0, 1.5, -0.25, -0.0, float("nan"), 0.5]
+    noise = torch.rand(N, K, generator=G)
+    pick = torch.randint(0, 3 * len(special), (N, K), generator=G)
+    pick[:, : K // 4] = 3 * len(special)  # the first columns keep ordinary noise, so that whole waves qualify
+    for i, val in enumerate(special):
+        noise[pick == i] = val
+    w = i8(N, K)
+    w[:, ::5] = 127
+    w[:, 1::5] = -128
+    up = torch.zeros(N, 4)
+    up[:, 0] = u
+    down = torch.zeros(4, K)
+    down[0] = v
+    with np.errstate(all="ignore"):
+        want = O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), up=up.numpy(), down=down.numpy(), lora_scale=1.0)
+        delta = O.lora_delta(up.numpy(), down.numpy(), 1.0)
+        want_given = O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), delta=delta)
+        want_dq = O.sr_delta(delta, ws.numpy(), noise.numpy())
+    fused = L.lora_merge_sr(w.to(dev), ws.to(dev), noise.to(dev), up=up.to(dev), down=down.to(dev), lora_scale=1.0)
+    given = L.lora_merge_sr(w.to(dev), ws.to(dev), noise.to(dev), delta=torch.from_numpy(delta).to(dev))
+    dq = L.sr_quant_delta(torch.from_numpy(delta).to(dev), ws.to(dev), noise.to(dev))
+    assert np.array_equal(fused.cpu().numpy(), want)
+    assert np.array_equal(given.cpu().numpy(), want_given)
+    assert np.array_equal(dq.cpu().numpy(), want_dq)
+    assert len(np.unique(want_dq)) > 40  # the deltas are not all saturated or all zero
+
+
 def test_sr_special_noise_values(L, dev):
     x = torch.tensor([[0.5, 0.3, -0.3, 0.26, -0.26, 0.0, 40.0, -40.0]])
     for noise in (torch.zeros(1, 8), torch.full((1, 8), 1 - 2.0**-24), torch.tensor([[0.0, 0.2, 0.8, 0.04, 0.96, 0.5, 0.5, 0.5]])):

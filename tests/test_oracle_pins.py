@@ -364,6 +364,66 @@ def test_sr_delta_special_cases():
     assert abs(O.sr_delta(xs, scale, noise).astype(np.float64).mean() - 1.2) < 5e-3
 
 
+def test_quotient_by_reciprocal_is_the_correctly_rounded_division():
+    """The HIP merge kernels compute delta / scale as q = delta * y, twice q += fma(-scale, q, delta) * y with
+    y = 1 / scale, where 2^-20 <= scale <= 2^20 and 2^-102 <= |delta| <= 2^80 (everything else takes the division).
+    That this equals the IEEE quotient is a theorem (Markstein) for a quotient estimate within one ulp, which the
+    first correction provides; here it is checked on random operands over the whole permitted range, on mantissas at
+    the ends of a binade and, the hard cases for a correctly rounded result, on quotients that lie as close to the
+    midpoint of two neighbouring floats as two 24-bit significands allow."""
+    rng = np.random.default_rng(11)
+    n = 2_000_000
+
+    def floats(mant, expo, sign=None):
+        bits = (mant.astype(np.uint32) & 0x7FFFFF) | ((expo + 127).astype(np.uint32) << 23)
+        if sign is not None:
+            bits |= sign.astype(np.uint32) << 31
+        return bits.view(np.float32)
+
+    # random mantissas, every permitted exponent, both signs of the numerator
+    a = floats(rng.integers(0, 1 << 23, n), rng.integers(-102, 81, n), rng.integers(0, 2, n))
+    b = floats(rng.integers(0, 1 << 23, n), rng.integers(-20, 21, n))
+    assert O.quotient_by_reciprocal_mismatches(a, b) == (0, -1)
+    # mantissas next to 1 and next to 2 on either side, and numerators next to the denominator
+    edge = np.concatenate([np.arange(0, 16), np.arange((1 << 23) - 16, 1 << 23)])
+    mb = rng.choice(edge, n)
+    ma = np.where(rng.integers(0, 2, n) == 0, rng.choice(edge, n), (mb + rng.integers(-2, 3, n)) & 0x7FFFFF)
+    a = floats(ma, rng.integers(-102, 81, n), rng.integers(0, 2, n))
+    b = floats(mb, rng.integers(-20, 21, n))
+    assert O.quotient_by_reciprocal_mismatches(a, b) == (0, -1)
+    a = floats(rng.integers(0, 1 << 23, n), rng.integers(-102, 81, n))
+    assert O.quotient_by_reciprocal_mismatches(a, floats(mb, rng.integers(-20, 21, n))) == (0, -1)
+    # Quotients next to a rounding boundary.  With integer significands A, B (24 bits) and an odd 25-bit M (the
+    # midpoint of two neighbouring floats), A / B lies closest to the midpoint when A 2^s - B M = k for a small odd k,
+    # s = 24 for quotients in [1, 2) and 25 for those in [1/2, 1): M = -k / B modulo 2^s, then A follows.
+    for s_bits in (24, 25):
+        B = (rng.integers(1 << 22, 1 << 23, n).astype(np.uint64) << np.uint64(1)) | np.uint64(1)   # odd, 24 bits
+        k = rng.choice(np.array([-3, -1, 1, 3]), n)
+        mask = np.uint64((1 << s_bits) - 1)
+        inv = B.copy()
+        for _ in range(5):                                                       # Newton: inverse of B modulo 2^s
+            inv = (inv * (np.uint64(2) - B * inv)) & mask
+        assert np.all((B * inv) & mask == 1)
+        M = ((-k).astype(np.int64).astype(np.uint64) * inv) & mask
+        if s_bits == 24:
+            M = M | np.uint64(1 << 24)
+        num = (B * M).astype(np.int64) + k
+        assert np.all(num % (1 << s_bits) == 0)
+        A = num >> s_bits
+        ok = (M >= (1 << 24)) & (A >= (1 << 23)) & (A < (1 << 24))
+        assert ok.mean() > 0.2
+        A, Bk, M, k = A[ok], B[ok].astype(np.int64), M[ok].astype(np.int64), k[ok]
+        a, b = A.astype(np.float32), Bk.astype(np.float32)                       # exact: 24-bit integers
+        # distance from the midpoint in units of the quotient's ulp (2^-23 below 2, 2^-24 below 1): |k| / B
+        assert np.all(A * (1 << s_bits) - Bk * M == k) and np.abs(k / Bk).max() < 2.0**-21
+        for ea, eb in ((0, 0), (-90, 13), (70, -19)):                            # scaling by powers of two changes nothing
+            assert O.quotient_by_reciprocal_mismatches(np.ldexp(a, ea), np.ldexp(b, eb)) == (0, -1)
+            assert O.quotient_by_reciprocal_mismatches(-np.ldexp(a, ea), np.ldexp(b, eb)) == (0, -1)
+    # and the check itself can fail: one correction fewer than needed for a poor reciprocal shows up
+    bad, first = O.quotient_by_reciprocal_mismatches(np.float32([1.0, np.inf, 1e-44]), np.float32([3.0, 2.0, 3.0]))
+    assert bad >= 1 and first >= 1                         # inf and denormal numerators are outside the permitted range
+
+
 def test_merge_i8_all_pairs():
     a = np.arange(-128, 128, dtype=np.int8)
     w, dq = np.meshgrid(a, a, indexing="ij")
