@@ -440,15 +440,16 @@ int launch_mfma(const MergeArgs &a, hipStream_t st) {
     if (col_blocks > 0x7fffffffll) return I8F_ERR_UNSUPPORTED;
     // Two workgroups fit a CU (LDS), so 512 run at a time.  Bands are chosen for the fewest block steps on the busiest
     // CU: rounds of 512 workgroups times the blocks of a band, plus half a step for a workgroup's start (its first
-    // product is not overlapped with anything); the smaller count wins a tie.
+    // product is not overlapped with anything); a tie goes to fewer rounds, then to more bands (more of the chip reading).
     constexpr int64_t SLOTS = 512;
     int64_t max_bands = 4 * SLOTS / col_blocks + 1;
     if (max_bands > nblocks) max_bands = nblocks;
     if (max_bands > 65535) max_bands = 65535;
-    int64_t bands = 1, best = -1;
+    int64_t bands = 1, best = -1, best_rounds = 0;
     for (int64_t b = 1; b <= max_bands; ++b) {
         const int64_t rounds = (col_blocks * b + SLOTS - 1) / SLOTS, steps2 = 2 * ((nblocks + b - 1) / b) + 1;
-        if (best < 0 || rounds * steps2 < best) best = rounds * steps2, bands = b;
+        if (best < 0 || rounds * steps2 < best || (rounds * steps2 == best && rounds <= best_rounds))
+            best = rounds * steps2, best_rounds = rounds, bands = b;
     }
     hipLaunchKernelGGL((lora_merge_mfma_kernel<RANK>), dim3((unsigned)col_blocks, (unsigned)bands), dim3(512), 0, st, a, (int)bands);
     return check_launch();
