@@ -106,19 +106,19 @@ __device__ __forceinline__ int quant_i8(float v) {
 // Maximum over the 64 lanes of a wave, returned to every lane.  Lane exchanges are DPP operands of
 // the max instructions (no LDS round trips: the butterfly through ds_bpermute costs six dependent
 // LDS latencies): quads, half rows and rows of 16 first, then row 0 -> 1, 2 -> 3 and rows 0..1 -> 2..3
-// by the row broadcasts, which leaves the result in lane 63.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_max_step(float v) {
-    const float o = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
-    return fmaxf(v, o);
-}
+// by the row broadcasts, which leaves the result in lane 63.  One v_max_f32 with a DPP operand per
+// step, from assembly (through the builtins the compiler makes a copy, a DPP move and a maximum of
+// it).  A DPP read of a register needs two wait states after the vector write of it: the s_nop.  In
+// the last two steps the rows that receive nothing are masked out of the write and keep their value.
 __device__ __forceinline__ float wave_max(float v) {
-    v = dpp_max_step<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
-    v = dpp_max_step<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
-    v = dpp_max_step<0x141, 0xf>(v);  // row_half_mirror
-    v = dpp_max_step<0x140, 0xf>(v);  // row_mirror: every lane of a row of 16 holds the row's maximum
-    v = dpp_max_step<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_max_step<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    asm volatile("s_nop 1\n\tv_max_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+                 "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"   // every lane of a row of 16 holds the row's maximum
+                 "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"  // into rows 1 and 3
+                 "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"  // into rows 2 and 3
+                 "s_nop 1"
+                 : "+v"(v));
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 

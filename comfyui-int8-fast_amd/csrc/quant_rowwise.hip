@@ -313,34 +313,33 @@ __device__ __forceinline__ uint32_t quant4_magic(float a, float b, float c, floa
     return lo | hi;
 }
 
-// WPR waves share a row (1 or 4); each lane holds RUNS runs of 16 elements.  With WPR == 1 a wave
-// walks NROW rows (grid-strided, so that the waves running together touch neighbouring rows) and
-// fetches the next row while it reduces, scales and stores the current one: loads and stores of
-// different rows overlap inside a wave instead of every wave of the grid moving from a read phase
-// to a write phase in step.
-template <int DT, bool ROT, int WPR, int RUNS, int NROW, int PRO = I8F_PRO_NONE>
+// WPR waves share a row (1 or 4); each lane holds RUNS runs of 16 elements; one row per wave or group of
+// waves (walking several rows per wave with the next row's loads in flight measured slower at every size:
+// fewer, longer-lived waves ramp up and drain more slowly).  FULL: every lane's runs exist and every row of
+// the grid exists (K = 16 RUNS 64 WPR, M a multiple of the rows of a workgroup), so nothing is tested or
+// zero-filled: 3 % at 4608 x 3072.
+template <int DT, bool ROT, int WPR, int RUNS, bool FULL, int PRO = I8F_PRO_NONE>
 __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x, int64_t M, int64_t K,
                                                        int64_t ldx_bytes, int8_t *__restrict__ q,
                                                        float *__restrict__ scale, const Prologue pro) {
-    static_assert(WPR == 1 || NROW == 1, "rows are walked only by single-wave rows");
     constexpr int TPR = 64 * WPR;
     constexpr int ROWS = 256 / TPR;  // the workgroup has ROWS * TPR threads: 256, or 192 with three waves to a row
     const int t = threadIdx.x % TPR;
     const int rb = threadIdx.x / TPR;
-    const int64_t row_stride = (int64_t)gridDim.x * ROWS;
-    const int64_t m_first = (int64_t)blockIdx.x * ROWS + rb;
+    const int64_t m = (int64_t)blockIdx.x * ROWS + rb;
     const int nruns = (int)(K / 16);
     // run held by this lane inside its group of 8: lanes 4..7 take runs 7..4
     const int p = t ^ (((t >> 2) & 1) * 3);
     const float s0 = (p & 1) ? -1.0f : 1.0f, s1 = (p & 2) ? -1.0f : 1.0f, s2 = (p & 4) ? -1.0f : 1.0f;
 
-    auto fetch = [&](int64_t m, uint4 (&raw)[RUNS][2]) {
-        const bool ok = m < M;
+    uint4 raw[RUNS][2];
+    {
+        const bool ok = FULL || m < M;
         const char *xrow = x + (ok ? m : 0) * ldx_bytes;
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
             const int R = r * TPR + p;
-            if (ok && R < nruns) {
+            if (FULL || (ok && R < nruns)) {
                 raw[r][0] = *(const uint4 *)(xrow + (int64_t)R * 32);
                 raw[r][1] = *(const uint4 *)(xrow + (int64_t)R * 32 + 16);
             } else {
@@ -348,31 +347,24 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
                 raw[r][1] = make_uint4(0, 0, 0, 0);
             }
         }
-    };
-
-    uint4 raw[2][RUNS][2];
-    fetch(m_first, raw[0]);
-#pragma unroll
-    for (int it = 0; it < NROW; ++it) {
-        const int64_t m = m_first + it * row_stride;
-        if (it + 1 < NROW) fetch(m + row_stride, raw[(it + 1) & 1]);
-
+    }
+    {
         float v[RUNS][16];
         float amax = 0.0f;
         [[maybe_unused]] int64_t vrow = 0;  // the row's pair of modulation vectors (M < 2^31: a 32-bit division)
-        if constexpr (PRO == I8F_PRO_MODULATE) vrow = (uint32_t)(m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
+        if constexpr (PRO == I8F_PRO_MODULATE) vrow = (uint32_t)(FULL || m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
-            expand16<DT>(raw[it & 1][r][0], raw[it & 1][r][1], v[r]);
+            expand16<DT>(raw[r][0], raw[r][1], v[r]);
             if constexpr (PRO == I8F_PRO_MODULATE) {
                 // the vectors of this row's group, same 16 columns (they come from cache: every row of the group reads them)
                 const int R = r * TPR + p;
-                const int64_t off = (vrow * K + (R < nruns ? R : 0) * 16) * 2;
+                const int64_t off = (vrow * K + (FULL || R < nruns ? R : 0) * 16) * 2;
                 float sv[16], tv[16];
                 expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), sv);
                 expand16<DT>(*(const uint4 *)((const char *)pro.t + off), *(const uint4 *)((const char *)pro.t + off + 16), tv);
 #pragma unroll
-                for (int j = 0; j < 16; ++j) v[r][j] = R < nruns ? apply_prologue<DT, PRO>(v[r][j], sv[j], tv[j]) : 0.0f;
+                for (int j = 0; j < 16; ++j) v[r][j] = FULL || R < nruns ? apply_prologue<DT, PRO>(v[r][j], sv[j], tv[j]) : 0.0f;
             } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) v[r][j] = apply_prologue<DT, PRO>(v[r][j], 0.0f, 0.0f);
@@ -395,12 +387,12 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
         s = s < 1e-30f ? 1e-30f : s;
         const float inv = 1.0f / s;
 
-        if (m < M) {
+        if (FULL || m < M) {
             int8_t *qrow = q + m * K;
 #pragma unroll
             for (int r = 0; r < RUNS; ++r) {
                 const int R = r * TPR + p;
-                if (R < nruns) {
+                if (FULL || R < nruns) {
                     uint4 o;
                     o.x = quant4_magic(v[r][0], v[r][1], v[r][2], v[r][3], inv);
                     o.y = quant4_magic(v[r][4], v[r][5], v[r][6], v[r][7], inv);
@@ -416,12 +408,14 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
 
 template <int DT, bool ROT, int WPR, int RUNS, int PRO = I8F_PRO_NONE>
 int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st, const Prologue &pro = Prologue{}) {
-    // One row per wave (NROW = 1): walking several rows per wave with the next row's loads in flight
-    // measured slower at every size (fewer, longer-lived waves ramp up and drain more slowly).
     constexpr int ROWS = 256 / (64 * WPR);
     const int64_t blocks = (M + ROWS - 1) / ROWS;
-    hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, 1, PRO>), dim3((unsigned)blocks), dim3(ROWS * 64 * WPR), 0, st, (const char *)x, M, K,
-                       ldx * 2, q, scale, pro);
+    if (PRO == I8F_PRO_NONE && K == (int64_t)RUNS * 64 * WPR * 16 && M % ROWS == 0)
+        hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, PRO == I8F_PRO_NONE, PRO>), dim3((unsigned)blocks), dim3(ROWS * 64 * WPR), 0, st,
+                           (const char *)x, M, K, ldx * 2, q, scale, pro);
+    else
+        hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, false, PRO>), dim3((unsigned)blocks), dim3(ROWS * 64 * WPR), 0, st,
+                           (const char *)x, M, K, ldx * 2, q, scale, pro);
     return check_launch();
 }
 
