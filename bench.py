@@ -217,8 +217,11 @@ def extras(L, dev, quick=False):
     qbytes = M * K * 3 + 4 * M
     reps = max(5, iters // 8)
     for name, rb in (("quant_4608x3072", 0), ("rotate_quant_4608x3072", 128)):
-        def call(i, rb=rb):
-            rc = lib.i8f_quant_rowwise(ptr(xs[i]), L.BF16, M, K, K, rb, ptr(qs[i]), ptr(ss[i]), stream)
+        # argument tuples built beforehand: the launches are 7-9 us apart and the host must stay ahead of them
+        qargs = [(ptr(xs[i]), L.BF16, M, K, K, rb, ptr(qs[i]), ptr(ss[i]), stream) for i in range(sets)]
+
+        def call(i, qargs=qargs, fn=lib.i8f_quant_rowwise):
+            rc = fn(*qargs[i])
             assert rc == 0, rc
         t = time_kernel(call, reps, sets=sets, burst=sets)
         gbs = qbytes / t["median_us"] / 1e3

@@ -49,14 +49,13 @@ struct Prologue {
     int64_t rows_per_vec;    // rows that share one pair of vectors
 };
 
+// 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3), written as x / (1 + exp(-2u)): five vector instructions and the
+// hardware's exp2 and reciprocal.  exp(-2u) = exp2(x (c1 + c2 x^2)) with c1 = -2 log2(e) sqrt(2/pi), c2 = 0.044715 c1; an
+// overflow to +inf gives x * 0, an underflow to 0 gives x.  No cancellation in the negative tail, unlike 1 + tanh.
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
-    const float kBeta = 0.7978845608028654f, kKappa = 0.044715f;
-    const float x3 = x * x * x;
-    const float inner = kBeta * (x + kKappa * x3);
-    // exp(2 inner) = exp2(2 log2(e) inner); an overflow to +inf gives tanh = 1, an underflow to 0 gives -1
-    const float e = __builtin_amdgcn_exp2f(inner * 2.885390081777927f);
-    const float th = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
-    return 0.5f * x * (1.0f + th);
+    const float c1 = -2.302208198144325f, c2 = -0.1029432395800235f;
+    const float a = x * __builtin_fmaf(x * x, c2, c1);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a));
 }
 
 template <int DT, int PRO>
