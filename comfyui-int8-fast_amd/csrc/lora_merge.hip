@@ -231,7 +231,7 @@ __global__ __launch_bounds__(256) void lora_merge_band_kernel(const MergeArgs a,
 // D[k][n] = sum_j down[j][k] * up[n][j]: a lane then holds, for ONE weight row n, four groups of
 // four consecutive k, so the rounding step works on 16-byte noise and 4-byte weight pieces.
 //
-// A workgroup of 8 waves owns 256 columns and walks a band of rows in blocks of 32.  The noise of a
+// A workgroup of 8 waves owns 256 columns and walks blocks of 32 rows (every bands-th one).  The noise of a
 // block goes from global memory straight into one of two LDS tiles (buffer_load ... lds: a wave
 // instruction moves 1 KB of one noise row, no registers involved) while the block before it is
 // worked on; weights and `up` travel through registers.  Every wave takes the 32 x 32 piece of its
@@ -475,7 +475,8 @@ int run(MergeArgs &a, hipStream_t st) {
     auto al = [](const void *p, int n) { return p == nullptr || (uintptr_t)p % n == 0; };
     const bool vec = a.K % 4 == 0 && al(a.w, 4) && al(a.out, 4) && al(a.noise, 16) && al(a.delta, 16) &&
                      (!fused || al(a.down, 16));
-    if (fused && vec && a.w && a.N < (1ll << 31) && a.K % 32 == 0 && al(a.up, 16) && al(a.w, 16) && al(a.out, 16)) {
+    // (K < 2^24: the 32 rows of a block are addressed with 32-bit byte offsets from the block's first element)
+    if (fused && vec && a.w && a.N < (1ll << 31) && a.K % 32 == 0 && a.K < (1 << 24) && al(a.up, 16) && al(a.w, 16) && al(a.out, 16)) {
         switch (a.rank) {
         case 4: return launch_mfma<4>(a, st);
         case 8: return launch_mfma<8>(a, st);
