@@ -296,6 +296,29 @@ def extras(L, dev, quick=False):
                                          "tops": round(2 * 256 * Nw * Kw / t["median_us"] / 1e6, 1)}
     del noises, outs
 
+    # few tiles and a long K (the text stream's down-projection of a DiT block): the K range of a tile dealt over
+    # several workgroups through a workspace, against the same call without one; weights rotate through > 256 MB
+    Ms, Ns, Ks, nset = 512, 3072, 12288, 8
+    sq = [torch.randint(-127, 128, (Ms, Ks), dtype=torch.int8, device=dev) for _ in range(nset)]
+    sw = [torch.randint(-127, 128, (Ns, Ks), dtype=torch.int8, device=dev) for _ in range(nset)]
+    sxs, sws = torch.rand(Ms, 1, device=dev) * 0.01 + 0.001, torch.rand(Ns, device=dev) * 0.01 + 0.001
+    sy = [torch.empty(Ms, Ns, dtype=torch.bfloat16, device=dev) for _ in range(nset)]
+    work = torch.zeros(lib.i8f_linear_w8a8_workspace_bytes(), dtype=torch.uint8, device=dev)
+    sargs = [(ptr(sq[i]), ptr(sxs), ptr(sw[i]), ptr(sws), 0.0, L.SCALE_ROW, None, 0, None, ptr(sy[i]), L.BF16, Ms, Ns, Ks, L.EPI_TORCH)
+             for i in range(nset)]
+
+    def split_call(i, ws_ptr, ws_bytes):
+        rc = lib.i8f_linear_w8a8_splitk(*sargs[i], ws_ptr, ws_bytes, stream)
+        assert rc == 0, rc
+
+    t_one = time_kernel(lambda i: split_call(i, None, 0), max(10, iters // 4), sets=nset, burst=nset)
+    t_split = time_kernel(lambda i: split_call(i, ptr(work), work.numel()), max(10, iters // 4), sets=nset, burst=nset)
+    out["k_split_gemm_512x3072x12288"] = {"one_workgroup_per_tile_median_us": round(t_one["median_us"], 2),
+                                          "k_split_median_us": round(t_split["median_us"], 2),
+                                          "k_split_tops": round(2 * Ms * Ns * Ks / t_split["median_us"] / 1e6, 1),
+                                          "note": "weights from HBM (8 sets of 37.7 MB); results are bit-identical"}
+    del sq, sw, sy, work
+
     # dynamic (unmerged) LoRA side branch, rank 32, on config 1's up-projection: the second rank-r product and the
     # addition inside the GEMM epilogue, against torch's F.linear for the [M,N] side tensor + the addition in the epilogue
     Mu, Nu, Ku, r = 4608, 12288, 3072, 32

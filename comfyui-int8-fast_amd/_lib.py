@@ -63,11 +63,14 @@ def lib() -> ctypes.CDLL:
     L.i8f_gemm_tile.restype = i32
     L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
+    L.i8f_linear_w8a8_splitk.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp, i64, vp]
+    L.i8f_linear_w8a8_workspace_bytes.argtypes = []
+    L.i8f_linear_w8a8_workspace_bytes.restype = i64
     L.i8f_linear_w8a8_lora.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i64, i32, f32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_lora",
+    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -77,7 +80,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue",
-    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
 
@@ -277,6 +280,26 @@ def _bias_arg(bias, N, device):
     return bias, dtype_code(bias.dtype)
 
 
+_SPLITK_WORKSPACES = {}
+
+
+def _splitk_workspace(t: torch.Tensor, M: int, N: int, K: int):
+    """The K-split workspace of (device, current stream) for shapes that can use one (a long K and few output
+    tiles), else None.  Allocated and zeroed once; launches on one stream run one after the other, so they can share
+    it.  None while a graph is being captured and there is none yet (memory allocated during a capture belongs to
+    the graph)."""
+    if K < 10240 or M * N > 128 * 128 * 128:
+        return None
+    key = (t.device.index, torch.cuda.current_stream(t.device).cuda_stream)
+    ws = _SPLITK_WORKSPACES.get(key)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        ws = torch.zeros(lib().i8f_linear_w8a8_workspace_bytes(), dtype=torch.uint8, device=t.device)
+        _SPLITK_WORKSPACES[key] = ws
+    return ws
+
+
 def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None, addend=None):
     """Quantised activations (a int8 [M,K], a_scale [M,1]) times int8 weight [N,K] with the fused dequant epilogue.
     addend ([M,N] of the output dtype) is added to the rounded result in the epilogue and the sum rounded again."""
@@ -305,9 +328,11 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
             raise ValueError(f"addend must have {M * N} elements of {out.dtype}")
         addend = addend.reshape(M, N).contiguous()
     with _on(a.device):
-        _check(lib().i8f_linear_w8a8_add(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
-                                         _ptr(addend), _ptr(out), dtype_code(out.dtype), M, N, K, order, _stream(a)),
-               "i8f_linear_w8a8_add")
+        work = _splitk_workspace(a, M, N, K)
+        _check(lib().i8f_linear_w8a8_splitk(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
+                                            _ptr(addend), _ptr(out), dtype_code(out.dtype), M, N, K, order, _ptr(work),
+                                            0 if work is None else work.numel(), _stream(a)),
+               "i8f_linear_w8a8_splitk")
     return out
 
 

@@ -23,12 +23,23 @@ extern "C" int i8f_gemm_i32(const int8_t *a, const int8_t *w, int64_t M, int64_t
     return launch<OUT_I32>(g, (hipStream_t)stream);
 }
 
+extern "C" int64_t i8f_linear_w8a8_workspace_bytes(void) { return i8f::gemm::SPLITK_WORKSPACE_BYTES; }
+
 extern "C" int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
                                    float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
                                    const void *addend, void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
                                    int order, void *stream) {
+    return i8f_linear_w8a8_splitk(a, a_scale, w, w_scale, w_scale_host, scale_mode, bias, bias_dtype, addend, out, out_dtype, M, N,
+                                  K, order, nullptr, 0, stream);
+}
+
+extern "C" int i8f_linear_w8a8_splitk(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                                      float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                                      const void *addend, void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                      int order, void *workspace, int64_t workspace_bytes, void *stream) {
     using namespace i8f;
     using namespace i8f::gemm;
+    if (workspace && (workspace_bytes < SPLITK_WORKSPACE_BYTES || (uintptr_t)workspace % 16)) return I8F_ERR_INVALID;
     if (int rc = validate(a, w, M, N, K, out)) return rc;
     if (!valid_dtype(out_dtype) || (bias && !valid_dtype(bias_dtype))) return I8F_ERR_INVALID;
     if (scale_mode != I8F_SCALE_TENSOR && scale_mode != I8F_SCALE_ROW) return I8F_ERR_INVALID;
@@ -41,6 +52,7 @@ extern "C" int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const 
     g.x = a, g.w = w, g.M = (int)M, g.N = (int)N, g.K = (int)K, g.out = out;
     g.xs = a_scale, g.ws = w_scale, g.ws_host = w_scale_host, g.row_scale = scale_mode == I8F_SCALE_ROW;
     g.bias = bias, g.bias_dtype = bias_dtype, g.order = order, g.addend = addend;
+    if (workspace) g.arrivals = (unsigned *)workspace, g.partials = (int *)((char *)workspace + SPLITK_COUNTER_BYTES);
     hipStream_t st = (hipStream_t)stream;
     switch (out_dtype) {
     case I8F_BF16: return launch<OUT_BF16>(g, st);

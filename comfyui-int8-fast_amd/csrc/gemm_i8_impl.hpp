@@ -70,6 +70,10 @@ struct GemmArgs {
     float side_alpha;
     void *out;
     int tiles_m, tiles_n;
+    // K split over `splits` workgroups per tile (1: none): partial sums and per-tile arrival counters in caller memory
+    int splits;
+    int *partials;          // [splits][tiles][BM * BN] int32, in the register order of the kernel
+    unsigned *arrivals;     // [tiles], zero before the launch and zero again after it
 };
 
 // SPLIT_ (two-stage configurations): how a wave's loads of one K-tile are dealt over the phases that
@@ -208,7 +212,7 @@ __device__ __forceinline__ uint4 add_rounded(uint4 y, uint4 s) {
 // What the prologue needs (operand pointers, sizes, tile counts) comes first in the argument list: the
 // first 16 dwords of the kernel arguments are preloaded into SGPRs at wave launch, the rest (epilogue
 // operands) is fetched by scalar loads that have the whole main loop to land.
-template <class C, int OUT, bool KTAIL, bool SIDE = false>
+template <class C, int OUT, bool KTAIL, bool SIDE = false, bool SPLITK = false>
 __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
                                                         const float *gxs, const float *gws, const void *gbias, int flags,
                                                         const GemmArgs g) {
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     int tile_m, tile_n;
     {
         const int T = tiles_m * tiles_n;
-        const int bid = blockIdx.x;
+        const int bid = SPLITK ? __builtin_amdgcn_readfirstlane((int)blockIdx.x % T) : (int)blockIdx.x;  // the K slices of a tile are T workgroup ids apart
         const int per = (T + 7) / 8;
         const int tall = (T % 8 == 0) ? 8 : (T % 8);
         const int xcd = bid % 8, loc = bid / 8;
@@ -283,7 +287,14 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         woff[t] = (row < BN && grow < gN) ? (uint32_t)(grow * K + wck[t]) : OOB;
     }
 
-    const int KT = (K + BK - 1) / BK;
+    // SPLITK: this workgroup multiplies k-tiles [kt_first, kt_first + KT) of its output tile only
+    const int KT_all = (K + BK - 1) / BK;
+    // (integer division runs on the vector ALUs: readfirstlane brings the quotients back to scalar registers, where the
+    // K offset of the loads has to be)
+    [[maybe_unused]] const int slice = SPLITK ? __builtin_amdgcn_readfirstlane((int)blockIdx.x / (tiles_m * tiles_n)) : 0;
+    const int kt_per = SPLITK ? __builtin_amdgcn_readfirstlane((KT_all + g.splits - 1) / g.splits) : KT_all;
+    const int kt_first = slice * kt_per;
+    const int KT = SPLITK ? max(min(kt_per, KT_all - kt_first), 0) : KT_all;
 
     // `live` false (a tile index past the end, at the tail of the loop) turns every lane's offset
     // out of range: the instruction is still issued, which keeps the loop body free of branches,
@@ -292,7 +303,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
     auto issue_one = [&](int kt, bool live, int r) {
         const uint32_t st = smem_base + (kt % S) * C::STAGE_BYTES + wave * 1024;
-        const int kb = kt * BK;
+        const int kb = (kt_first + kt) * BK;
         const bool is_x = r < C::X_LOADS;
         const int t = is_x ? r : r - C::X_LOADS;
         uint32_t vo = live ? (is_x ? xoff[t] : woff[t]) : OOB;
@@ -450,6 +461,50 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // The loads issued past the last tile move no data from memory but still zero-fill their LDS
     // destination: they must have landed before the stages are reused.
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    if constexpr (SPLITK) {
+        // Every slice leaves its sums in memory (in register order: thread t of the workgroup writes 16 bytes at
+        // 16 (q NT + t) of its block for its q-th group of four) and counts itself in; the slice that arrives
+        // last adds the others' to its own and carries on into the epilogue, the others are done.  Integer sums:
+        // the order of the slices changes nothing.  Nobody waits for anybody.
+        // The sums travel with sc1 (agent-coherent) stores and loads, which go to the level where all eight L2s
+        // agree, and the count is taken once this workgroup's stores are acknowledged: no cache-wide write-back or
+        // invalidate, which a release/acquire fence pair at agent scope would cost every workgroup on the XCD.
+        __shared__ unsigned s_arrived;
+        const int T = tiles_m * tiles_n, tile = __builtin_amdgcn_readfirstlane((int)blockIdx.x % T);
+        constexpr int QUADS = MI * NI * 4;
+        int *mine = g.partials + ((int64_t)slice * T + tile) * (BM * BN);
+#pragma unroll
+        for (int qd = 0; qd < QUADS; ++qd) {
+            const int i = qd / (NI * 4), j = qd / 4 % NI, k4 = qd % 4 * 4;
+            const v4i o = {acc[i][j][k4], acc[i][j][k4 + 1], acc[i][j][k4 + 2], acc[i][j][k4 + 3]};
+            asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(mine + ((int64_t)qd * C::NT + tid) * 4), "v"(o) : "memory");
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) s_arrived = __hip_atomic_fetch_add(g.arrivals + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_arrived + 1 != (unsigned)g.splits) return;
+        for (int o = 0; o < g.splits; ++o) {
+            if (o == slice) continue;
+            const int *theirs = g.partials + ((int64_t)o * T + tile) * (BM * BN);
+#pragma unroll
+            for (int q0 = 0; q0 < QUADS; q0 += 4) {
+                v4i v[4];
+                const int *p0 = theirs + ((int64_t)q0 * C::NT + tid) * 4;
+                asm volatile("global_load_dwordx4 %0, %4, off sc1\n\tglobal_load_dwordx4 %1, %5, off sc1\n\t"
+                             "global_load_dwordx4 %2, %6, off sc1\n\tglobal_load_dwordx4 %3, %7, off sc1\n\ts_waitcnt vmcnt(0)"
+                             : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
+                             : "v"(p0), "v"(p0 + C::NT * 4), "v"(p0 + 2 * C::NT * 4), "v"(p0 + 3 * C::NT * 4)
+                             : "memory");
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int qd = q0 + u, i = qd / (NI * 4), j = qd / 4 % NI, k4 = qd % 4 * 4;
+                    acc[i][j][k4] += v[u].x, acc[i][j][k4 + 1] += v[u].y, acc[i][j][k4 + 2] += v[u].z, acc[i][j][k4 + 3] += v[u].w;
+                }
+            }
+        }
+        if (tid == 0) __hip_atomic_store(g.arrivals + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    }
     if constexpr (OUT != OUT_I32) {
         if (!gws) ws_one = g.ws_host;
 #pragma unroll
@@ -705,6 +760,18 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
             return check_launch();
         }
     }
+    if constexpr (C::STAGES == 4) {  // the K split exists for the few-tile configurations
+        if (g.splits > 1) {
+            const unsigned wgs = (unsigned)(tiles * g.splits);
+            if (g.K % C::BK)
+                hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true, false, true>), dim3(wgs), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
+                                   g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
+            else
+                hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, false, true>), dim3(wgs), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
+                                   g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
+            return check_launch();
+        }
+    }
     if (g.K % C::BK)
         hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
                            g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
@@ -771,6 +838,45 @@ inline Tile choose_tile(int64_t M, int64_t N) {
     return TILE_B192;
 }
 
+// Workspace of the K split: arrival counters (one per tile, at most 1024), then the partial sums of at most 256
+// workgroups of at most 128 x 128 outputs.
+constexpr int64_t SPLITK_COUNTER_BYTES = 4096, SPLITK_WORKSPACE_BYTES = SPLITK_COUNTER_BYTES + 256ll * 128 * 128 * 4;
+
+// Few tiles and a long K: the tile's K range is dealt over `splits` workgroups, which exchange their sums through
+// memory (integer sums, so the result is the same).  It pays where it fills idle CUs and a slice still has a long
+// loop: measured with weights from HBM, 512 x 3072 x 12288 42 -> 34 us, 256 x 3072 x 12288 33 -> 26 us,
+// 64 x 3072 x 12288 33 -> 15 us, nothing at K = 6144.  A candidate costs what its busiest CU fetches,
+// (K / splits) (BM + BN), plus 7 splits BM BN for the exchange (fitted to those measurements); one round of
+// workgroups at most, slices of at least 2048.
+inline void choose_split(int64_t M, int64_t N, int64_t K, Tile &t, int &splits) {
+    splits = 1;
+    if (K < 10240) return;
+    if (t != TILE_MID_DEEP && t != TILE_M96_DEEP && t != TILE_S64_DEEP && t != TILE_T64_DEEP) return;
+    const int64_t CUS = 256;
+    struct Cand { Tile tile; int bm, bn; };
+    const Cand cands[4] = {{TILE_MID_DEEP, 128, 128}, {TILE_M96_DEEP, 128, 96}, {TILE_S64_DEEP, 128, 64}, {TILE_T64_DEEP, 64, 64}};
+    int64_t best = -1;
+    for (const Cand &c : cands) {
+        const int64_t tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        if (c.tile == t) {
+            const int64_t cost = ((tiles + CUS - 1) / CUS) * K * (c.bm + c.bn);
+            if (best < 0 || cost < best) best = cost, splits = 1;  // (t stays)
+        }
+    }
+    Tile keep = t;
+    for (const Cand &c : cands) {
+        const int64_t tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        if (tiles > CUS / 2 || tiles > SPLITK_COUNTER_BYTES / 4) continue;
+        int64_t sp = CUS / tiles;
+        if (sp > 8) sp = 8;
+        while (sp > 1 && K / sp < 2048) --sp;
+        if (sp <= 1) continue;
+        const int64_t cost = (K / sp) * (c.bm + c.bn) + 7 * sp * c.bm * c.bn;
+        if (cost < best) best = cost, keep = c.tile, splits = (int)sp;
+    }
+    t = keep;
+}
+
 template <int OUT>
 int launch_tile(Tile t, GemmArgs &g, hipStream_t st) {
     switch (t) {
@@ -823,6 +929,9 @@ int launch(GemmArgs &g, hipStream_t st) {
     }
     Tile t = choose_tile(g.M, g.N);
     if (g.side_t && (t == TILE_TALL || t == TILE_WIDE)) t = TILE_BIG;  // the side branch exists for the eight-wave tiles
+    int splits = 1;
+    if (g.partials && !g.side_t) choose_split(g.M, g.N, g.K, t, splits);
+    g.splits = splits;
     return launch_tile<OUT>(t, g, st);
 }
 

@@ -221,6 +221,24 @@ int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const int8_t *w, 
                         int order, void *stream);
 
 /*
+ * i8f_linear_w8a8_add with a workspace, which lets outputs of few tiles and a long K (K >= 10240: a text
+ * stream's down-projection, a decode-sized batch) deal the K range of a tile over several workgroups that
+ * exchange their integer sums through the workspace.  Same arguments, same results bit for bit (integer
+ * sums do not depend on their order); the same Triton launches as i8f_linear_w8a8 (int8_fused_kernel.py:216,
+ * 357), whose grids cover the output only.  512 x 3072 x 12288 with weights from HBM: 42 -> 34 us.
+ *   workspace        device memory of i8f_linear_w8a8_workspace_bytes() bytes (16 MB + 4 KB), 16-byte aligned,
+ *                    whose first 4096 bytes are ZERO before the first call; every call leaves them zero again.
+ *                    One workspace serves any number of calls that do not overlap in time (one per stream);
+ *                    NULL gives i8f_linear_w8a8_add exactly.
+ * I8F_ERR_INVALID for a workspace that is too small or misaligned.
+ */
+int64_t i8f_linear_w8a8_workspace_bytes(void);
+int i8f_linear_w8a8_splitk(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                           float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                           const void *addend, void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                           int order, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * i8f_linear_w8a8 with the second product of the dynamic (unmerged) LoRA side branch
  * computed inside the epilogue on the matrix cores:
  *   out[m,n] = round( i8f_linear_w8a8(...)[m,n] + side[m,n] )

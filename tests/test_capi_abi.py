@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 17
+    assert len(names) == 19
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -52,6 +52,13 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_quant_rowwise(null, L.BF16, 4, 256, 256, 0, one, one, null) == INVALID    # NULL input
     assert lib.i8f_quant_rowwise(null, L.BF16, 0, 256, 256, 0, null, null, null) == 0        # empty: nothing to do
     assert lib.i8f_rotate128(one, L.F32, 4, 100, 100, one, null) == INVALID
+    # K-split workspace: too small, misaligned; the size is what the header says (16 MB + 4 KB)
+    nbytes = lib.i8f_linear_w8a8_workspace_bytes()
+    assert nbytes == 4096 + 256 * 128 * 128 * 4
+    args = (one, one, one, one, 1.0, 0, null, 0, null, one, L.BF16, 4, 8, 16, 0)
+    assert lib.i8f_linear_w8a8_splitk(*args, one, nbytes - 1, null) == INVALID
+    assert lib.i8f_linear_w8a8_splitk(*args, ctypes.c_void_p(24), nbytes, null) == INVALID
+    assert lib.i8f_linear_w8a8_splitk(one, one, one, one, 1.0, 0, null, 0, null, one, 9, 4, 8, 16, 0, one, nbytes, null) == INVALID  # bad dtype
     # quantiser with a prologue: unknown operation, modulation without its vectors or with a bad group size
     assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, 7, null, null, 1, 0, one, one, null) == INVALID
     assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, L.PRO_MODULATE, null, one, 4, 0, one, one, null) == INVALID

@@ -309,6 +309,69 @@ def test_linear_w8a8_bit_exact(L, dev, M, N, K, row, bdt, odt, order):
         assert np.array_equal(bits(got2), want)
 
 
+SPLITK_CASES = [
+    # M, N, K, output dtype: few tiles and a long K, where the tile's K range is dealt over several workgroups
+    (512, 3072, 12288, torch.bfloat16),   # 128 x 96 tiles, two slices
+    (250, 3064, 12304, torch.float16),    # ragged everywhere, K not a multiple of the 128-byte K-tile
+    (64, 3072, 12288, torch.bfloat16),    # 64 x 64 tiles, five slices of unequal length
+    (100, 1000, 16400, torch.float32),
+    (16, 12288, 10240, torch.bfloat16),   # the shortest K that is split
+]
+
+
+@pytest.mark.parametrize("M,N,K,odt", SPLITK_CASES)
+def test_linear_w8a8_k_split_bit_exact(L, dev, M, N, K, odt):
+    """Outputs of few tiles with K >= 10240 take the K split when a workspace is given (the Python layer keeps one
+    per stream): bit-equal to the oracle and to the same call without a workspace, the arrival counters are zero
+    again afterwards, and a second call on the same workspace gives the same result."""
+    x = acts(M, K)
+    wq = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=G)
+    ws = (torch.rand(N, generator=G) * 0.002 + 0.0005)
+    bias = (torch.randn(N, generator=G) * 0.01).to(torch.bfloat16)
+    xa, code = O.from_torch(x)
+    ocode = {torch.bfloat16: O.BF16, torch.float16: O.F16, torch.float32: O.F32}[odt]
+    ba, bcode = O.from_torch(bias)
+    want = O.linear_w8a8(xa, code, wq.numpy(), ws.numpy(), ba, bcode, ocode, 0, L.EPI_TORCH)
+    q, s = L.quant_rowwise(x.to(dev))
+    wd, wsd, bd = wq.to(dev), ws.to(dev), bias.to(dev)
+    got = L.linear_w8a8(q, s, wd, wsd, bd, odt, L.EPI_TORCH)
+    assert np.array_equal(bits(got), want)
+    work = L._splitk_workspace(q, M, N, K)
+    assert work is not None and int(work[:4096].view(torch.int32).abs().sum()) == 0
+    again = L.linear_w8a8(q, s, wd, wsd, bd, odt, L.EPI_TORCH)
+    assert torch.equal(again.view(torch.uint8), got.view(torch.uint8))
+    plain = torch.empty_like(got)
+    rc = L.lib().i8f_linear_w8a8(q.data_ptr(), s.data_ptr(), wd.data_ptr(), wsd.data_ptr(), 0.0, L.SCALE_ROW, bd.data_ptr(), L.BF16,
+                                 plain.data_ptr(), L.dtype_code(odt), M, N, K, L.EPI_TORCH, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.equal(plain.view(torch.uint8), got.view(torch.uint8))
+
+
+def test_linear_w8a8_long_k_under_hip_graph_equals_eager(L, dev):
+    """A shape that takes the K split in eager mode, captured in a HIP graph: the Python layer allocates no workspace
+    while a stream is capturing (the capture then runs one workgroup per tile), and with or without the split every
+    replay gives the eager result bit for bit."""
+    M, N, K = 64, 1024, 12288
+    q = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=G).to(dev)
+    w = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=G).to(dev)
+    s = (torch.rand(M, 1, generator=G) * 0.01 + 0.001).to(dev)
+    ws = (torch.rand(N, generator=G) * 0.01 + 0.001).to(dev)
+    eager = L.linear_w8a8(q, s, w, ws)
+    static_q = q.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = L.linear_w8a8(static_q, s, w, ws)
+    for i in range(3):
+        q2 = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=G).to(dev)
+        want = L.linear_w8a8(q2, s, w, ws)      # eager work (with the split) between the replays
+        torch.cuda.synchronize()
+        static_q.copy_(q2)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y.view(torch.int16), want.view(torch.int16)), f"replay {i}"
+    assert torch.equal(L.linear_w8a8(q, s, w, ws).view(torch.int16), eager.view(torch.int16))
+
+
 def test_linear_w8a8_random_shapes_and_flags(L, dev):
     """24 seeded cases over the whole range of output sizes (every tile configuration the host can pick),
     with the scale mode, bias dtype, output dtype and operation order drawn at random; K stays short so
