@@ -615,16 +615,25 @@ def test_linear_w8a8_lora_side_branch(L, dev, M, N, K, r, dt, alpha, row):
 
 # ------------------------------------------------------------------ small batch W8A16 (a8)
 ULP = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-23}
+MANT_BITS = {torch.bfloat16: 7, torch.float16: 10, torch.float32: 23}
+
+
+def spacing(v, dt):
+    """Distance between neighbouring values of dtype dt at |v| (one unit in the last place: between 2^-(p+1) and
+    2^-p of |v| for p mantissa bits, the larger just above a power of two)."""
+    a = np.maximum(np.abs(np.asarray(v, dtype=np.float64)), 2.0**-126)
+    return np.ldexp(1.0, np.floor(np.log2(a)).astype(np.int64) - MANT_BITS[dt])
 
 
 def w8a16_bound(x, wq, ws, ref, dt):
     """Per-element bound for a product of dtype-rounded operands accumulated in binary32 in any order and
-    rounded once: one ulp of the result's dtype on the result itself plus K * 2^-24 * sum_k |x||w| for the
-    accumulation (no term that scales with the largest output of the tensor)."""
+    rounded once: one unit in the last place of the result's dtype at the result (two sums on either side of a
+    rounding boundary land on neighbouring values) plus K * 2^-24 * sum_k |x||w| for the accumulation (no term
+    that scales with the largest output of the tensor)."""
     K = x.shape[1]
     wdq = (wq.float() * ws.reshape(-1, 1)).to(dt).double().abs()
     S = (x.double().abs() @ wdq.T).numpy()
-    return ULP[dt] * np.abs(ref) + K * 2.0**-24 * S + 1e-30
+    return spacing(ref, dt) + K * 2.0**-24 * S + 1e-30
 
 
 @pytest.mark.parametrize("M,N,K,dt", [
