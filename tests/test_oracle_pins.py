@@ -485,7 +485,7 @@ def test_prologue_gelu_tanh_agrees_with_torch(dt):
     xa, code = O.from_torch(x)
     got = O.to_f32(O.prologue(xa, code, O.PRO_GELU_TANH), code)
     w = want.float().numpy()
-    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-22}[dt]
+    ulp = {torch.bfloat16: 2.0**-7, torch.float16: 2.0**-10, torch.float32: 2.0**-22}[dt]   # the largest spacing relative to the value
     # far in the negative tail 1 + tanh cancels to the last bit of binary32: an absolute 2^-23 |x| on top
     assert (np.abs(got - w) <= ulp * np.abs(w) + 2.0**-23 * np.abs(x.float().numpy())).all()
     assert (got != w).mean() < (1e-2 if dt != torch.float32 else 0.5)
