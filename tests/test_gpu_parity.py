@@ -761,3 +761,55 @@ def test_sr_special_noise_values(L, dev):
     for noise in (torch.zeros(1, 8), torch.full((1, 8), 1 - 2.0**-24), torch.tensor([[0.0, 0.2, 0.8, 0.04, 0.96, 0.5, 0.5, 0.5]])):
         got = L.sr_quant_delta(x.to(dev), 0.25, noise.to(dev)).cpu().numpy()
         assert np.array_equal(got, O.sr_delta(x.numpy(), np.float32(0.25), noise.numpy()))
+
+
+# ------------------------------------------------------------------ seeded sweeps with generators of their own
+def test_lora_merge_matrix_core_form_shape_sweep(L, dev):
+    """The matrix-core merge over shapes drawn at random: row counts that leave ragged last blocks and uneven bands,
+    one to many column blocks of 256 (K a multiple of 32), every rank it takes, both scale modes."""
+    g = torch.Generator().manual_seed(4242)
+    rng = np.random.default_rng(4242)
+    for case in range(12):
+        N = int(rng.integers(1, 2600))
+        K = 32 * int(rng.integers(1, 40))
+        r = int(rng.choice([4, 8, 16, 32]))
+        row = bool(rng.integers(0, 2))
+        w = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g)
+        ws = torch.rand(N if row else 1, generator=g) * 0.002 + 0.0005
+        up, down = torch.randn(N, r, generator=g) * 0.05, torch.randn(r, K, generator=g) * 0.05
+        noise = torch.rand(N, K, generator=g)
+        scale = float(rng.choice([1.0, 0.7, -1.3]))
+        want = O.lora_merge_sr(w.numpy(), ws.numpy(), noise.numpy(), up=up.numpy(), down=down.numpy(), lora_scale=scale)
+        got = L.lora_merge_sr(w.to(dev), ws.to(dev) if row else float(ws[0]), noise.to(dev), up=up.to(dev), down=down.to(dev), lora_scale=scale)
+        assert np.array_equal(got.cpu().numpy(), want), f"case {case}: N={N} K={K} r={r} row={row}"
+
+
+def test_linear_w8a8_k_split_flags_sweep(L, dev):
+    """The K split with every epilogue flavour: tensor and row scales, with and without bias, both operation orders,
+    an addend, every output dtype; against the oracle."""
+    g = torch.Generator().manual_seed(777)
+    rng = np.random.default_rng(777)
+    dts = [torch.bfloat16, torch.float16, torch.float32]
+    for case in range(8):
+        M = int(rng.integers(17, 300))
+        N = 8 * int(rng.integers(8, 200))
+        K = 16 * int(rng.integers(640, 900))
+        row, with_bias, order = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), int(rng.integers(0, 2))
+        odt = dts[case % 3]
+        x = (torch.randn(M, K, generator=g) * 0.5).to(torch.bfloat16)
+        wq = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g)
+        ws = torch.rand(N if row else 1, generator=g) * 0.002 + 0.0005
+        bias = (torch.randn(N, generator=g) * 0.01).to(dts[(case + 1) % 3]) if with_bias else None
+        xa, code = O.from_torch(x)
+        ocode = {torch.bfloat16: O.BF16, torch.float16: O.F16, torch.float32: O.F32}[odt]
+        ba, bcode = (None, O.BF16) if bias is None else O.from_torch(bias)
+        want = O.linear_w8a8(xa, code, wq.numpy(), ws.numpy(), ba, bcode, ocode, 0, order)
+        q, s = L.quant_rowwise(x.to(dev))
+        assert L._splitk_workspace(q, M, N, K) is not None
+        got = L.linear_w8a8(q, s, wq.to(dev), ws.to(dev) if row else float(ws[0]), None if bias is None else bias.to(dev), odt, order)
+        assert np.array_equal(bits(got), want), f"case {case}: {M}x{N}x{K} row={row} bias={with_bias} order={order} {odt}"
+        if case % 2 == 0:   # and with an addend in the epilogue: bit-equal to adding it afterwards
+            add = (torch.randn(M, N, generator=g) * 0.1).to(odt).to(dev)
+            fused = L.linear_w8a8(q, s, wq.to(dev), ws.to(dev) if row else float(ws[0]), None if bias is None else bias.to(dev), odt, order, addend=add)
+            assert torch.equal(fused, (got + add).to(odt))
+
