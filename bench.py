@@ -294,7 +294,37 @@ def extras(L, dev, quick=False):
     t = time_kernel(lambda i: L.linear_w8a8(q4, s4, outs[0], w4s, None, torch.bfloat16, L.EPI_TORCH, y4), max(10, iters // 4), burst=8)
     out["skinny_gemm_256x12288x3072"] = {"median_us": round(t["median_us"], 2),
                                          "tops": round(2 * 256 * Nw * Kw / t["median_us"] / 1e6, 1)}
-    del noises, outs
+    # the load-time and patch-time forms of the same machinery, at config 4's weight shape: stochastic rounding of a
+    # given float delta alone and merged into the weights, the 128-block rotation of a float delta, the rotating
+    # quantiser on float32 weights (on-the-fly quantisation of a QuaRot layer) and the one-scale quantiser
+    nk = Nw * Kw
+    deltas = [torch.randn(Nw, Kw, device=dev) * 0.003 for _ in range(2)]
+    rot_out = torch.empty(Nw, Kw, device=dev)
+    dq = torch.empty(Nw, Kw, dtype=torch.int8, device=dev)
+    sw1 = torch.empty(Nw, 1, device=dev)
+    few = max(6, iters // 8)
+
+    def load_time(name, call, nbytes, sets=2):
+        t = time_kernel(call, few, sets=sets, burst=sets)
+        gbs = nbytes / t["median_us"] / 1e3
+        out[name] = {"median_us": round(t["median_us"], 2), "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                     "bytes": nbytes}
+
+    def chk(rc):
+        assert rc == 0, rc
+
+    load_time("sr_quant_delta_12288x3072", lambda i: chk(lib.i8f_sr_quant_delta(
+        ptr(deltas[i]), ptr(w4s_row), 0.0, L.SCALE_ROW, ptr(noises[i]), Nw, Kw, ptr(dq), stream)), nk * 9 + 4 * Nw)
+    load_time("lora_merge_given_delta_12288x3072", lambda i: chk(lib.i8f_lora_merge_sr(
+        ptr(w4q), ptr(w4s_row), 0.0, L.SCALE_ROW, ptr(deltas[i]), None, None, 0, 1.0, ptr(noises[i]), Nw, Kw, ptr(outs[i]), stream)),
+        nk * 10 + 4 * Nw)
+    load_time("rotate128_f32_12288x3072", lambda i: chk(lib.i8f_rotate128(ptr(deltas[i]), L.F32, Nw, Kw, Kw, ptr(rot_out), stream)), nk * 8)
+    load_time("weight_rotate_quant_f32_12288x3072", lambda i: chk(lib.i8f_quant_rowwise(
+        ptr(deltas[i]), L.F32, Nw, Kw, Kw, 128, ptr(dq), ptr(sw1), stream)), nk * 5 + 4 * Nw)
+    wb = [(torch.randn(Nw, Kw, device=dev) * 0.02).bfloat16() for _ in range(4)]
+    load_time("weight_quant_one_scale_bf16_12288x3072", lambda i: L.quant_tensorwise(wb[i]), nk * 5 + 4, sets=4)
+    out["weight_quant_one_scale_bf16_12288x3072"]["note"] = "two passes over the tensor (absmax, then quantise): 2+2 bytes read, 1 written per element"
+    del noises, outs, deltas, rot_out, dq, wb
 
     # few tiles and a long K (the text stream's down-projection of a DiT block): the K range of a tile dealt over
     # several workgroups through a workspace, against the same call without one; weights rotate through > 256 MB
