@@ -12,10 +12,11 @@
 //   * LDS rows keep the K-contiguous layout of the operands; the 16-byte chunk
 //     index is XOR-swizzled with the row so that the 32 lanes reading one K
 //     chunk of 32 different rows hit different banks.
-//   * v_mfma_i32_32x32x32_i8, W fragments as the A operand and X fragments as
-//     the B operand, so that a lane ends up with 4 consecutive n of one m:
-//     integer sums do not depend on the order of k, so any k permutation that
-//     is the same for both operands is allowed and none has to be undone.
+//   * v_mfma_i32_16x16x64_i8 (or v_mfma_i32_32x32x32_i8, per configuration), W
+//     fragments as the A operand and X fragments as the B operand, so that a
+//     lane ends up with 4 consecutive n of one m: integer sums do not depend
+//     on the order of k, so any k permutation that is the same for both
+//     operands is allowed and none has to be undone.
 //   * epilogue: scale/bias/round in registers, then a per-wave transpose
 //     through LDS so that every global store is 16 bytes per lane and covers
 //     whole 128-byte lines.
@@ -79,14 +80,15 @@ struct GemmArgs {
 // SPLIT_ (two-stage configurations): how a wave's loads of one K-tile are dealt over the phases that
 // follow the barrier which frees their stage, one hex digit per phase, first phase in the top digit
 // (0 = all of them in the first phase).
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_, int SPLIT_ = 0>
+// MF_: the MFMA shape, 32 (v_mfma_i32_32x32x32_i8) or 16 (v_mfma_i32_16x16x64_i8).
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_, int SPLIT_ = 0, int MF_ = 32>
 struct Cfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_, GROUP_M = GROUP_M_;
-    static constexpr int SPLIT = SPLIT_;
+    static constexpr int SPLIT = SPLIT_, MF = MF_;
     static constexpr int NW = WM * WN;
     static constexpr int NT = NW * 64;
     static constexpr int WTM = BM / WM, WTN = BN / WN;  // per-wave tile
-    static constexpr int MI = WTM / 32, NI = WTN / 32;  // 32x32 MFMA blocks per wave
+    static constexpr int MI = WTM / 32, NI = WTN / 32;  // 32 x 32 accumulator blocks per wave
     static constexpr int CPR = BK / 16;                 // 16-byte chunks per LDS row
     static constexpr int X_BYTES = BM * BK, W_BYTES = BN * BK;
     // every wave issues the same number of 1 KB loads per tile; a tile that does not split evenly
@@ -99,6 +101,7 @@ struct Cfg {
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert(X_BYTES % 1024 == 0 && W_BYTES % 1024 == 0, "tile must split into whole wave loads");
     static_assert(BK == 64 || BK == 128, "BK");
+    static_assert(MF == 32 || (MF == 16 && BK == 128), "the 16x16x64 form takes 128-byte K-tiles");
 };
 
 // chunk swizzle: a function of the low 5 bits of the row only
@@ -219,8 +222,11 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NI = C::NI, CPR = C::CPR;
     constexpr int S = C::STAGES;
     constexpr int OB = OutElem<OUT>::BYTES;
-    constexpr int KS = BK / 32;  // MFMA k-steps per tile
+    constexpr int KS = BK / 32;  // phases per tile (a k-step of 32 each, or half a wave tile's share of a k-step of 64)
     static_assert(KS % 2 == 0, "fragment double-buffering alternates over an even number of k-steps");
+    constexpr bool M16 = C::MF == 16;
+    static_assert(!(M16 && SIDE), "the side product has the accumulator layout of the 32x32x32 form");
+    constexpr int NQ = M16 ? 2 : 4;  // distinct column quads of a 32-column block among a lane's four
     // The epilogue stages EPI_STRIPS 32-row strips of a wave's tile at once (all of it for 2-byte
     // outputs), padded so that the transposing writes do not collide on banks.
     constexpr int ROW_BYTES = C::WTN * OB;
@@ -326,24 +332,95 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     for (int ks = 0; ks < KS; ++ks) koff[ks] = ((ks * 2 + lhalf) ^ sw) * 16;
     const int xrow_off = (wm * C::WTM + l32) * BK;
     const int wrow_off = C::X_ALLOC + (wn * C::WTN + l32) * BK;
+    // 16x16x64 form: a fragment is 16 rows x 64 k; lane l fetches the 16 bytes of row l % 16 at k-chunk l / 16 of the
+    // k-step (any k order will do as long as both operands use the same one).  The swizzle looks at the low five bits
+    // of the row, so the odd 16-row groups have their own chunk offsets.  Which chunk a lane quarter takes is chosen so
+    // that lane l touches the banks that lane l of the 32x32x32 form touches (lanes l and l + 32 read neighbouring
+    // chunks of one row): quarters 0, 1, 2, 3 take chunks 0, 2, 1, 3.
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int lchunk = ((lq & 1) << 1) | (lq >> 1);
+    [[maybe_unused]] int koff16[2][2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int hp = 0; hp < 2; ++hp) koff16[kk][hp] = ((kk * 4 + lchunk) ^ swz<CPR>(hp * 16 + l16)) * 16;
+    [[maybe_unused]] const int xrow16 = (wm * C::WTM + l16) * BK;
+    [[maybe_unused]] const int wrow16 = C::X_ALLOC + (wn * C::WTN + l16) * BK;
 
-    v16i acc[MI][NI];
+    // accumulators: per 32 x 32 block sixteen values per lane, as four quads of 4 consecutive n.
+    //   32x32x32: quad qd holds n = 8 qd + 4 (lane / 32) + e of row m = lane % 32
+    //   16x16x64: quad qd = 2 u + v holds n = 16 v + 4 (lane / 16) + e of row m = 16 u + lane % 16
+    v16i acc[M16 ? 1 : MI][M16 ? 1 : NI];
+    v4i acc16[M16 ? MI : 1][M16 ? NI : 1][4];
+    if constexpr (M16) {
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < NI; ++j)
+            for (int j = 0; j < NI; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-    auto load_frags = [&](const char *st, int ks, v4i (&xf)[MI], v4i (&wf)[NI]) {
+                for (int qd = 0; qd < 4; ++qd) acc16[i][j][qd] = (v4i)0;
+    } else {
 #pragma unroll
-        for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ks]);
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ks]);
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    }
+    // the lane's quad qd of block (i, j), and where it sits inside the block
+    auto quad_of = [&](int i, int j, int qd) -> v4i {
+        if constexpr (M16) return acc16[i][j][qd];
+        else return v4i{acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
     };
-    auto mma_one = [&](const v4i (&xf)[MI], const v4i (&wf)[NI], int r) {
-        const int i = r / NI, j = r % NI;
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+    auto quad_add = [&](int i, int j, int qd, v4i v) {
+        if constexpr (M16) acc16[i][j][qd] += v;
+        else acc[i][j][4 * qd] += v.x, acc[i][j][4 * qd + 1] += v.y, acc[i][j][4 * qd + 2] += v.z, acc[i][j][4 * qd + 3] += v.w;
+    };
+    auto quad_m = [&](int qd) { return M16 ? (qd >> 1) * 16 + l16 : l32; };              // row inside the 32-row strip
+    auto quad_n = [&](int qd) { return M16 ? (qd & 1) * 16 + lq * 4 : qd * 8 + lhalf * 4; };  // first column inside the block
+    auto quad_c = [&](int qd) constexpr { return M16 ? (qd & 1) : qd; };                  // which of the NQ column quads
+
+    // Fragment registers per phase.  32x32x32: MI + NI fragments of one k-step of 32.  16x16x64: a phase is one half of
+    // the wave tile's rows (MI fragments of 16 rows) against all 2 NI column fragments for a k-step of 64; phases 0, 1
+    // share the column fragments of k-step 0, phases 2, 3 those of k-step 1.
+    constexpr int XF = MI, WF = M16 ? 2 * NI : NI;
+    constexpr int MN = M16 ? MI * 2 * NI : MI * NI;  // MFMAs per phase
+    auto load_x = [&](const char *st, int ph, v4i (&xf)[XF]) {
+        if constexpr (M16) {
+            const int h = ph & 1, kk = (ph >> 1) & 1;
+#pragma unroll
+            for (int t = 0; t < MI; ++t) {
+                const int ii = h * MI + t;
+                xf[t] = *(const v4i *)(st + xrow16 + ii * 16 * BK + koff16[kk][ii & 1]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) xf[i] = *(const v4i *)(st + xrow_off + i * 32 * BK + koff[ph]);
+        }
+    };
+    auto load_w = [&](const char *st, int ph, v4i (&wf)[WF]) {
+        if constexpr (M16) {
+            const int kk = (ph >> 1) & 1;
+#pragma unroll
+            for (int jj = 0; jj < WF; ++jj) wf[jj] = *(const v4i *)(st + wrow16 + jj * 16 * BK + koff16[kk][jj & 1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ph]);
+        }
+    };
+    auto load_frags = [&](const char *st, int ph, v4i (&xf)[XF], v4i (&wf)[WF]) {
+        load_w(st, ph, wf);
+        load_x(st, ph, xf);
+    };
+    auto mma_one = [&](const v4i (&xf)[XF], const v4i (&wf)[WF], int ph, int r) {
+        if constexpr (M16) {
+            const int jj = r / MI, t = r % MI, ii = (ph & 1) * MI + t;  // a column fragment is done with after MI MFMAs
+            v4i &a = acc16[ii >> 1][jj >> 1][(ii & 1) * 2 + (jj & 1)];
+            a = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[jj], xf[t], a, 0, 0, 0);
+        } else {
+            const int i = r / NI, j = r % NI;
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
+        }
     };
 
     // ---- prologue: S tiles in flight, fragments of the first k-step in registers --------------
@@ -408,7 +485,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // K-tile, in front of its last MFMA group: by then every wave has finished reading tile kt
     // (its last fragments are in registers), so the stage of tile kt is refilled with tile kt+S
     // right away, and tile kt+1 is known to have landed, so its first fragments can be fetched.
-    v4i xa[MI] = {}, wa[NI] = {}, xb[MI] = {}, wb[NI] = {};
+    v4i xa[XF] = {}, wa[WF] = {}, xb[XF] = {}, wb[WF] = {};
     if (KT > 0) load_frags(smem, 0, xa, wa);
     // Drain scalar loads (kernel arguments) here: a scalar load still pending at the loop header
     // would turn every LDS wait inside the loop into a full lgkmcnt(0).
@@ -420,7 +497,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const bool last = ks == KS - 1;
-            constexpr int MN = MI * NI;
             if (last) {
                 // my part of tile kt+1 has landed and my LDS reads of tile kt have returned; what may
                 // still be in flight are the younger tiles (and, spread, the part of the newest one
@@ -429,14 +505,18 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(YOUNGER) & 0xF0FF);
                 __builtin_amdgcn_s_barrier();
             }
-            v4i(&xc)[MI] = (ks & 1) ? xb : xa;
-            v4i(&wc)[NI] = (ks & 1) ? wb : wa;
-            v4i(&xn)[MI] = (ks & 1) ? xa : xb;
-            v4i(&wn_)[NI] = (ks & 1) ? wa : wb;
+            v4i(&xc)[XF] = (ks & 1) ? xb : xa;
+            v4i(&xn)[XF] = (ks & 1) ? xa : xb;
+            // (16x16x64: one set of column fragments, each replaced as soon as its last MFMA of a k-step has issued)
+            v4i(&wc)[WF] = (!M16 && (ks & 1)) ? wb : wa;
+            v4i(&wn_)[WF] = (M16 || (ks & 1)) ? wa : wb;
             // past the last tile the next-fragment reads fetch stale LDS that nobody uses
             const char *fsrc = last ? nx : st;
             const int fks = last ? 0 : ks + 1;
-            load_frags(fsrc, fks, xn, wn_);
+            // 32x32x32: the next phase's fragments are requested in front of this phase's MFMAs.  16x16x64: one fragment
+            // behind each of the first MFMAs instead (a 16-cycle MFMA covers three or four other instructions, not a
+            // burst of eight LDS reads with their address arithmetic, and the two waves of a SIMD run in step).
+            if constexpr (!M16) load_frags(fsrc, fks, xn, wn_);
             __builtin_amdgcn_sched_barrier(0);
             // the tile being fetched: two stages refill the stage that this iteration's barrier frees
             // (tile kt+2) from the last phase on and finish in the following phases of the next iteration
@@ -446,12 +526,35 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
             // this phase's share of its loads
             const int la = SPREAD_DMA ? ks * C::LOADS / KS : (last ? 0 : cut(ks + 1));
             const int lb = SPREAD_DMA ? (ks + 1) * C::LOADS / KS : (last ? cut(1) : cut(ks + 2));
+            [[maybe_unused]] int frag = 0;  // row fragments of the next phase requested so far
 #pragma unroll
             for (int r = 0; r < MN; ++r) {
-                mma_one(xc, wc, r);
+                mma_one(xc, wc, ks, r);
+                const int l0 = la + r * (lb - la) / MN, l1 = la + (r + 1) * (lb - la) / MN;
+                if constexpr (M16) {
+                    const int kk = (fks >> 1) & 1;
+                    if ((ks & 1) && r % MI == MI - 1) {  // the k-step ends with this phase: the column fragment is free
+                        const int jj = r / MI;
+                        wn_[jj] = *(const v4i *)(fsrc + wrow16 + jj * 16 * BK + koff16[kk][jj & 1]);
+                    } else if (l0 == l1 && frag < XF) {  // a slot with nothing else to issue takes a row fragment
+                        const int ii = (fks & 1) * MI + frag;
+                        xn[frag] = *(const v4i *)(fsrc + xrow16 + ii * 16 * BK + koff16[kk][ii & 1]);
+                        ++frag;
+                    }
+                }
 #pragma unroll
-                for (int l = la + r * (lb - la) / MN; l < la + (r + 1) * (lb - la) / MN; ++l) issue_one(ft, live, l);
+                for (int l = l0; l < l1; ++l) issue_one(ft, live, l);
                 __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (M16) {  // (a phase with fewer free slots than row fragments)
+                const int kk = (fks >> 1) & 1;
+#pragma unroll
+                for (int f = 0; f < XF; ++f) {
+                    if (f >= frag) {
+                        const int ii = (fks & 1) * MI + f;
+                        xn[f] = *(const v4i *)(fsrc + xrow16 + ii * 16 * BK + koff16[kk][ii & 1]);
+                    }
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -475,9 +578,12 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         int *mine = g.partials + ((int64_t)slice * T + tile) * (BM * BN);
 #pragma unroll
         for (int qd = 0; qd < QUADS; ++qd) {
-            const int i = qd / (NI * 4), j = qd / 4 % NI, k4 = qd % 4 * 4;
-            const v4i o = {acc[i][j][k4], acc[i][j][k4 + 1], acc[i][j][k4 + 2], acc[i][j][k4 + 3]};
-            asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(mine + ((int64_t)qd * C::NT + tid) * 4), "v"(o) : "memory");
+            const int i = qd / (NI * 4), j = qd / 4 % NI;
+            const v4i o = quad_of(i, j, qd % 4);
+            // (s_nop 1: a 16-byte store reads its data registers after it has issued, and the two wait states that keep a
+            // following vector instruction from overwriting them are the compiler's job, which it cannot do for an
+            // instruction it does not see)
+            asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(mine + ((int64_t)qd * C::NT + tid) * 4), "v"(o) : "memory");
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -498,8 +604,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                              : "memory");
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int qd = q0 + u, i = qd / (NI * 4), j = qd / 4 % NI, k4 = qd % 4 * 4;
-                    acc[i][j][k4] += v[u].x, acc[i][j][k4 + 1] += v[u].y, acc[i][j][k4 + 2] += v[u].z, acc[i][j][k4 + 3] += v[u].w;
+                    const int qd = q0 + u, i = qd / (NI * 4), j = qd / 4 % NI;
+                    quad_add(i, j, qd % 4, v[u]);
                 }
             }
         }
@@ -535,16 +641,23 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // scale, bias, round.  The per-column operands (4 consecutive n per lane and MFMA block) are
     // fetched from LDS into registers once, in front of the strips: fetched inside, every group of
     // four values would wait for an LDS round trip.
+    // the activation scales of the lane's rows of strip i: one row, or (16x16x64) one per 16-row half
+    auto strip_scales = [&](int i, float (&xs2)[2]) {
+        xs2[0] = s_xs[wm * C::WTM + i * 32 + quad_m(0)];
+        xs2[1] = M16 ? s_xs[wm * C::WTM + i * 32 + quad_m(2)] : xs2[0];
+    };
     auto convert_strip = [&](int i, char *dst_rows, const auto &wr, const auto &br, auto ORDER, auto ROW, auto BIAS) {
-        const float xs = s_xs[wm * C::WTM + i * 32 + l32];
+        float xs2[2];
+        strip_scales(i, xs2);
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
-                const int nl = j * 32 + qd * 8 + lhalf * 4;  // first of 4 consecutive n held by this lane
-                const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
+                const int nl = j * 32 + quad_n(qd);  // first of 4 consecutive n held by this lane
+                const v4i q4 = quad_of(i, j, qd);
+                const int a4[4] = {q4.x, q4.y, q4.z, q4.w};
                 epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value>(
-                    a4, xs, wr[j][qd], br[j][qd], dst_rows + l32 * PITCH + nl * OB);
+                    a4, xs2[qd >> 1], wr[j][quad_c(qd)], br[j][quad_c(qd)], dst_rows + quad_m(qd) * PITCH + nl * OB);
             }
         }
     };
@@ -564,15 +677,15 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     constexpr bool PRELOAD_ALL = C::NT <= 512 && !SIDE;
     auto run_epilogue = [&](auto ORDER, auto ROW, auto BIAS) {
         constexpr int NPRE = PRELOAD_ALL ? NI : 1;
-        float4 wr[NPRE][4], br[NPRE][4];
-        auto fetch_cols = [&](int j, float4 (&wj)[4], float4 (&bj)[4]) __attribute__((always_inline)) {
+        float4 wr[NPRE][NQ], br[NPRE][NQ];
+        auto fetch_cols = [&](int j, float4 (&wj)[NQ], float4 (&bj)[NQ]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int nl = wn * C::WTN + j * 32 + qd * 8 + lhalf * 4;
-                if constexpr (decltype(ROW)::value) wj[qd] = *(const float4 *)&s_ws[nl];
-                else wj[qd] = make_float4(s_ws[0], s_ws[0], s_ws[0], s_ws[0]);
-                if constexpr (decltype(BIAS)::value) bj[qd] = *(const float4 *)&s_bias[nl];
-                else bj[qd] = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int c = 0; c < NQ; ++c) {
+                const int nl = wn * C::WTN + j * 32 + quad_n(c);  // (16x16x64: quads 0 and 1 are the two distinct ones)
+                if constexpr (decltype(ROW)::value) wj[c] = *(const float4 *)&s_ws[nl];
+                else wj[c] = make_float4(s_ws[0], s_ws[0], s_ws[0], s_ws[0]);
+                if constexpr (decltype(BIAS)::value) bj[c] = *(const float4 *)&s_bias[nl];
+                else bj[c] = make_float4(0.f, 0.f, 0.f, 0.f);
             }
         };
         if constexpr (OUT != OUT_I32 && PRELOAD_ALL) {
@@ -590,9 +703,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                     for (int j = 0; j < NI; ++j)
 #pragma unroll
                         for (int qd = 0; qd < 4; ++qd) {
-                            const int nl = j * 32 + qd * 8 + lhalf * 4;
-                            v4i o = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
-                            *(v4i *)(rows + l32 * PITCH + nl * 4) = o;
+                            const int nl = j * 32 + quad_n(qd);
+                            *(v4i *)(rows + quad_m(qd) * PITCH + nl * 4) = quad_of(i, j, qd);
                         }
                 } else if constexpr (PRELOAD_ALL) {
                     convert_strip(i, rows, wr, br, ORDER, ROW, BIAS);
@@ -617,7 +729,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
 #pragma unroll
                     for (int is = 0; is < EPI_STRIPS; ++is) {
                         const int i = i0 + is;
-                        const float xs = s_xs[wm * C::WTM + i * 32 + l32];
+                        float xs2[2];
+                        strip_scales(i, xs2);
                         [[maybe_unused]] float sd[16];
                         if constexpr (SIDE) {
                             const int m = min(m0 + wm * C::WTM + i * 32 + l32, gM - 1);
@@ -641,10 +754,12 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                         }
 #pragma unroll
                         for (int qd = 0; qd < 4; ++qd) {
-                            const int nl = j * 32 + qd * 8 + lhalf * 4;
-                            const int a4[4] = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
+                            const int nl = j * 32 + quad_n(qd);
+                            const v4i q4 = quad_of(i, j, qd);
+                            const int a4[4] = {q4.x, q4.y, q4.z, q4.w};
                             epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value, SIDE>(
-                                a4, xs, wr[0][qd], br[0][qd], ebuf + (is * 32 + l32) * PITCH + nl * OB, SIDE ? &sd[4 * qd] : nullptr);
+                                a4, xs2[qd >> 1], wr[0][quad_c(qd)], br[0][quad_c(qd)], ebuf + (is * 32 + quad_m(qd)) * PITCH + nl * OB,
+                                SIDE ? &sd[4 * qd] : nullptr);
                         }
                     }
                 }
@@ -732,20 +847,31 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
     }
 }
 
-// tile configurations
-using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400>;  // 8 waves, 2 x 64 KB stages, one workgroup per CU; refill in two halves (2-3 % faster than one burst)
-using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
-using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
-using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8>;  // 12 waves of 96 x 64, 2 x 72 KB stages
-using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8>;  // 12 waves of 64 x 96, the same transposed
+// tile configurations.  The one-workgroup-per-CU tiles run on v_mfma_i32_16x16x64_i8: on realistic operands the chip is at
+// its power limit, and the same multiply-accumulates cost less energy in that form than as v_mfma_i32_32x32x32_i8 (with
+// nothing but MFMAs in a loop, operands in registers, the chip sustains 3.9 POP/s against 3.2; on all-zero operands both
+// reach 4.9), so the clock settles higher.  The shorter instruction covers fewer other instructions, which is why that form
+// deals its LDS reads out one by one; the few-tile configurations (one wave per SIMD, bound by the global->LDS path) lose
+// more to that than they gain and keep the 32x32x32 form, as does the variant with the low-rank side product, whose own
+// MFMAs produce the 32x32 accumulator layout.
+using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400, 16>;  // 8 waves, 2 x 64 KB stages, one workgroup per CU; refill in two halves (2-3 % faster than one burst)
+using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6, 0, 16>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
+using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8, 0, 16>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
+using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8, 0, 16>;  // 12 waves of 96 x 64, 2 x 72 KB stages
+using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8, 0, 16>;  // 12 waves of 64 x 96, the same transposed
 // Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
 // loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
 // flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
-using CfgW96 = Cfg<256, 96, 128, 8, 1, 3, 8>;      // 8 waves of 32 x 96, 3 x 44 KB stages
+using CfgW96 = Cfg<256, 96, 128, 8, 1, 3, 8, 0, 16>;      // 8 waves of 32 x 96, 3 x 44 KB stages
 using CfgMidDeep = Cfg<128, 128, 128, 2, 2, 4, 8>;
 using CfgM96Deep = Cfg<128, 96, 128, 4, 1, 4, 8>;
 using CfgS64Deep = Cfg<128, 64, 128, 2, 2, 4, 8>;
 using CfgT64Deep = Cfg<64, 64, 128, 2, 2, 4, 8>;
+// the tiles that take the low-rank side product, in the 32x32x32 form
+using CfgBigSide = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400>;
+using CfgB192Side = Cfg<256, 192, 128, 4, 2, 2, 6>;
+using CfgMidSide = Cfg<128, 128, 128, 2, 2, 2, 8>;
+using CfgW96Side = Cfg<256, 96, 128, 8, 1, 3, 8>;
 
 template <class C, int OUT>
 int launch_cfg(GemmArgs &g, hipStream_t st) {
@@ -753,11 +879,13 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
     g.tiles_n = (g.N + C::BN - 1) / C::BN;
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
     const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);  // what the prologue wants to know of the epilogue
-    if constexpr ((OUT == OUT_BF16 || OUT == OUT_F16) && C::NT <= 512) {  // (twelve-wave tiles have no registers to spare for it)
-        if (g.side_t) {  // validated by the entry point: K % BK == 0 here
+    if (g.side_t) {  // validated by the entry point: K % BK == 0 here
+        if constexpr ((OUT == OUT_BF16 || OUT == OUT_F16) && C::NT <= 512 && C::MF == 32) {  // (twelve-wave tiles have no registers to spare for it)
             hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N,
                                g.K, g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
             return check_launch();
+        } else {
+            return I8F_ERR_UNSUPPORTED;
         }
     }
     if constexpr (C::STAGES == 4) {  // the K split exists for the few-tile configurations
@@ -877,8 +1005,33 @@ inline void choose_split(int64_t M, int64_t N, int64_t K, Tile &t, int &splits) 
     t = keep;
 }
 
+// the side product alone (the configurations above without it are never launched in this form)
+template <class C, int OUT>
+int launch_side(GemmArgs &g, hipStream_t st) {
+    if constexpr (OUT == OUT_BF16 || OUT == OUT_F16) {
+        g.tiles_m = (g.M + C::BM - 1) / C::BM;
+        g.tiles_n = (g.N + C::BN - 1) / C::BN;
+        const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+        const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);
+        hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
+                           g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
+        return check_launch();
+    } else {
+        return I8F_ERR_UNSUPPORTED;
+    }
+}
+
 template <int OUT>
 int launch_tile(Tile t, GemmArgs &g, hipStream_t st) {
+    if (g.side_t) {
+        switch (t) {
+        case TILE_BIG: return launch_side<CfgBigSide, OUT>(g, st);
+        case TILE_B192: return launch_side<CfgB192Side, OUT>(g, st);
+        case TILE_MID: return launch_side<CfgMidSide, OUT>(g, st);
+        case TILE_W96: return launch_side<CfgW96Side, OUT>(g, st);
+        default: break;  // the few-tile configurations below are in the 32x32x32 form themselves
+        }
+    }
     switch (t) {
     case TILE_BIG: return launch_cfg<CfgBig, OUT>(g, st);
     case TILE_B192: return launch_cfg<CfgB192, OUT>(g, st);
