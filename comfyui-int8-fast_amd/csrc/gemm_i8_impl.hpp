@@ -851,12 +851,12 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 // its power limit, and the same multiply-accumulates cost less energy in that form than as v_mfma_i32_32x32x32_i8 (with
 // nothing but MFMAs in a loop, operands in registers, the chip sustains 3.9 POP/s against 3.2; on all-zero operands both
 // reach 4.9), so the clock settles higher.  The shorter instruction covers fewer other instructions, which is why that form
-// deals its LDS reads out one by one; the few-tile configurations (one wave per SIMD, bound by the global->LDS path) lose
-// more to that than they gain and keep the 32x32x32 form, as does the variant with the low-rank side product, whose own
+// deals its LDS reads out one by one; the 128 x 128 tile and the few-tile configurations (one wave per SIMD, bound by the
+// global->LDS path) lose more to that than they gain and keep the 32x32x32 form, as does the variant with the low-rank side product, whose own
 // MFMAs produce the 32x32 accumulator layout.
 using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400, 16>;  // 8 waves, 2 x 64 KB stages, one workgroup per CU; refill in two halves (2-3 % faster than one burst)
 using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6, 0, 16>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
-using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8, 0, 16>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU
+using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU (10 % slower with the 16x16x64 MFMA: 32x32x32)
 using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8, 0, 16>;  // 12 waves of 96 x 64, 2 x 72 KB stages
 using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8, 0, 16>;  // 12 waves of 64 x 96, the same transposed
 // Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
@@ -870,7 +870,6 @@ using CfgT64Deep = Cfg<64, 64, 128, 2, 2, 4, 8>;
 // the tiles that take the low-rank side product, in the 32x32x32 form
 using CfgBigSide = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400>;
 using CfgB192Side = Cfg<256, 192, 128, 4, 2, 2, 6>;
-using CfgMidSide = Cfg<128, 128, 128, 2, 2, 2, 8>;
 using CfgW96Side = Cfg<256, 96, 128, 8, 1, 3, 8>;
 
 template <class C, int OUT>
@@ -1027,9 +1026,8 @@ int launch_tile(Tile t, GemmArgs &g, hipStream_t st) {
         switch (t) {
         case TILE_BIG: return launch_side<CfgBigSide, OUT>(g, st);
         case TILE_B192: return launch_side<CfgB192Side, OUT>(g, st);
-        case TILE_MID: return launch_side<CfgMidSide, OUT>(g, st);
         case TILE_W96: return launch_side<CfgW96Side, OUT>(g, st);
-        default: break;  // the few-tile configurations below are in the 32x32x32 form themselves
+        default: break;  // the 128 x 128 tile and the few-tile configurations are in the 32x32x32 form themselves
         }
     }
     switch (t) {
