@@ -149,6 +149,21 @@ def test_random_linear_w8a8_long_k(L, dev):
     check(bad)
 
 
+def test_random_linear_w8a8_large(L, dev):
+    """Outputs of hundreds of 256-row tiles, ragged on every side: the one-workgroup-per-CU configurations
+    (256x256, 256x192, 288x256, 256x288 and the rounds they are chosen by), which the draws above seldom reach."""
+    rng, g = gens(108)
+    bad, tiles = [], set()
+    for case in range(32):
+        M, N, K = int(rng.integers(900, 6000)), 8 * int(rng.integers(100, 1700)), 16 * int(rng.integers(1, 130))
+        tiles.add(L.gemm_tile(M, N, K)[:2])
+        ok, what = linear_case(L, dev, rng, g, M, N, K, case % 4 == 0)
+        if not ok:
+            bad.append(what)
+    assert not bad, f"{len(bad)} of 32 draws differ from the oracle: {bad[:6]}"
+    assert len(tiles) >= 4, tiles
+
+
 def test_random_small_m_w8a16(L, dev):
     """Small-batch W8A16 (int8_quant.py:666-674): |y - y_ref| <= spacing(y_ref) + K 2^-24 sum |x||w|."""
     rng, g = gens(106)
