@@ -52,6 +52,19 @@ __device__ __forceinline__ v16f side_mfma(v4i a, v4i b, v16f c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, a), __builtin_bit_cast(v8h_t, b), c, 0, 0, 0);
 }
 
+// 16 x 16 x 16 product of two 16-bit fragments (4 values per lane each) into a binary32 block
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef short v4s_t __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h_t __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+template <int OUT>
+__device__ __forceinline__ v4f side_mfma16(v2i a, v2i b, v4f c) {
+    if constexpr (OUT == OUT_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(v4s_t, a), __builtin_bit_cast(v4s_t, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(v4h_t, a), __builtin_bit_cast(v4h_t, b), c, 0, 0, 0);
+}
+
 struct GemmArgs {
     const int8_t *x;
     const int8_t *w;
@@ -225,7 +238,6 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     constexpr int KS = BK / 32;  // phases per tile (a k-step of 32 each, or half a wave tile's share of a k-step of 64)
     static_assert(KS % 2 == 0, "fragment double-buffering alternates over an even number of k-steps");
     constexpr bool M16 = C::MF == 16;
-    static_assert(!(M16 && SIDE), "the side product has the accumulator layout of the 32x32x32 form");
     constexpr int NQ = M16 ? 2 : 4;  // distinct column quads of a 32-column block among a lane's four
     // The epilogue stages EPI_STRIPS 32-row strips of a wave's tile at once (all of it for 2-byte
     // outputs), padded so that the transposing writes do not collide on banks.
@@ -717,14 +729,26 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                     // side branch: the rank-r product of this 32 x 32 block on the matrix cores, with the same
                     // operand roles as the main product (rows n from side_b, columns m from side_t), so that
                     // the result has the accumulators' layout
+                    // (16x16x64 form: four 16 x 16 products per block, a lane's fragment being 4 ranks of one row)
                     constexpr int RMAX = 64;
-                    [[maybe_unused]] v4i bfr[RMAX / 16];
-                    if constexpr (SIDE) {
+                    [[maybe_unused]] v4i bfr[M16 ? 1 : RMAX / 16];
+                    [[maybe_unused]] v2i bfr16[M16 ? 2 : 1][RMAX / 16];
+                    if constexpr (SIDE && !M16) {
                         const int n = min(n0 + wn * C::WTN + j * 32 + l32, gN - 1);
 #pragma unroll
                         for (int ks = 0; ks < RMAX / 16; ++ks)
                             if (ks * 16 < g.side_rank)
                                 bfr[ks] = *(const v4i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lhalf * 8) * 2);
+                    }
+                    if constexpr (SIDE && M16) {
+#pragma unroll
+                        for (int v = 0; v < 2; ++v) {
+                            const int n = min(n0 + wn * C::WTN + j * 32 + v * 16 + l16, gN - 1);
+#pragma unroll
+                            for (int ks = 0; ks < RMAX / 16; ++ks)
+                                if (ks * 16 < g.side_rank)
+                                    bfr16[v][ks] = *(const v2i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lq * 4) * 2);
+                        }
                     }
 #pragma unroll
                     for (int is = 0; is < EPI_STRIPS; ++is) {
@@ -732,7 +756,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                         float xs2[2];
                         strip_scales(i, xs2);
                         [[maybe_unused]] float sd[16];
-                        if constexpr (SIDE) {
+                        constexpr int SDT = OUT == OUT_F16 ? I8F_F16 : I8F_BF16;
+                        if constexpr (SIDE && !M16) {
                             const int m = min(m0 + wm * C::WTM + i * 32 + l32, gM - 1);
                             v16f sacc;
 #pragma unroll
@@ -744,12 +769,34 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                                     sacc = side_mfma<OUT>(bfr[ks], tfr, sacc);
                                 }
                             }
-                            constexpr int DT = OUT == OUT_BF16 ? I8F_BF16 : I8F_F16;
 #pragma unroll
                             for (int r = 0; r < 16; ++r) {
-                                float v = round_to_dtype<DT>(sacc[r]);
-                                if (g.side_has_alpha) v = round_to_dtype<DT>(v * g.side_alpha);
+                                float v = round_to_dtype<SDT>(sacc[r]);
+                                if (g.side_has_alpha) v = round_to_dtype<SDT>(v * g.side_alpha);
                                 sd[r] = v;
+                            }
+                        }
+                        if constexpr (SIDE && M16) {
+#pragma unroll
+                            for (int u = 0; u < 2; ++u) {
+                                const int m = min(m0 + wm * C::WTM + i * 32 + u * 16 + l16, gM - 1);
+                                v4f sacc[2] = {(v4f)0.0f, (v4f)0.0f};
+#pragma unroll
+                                for (int ks = 0; ks < RMAX / 16; ++ks) {
+                                    if (ks * 16 < g.side_rank) {
+                                        const v2i tfr = *(const v2i *)((const char *)g.side_t + ((int64_t)m * g.side_rank + ks * 16 + lq * 4) * 2);
+#pragma unroll
+                                        for (int v = 0; v < 2; ++v) sacc[v] = side_mfma16<OUT>(bfr16[v][ks], tfr, sacc[v]);
+                                    }
+                                }
+#pragma unroll
+                                for (int v = 0; v < 2; ++v)
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) {
+                                        float y = round_to_dtype<SDT>(sacc[v][e]);
+                                        if (g.side_has_alpha) y = round_to_dtype<SDT>(y * g.side_alpha);
+                                        sd[4 * (u * 2 + v) + e] = y;
+                                    }
                             }
                         }
 #pragma unroll
@@ -852,8 +899,7 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 // nothing but MFMAs in a loop, operands in registers, the chip sustains 3.9 POP/s against 3.2; on all-zero operands both
 // reach 4.9), so the clock settles higher.  The shorter instruction covers fewer other instructions, which is why that form
 // deals its LDS reads out one by one; the 128 x 128 tile and the few-tile configurations (one wave per SIMD, bound by the
-// global->LDS path) lose more to that than they gain and keep the 32x32x32 form, as does the variant with the low-rank side product, whose own
-// MFMAs produce the 32x32 accumulator layout.
+// global->LDS path) lose more to that than they gain and keep the 32x32x32 form.
 using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400, 16>;  // 8 waves, 2 x 64 KB stages, one workgroup per CU; refill in two halves (2-3 % faster than one burst)
 using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6, 0, 16>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU (10 % slower with the 16x16x64 MFMA: 32x32x32)
@@ -867,11 +913,6 @@ using CfgMidDeep = Cfg<128, 128, 128, 2, 2, 4, 8>;
 using CfgM96Deep = Cfg<128, 96, 128, 4, 1, 4, 8>;
 using CfgS64Deep = Cfg<128, 64, 128, 2, 2, 4, 8>;
 using CfgT64Deep = Cfg<64, 64, 128, 2, 2, 4, 8>;
-// the tiles that take the low-rank side product, in the 32x32x32 form
-using CfgBigSide = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400>;
-using CfgB192Side = Cfg<256, 192, 128, 4, 2, 2, 6>;
-using CfgW96Side = Cfg<256, 96, 128, 8, 1, 3, 8>;
-
 template <class C, int OUT>
 int launch_cfg(GemmArgs &g, hipStream_t st) {
     g.tiles_m = (g.M + C::BM - 1) / C::BM;
@@ -879,7 +920,7 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
     const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);  // what the prologue wants to know of the epilogue
     if (g.side_t) {  // validated by the entry point: K % BK == 0 here
-        if constexpr ((OUT == OUT_BF16 || OUT == OUT_F16) && C::NT <= 512 && C::MF == 32) {  // (twelve-wave tiles have no registers to spare for it)
+        if constexpr ((OUT == OUT_BF16 || OUT == OUT_F16) && C::NT <= 512) {  // (twelve-wave tiles have no registers to spare for it)
             hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N,
                                g.K, g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
             return check_launch();
@@ -1004,32 +1045,8 @@ inline void choose_split(int64_t M, int64_t N, int64_t K, Tile &t, int &splits) 
     t = keep;
 }
 
-// the side product alone (the configurations above without it are never launched in this form)
-template <class C, int OUT>
-int launch_side(GemmArgs &g, hipStream_t st) {
-    if constexpr (OUT == OUT_BF16 || OUT == OUT_F16) {
-        g.tiles_m = (g.M + C::BM - 1) / C::BM;
-        g.tiles_n = (g.N + C::BN - 1) / C::BN;
-        const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-        const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);
-        hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N, g.K,
-                           g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
-        return check_launch();
-    } else {
-        return I8F_ERR_UNSUPPORTED;
-    }
-}
-
 template <int OUT>
 int launch_tile(Tile t, GemmArgs &g, hipStream_t st) {
-    if (g.side_t) {
-        switch (t) {
-        case TILE_BIG: return launch_side<CfgBigSide, OUT>(g, st);
-        case TILE_B192: return launch_side<CfgB192Side, OUT>(g, st);
-        case TILE_W96: return launch_side<CfgW96Side, OUT>(g, st);
-        default: break;  // the 128 x 128 tile and the few-tile configurations are in the 32x32x32 form themselves
-        }
-    }
     switch (t) {
     case TILE_BIG: return launch_cfg<CfgBig, OUT>(g, st);
     case TILE_B192: return launch_cfg<CfgB192, OUT>(g, st);
