@@ -435,6 +435,27 @@ def extras(L, dev, quick=False):
     return out
 
 
+# --------------------------------------------------------------------------- the north-star launch alone
+def target_only(L, dev, mode, steps, warmup):
+    """Nothing but launches of the north-star GEMM (M=4608, N=K=3072, W8A8 rowwise, bf16 out), for profilers:
+    `warm` repeats one operand set (resident in the memory-side cache), `cold` walks 12 sets (623 MB).  Every GEMM
+    launch of the process is one of these, so a counter file needs no filtering beyond the kernel name."""
+    M, N, K = 4608, 3072, 3072
+    g = torch.Generator().manual_seed(99)
+    nset = 12 if mode == "cold" else 1
+    q, s = L.quant_rowwise(_acts(g, M, K, 0.01, 20.0).to(dev))
+    wq, ws = L.quant_rowwise((torch.randn(N, K, generator=g) * 0.02).to(dev))
+    qs = [q] + [q.clone() for _ in range(nset - 1)]
+    wqs = [wq] + [wq.clone() for _ in range(nset - 1)]
+    ys = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nset)]
+    t = time_kernel(lambda i: L.linear_w8a8(qs[i], s, wqs[i], ws, None, torch.bfloat16, L.EPI_TORCH, ys[i]),
+                    iters=max(1, steps // nset), warmup=warmup, sets=nset, burst=nset)
+    ops = 2 * M * N * K
+    return {"kernel": "gemm_i8_kernel", "shape": "4608x3072x3072", "operands": mode, "tile": "%dx%d" % L.gemm_tile(M, N, K)[:2],
+            "median_us": round(t["median_us"], 2), "min_us": round(t["min_us"], 2),
+            "frac_of_int8_peak": round(ops / t["median_us"] / 1e6 / PEAK_INT8_TOPS, 4)}
+
+
 # --------------------------------------------------------------------------- CPU baseline
 def cpu_baseline(reps=3):
     """The reference's torch CPU path on config 1.  A 512-row probe sizes the sample: the whole
@@ -473,6 +494,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--quick", action="store_true", help="fewer iterations in the extra measurements")
+    ap.add_argument("--target-only", choices=("warm", "cold"),
+                    help="profiling aid: launch nothing but the north-star GEMM (4608x3072x3072) on warm or cold operands, "
+                         "print its timing and exit")
     ap.add_argument("--zero-operands", action="store_true",
                     help="diagnostic: all-zero activations and weights (same instructions, no switching in the multipliers), "
                          "to show what the power limit costs; the line says data = zeros and is not a benchmark result")
@@ -488,6 +512,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if a.target_only:
+        print(json.dumps(target_only(L, dev, a.target_only, a.steps, a.warmup)))
+        return
     step = MlpStep(L, dev)
     if a.zero_operands:
         for t in (step.x, step.h, step.wq_up, step.wq_dn):

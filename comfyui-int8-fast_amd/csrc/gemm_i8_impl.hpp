@@ -94,24 +94,35 @@ struct GemmArgs {
 // follow the barrier which frees their stage, one hex digit per phase, first phase in the top digit
 // (0 = all of them in the first phase).
 // MF_: the MFMA shape, 32 (v_mfma_i32_32x32x32_i8) or 16 (v_mfma_i32_16x16x64_i8).
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_, int SPLIT_ = 0, int MF_ = 32>
+// WSTAGES_: stages of the W tile if not STAGES_ (which the X tile always has): 160 KB of LDS hold two 256 x 128-byte
+// X tiles and three W tiles but not three of each, and one operand a stage ahead of the other is enough to take the
+// global->LDS latency out of the loop's critical path (the W refill then has two K-tiles of time to land, and the X
+// refill, half the bytes of a whole stage, is issued first behind the barrier).
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int GROUP_M_, int SPLIT_ = 0, int MF_ = 32, int WSTAGES_ = STAGES_>
 struct Cfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_, GROUP_M = GROUP_M_;
-    static constexpr int SPLIT = SPLIT_, MF = MF_;
+    static constexpr int SPLIT = SPLIT_, MF = MF_, WSTAGES = WSTAGES_;
     static constexpr int NW = WM * WN;
     static constexpr int NT = NW * 64;
     static constexpr int WTM = BM / WM, WTN = BN / WN;  // per-wave tile
-    static constexpr int MI = WTM / 32, NI = WTN / 32;  // 32 x 32 accumulator blocks per wave
+    // A wave's accumulators are blocks of 32 rows x CB columns: 32 x 32 with the 32x32x32 MFMA, 32 x 16 (two 16 x 16
+    // products one above the other) with the 16x16x64 MFMA, whose wave tiles may therefore be 48 columns wide.
+    static constexpr int CB = MF_ == 16 ? 16 : 32;
+    static constexpr int MI = WTM / 32, NJ = WTN / CB;
     static constexpr int CPR = BK / 16;                 // 16-byte chunks per LDS row
     static constexpr int X_BYTES = BM * BK, W_BYTES = BN * BK;
     // every wave issues the same number of 1 KB loads per tile; a tile that does not split evenly
     // over the waves is rounded up, and the surplus loads are out of range (they move nothing)
     static constexpr int X_LOADS = (X_BYTES / 1024 + NW - 1) / NW, W_LOADS = (W_BYTES / 1024 + NW - 1) / NW;
     static constexpr int X_ALLOC = X_LOADS * NW * 1024, W_ALLOC = W_LOADS * NW * 1024;
-    static constexpr int STAGE_BYTES = X_ALLOC + W_ALLOC;
     static constexpr int LOADS = X_LOADS + W_LOADS;
-    static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
-    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
+    // LDS: stages of an X tile followed by its W tile; with W a stage deeper, the X stages and then the W stages
+    static constexpr int W_BASE = WSTAGES == STAGES ? X_ALLOC : X_ALLOC * STAGES;
+    static constexpr int X_STRIDE = WSTAGES == STAGES ? X_ALLOC + W_ALLOC : X_ALLOC;
+    static constexpr int W_STRIDE = WSTAGES == STAGES ? X_ALLOC + W_ALLOC : W_ALLOC;
+    static constexpr int LDS_BYTES = X_ALLOC * STAGES + W_ALLOC * WSTAGES;
+    static_assert(WSTAGES == STAGES || (STAGES == 2 && WSTAGES == 3), "W may be one stage ahead of a two-stage X");
+    static_assert(WTM % 32 == 0 && WTN % CB == 0, "wave tile must be a multiple of 32 rows x CB columns");
     static_assert(X_BYTES % 1024 == 0 && W_BYTES % 1024 == 0, "tile must split into whole wave loads");
     static_assert(BK == 64 || BK == 128, "BK");
     static_assert(MF == 32 || (MF == 16 && BK == 128), "the 16x16x64 form takes 128-byte K-tiles");
@@ -232,23 +243,28 @@ template <class C, int OUT, bool KTAIL, bool SIDE = false, bool SPLITK = false>
 __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
                                                         const float *gxs, const float *gws, const void *gbias, int flags,
                                                         const GemmArgs g) {
-    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NI = C::NI, CPR = C::CPR;
-    constexpr int S = C::STAGES;
+    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NJ = C::NJ, CB = C::CB, CPR = C::CPR;
+    constexpr int S = C::STAGES, WS = C::WSTAGES;
+    constexpr bool ASYM = WS != S;  // the W tile one stage deeper than the X tile
     constexpr int OB = OutElem<OUT>::BYTES;
     constexpr int KS = BK / 32;  // phases per tile (a k-step of 32 each, or half a wave tile's share of a k-step of 64)
     static_assert(KS % 2 == 0, "fragment double-buffering alternates over an even number of k-steps");
     constexpr bool M16 = C::MF == 16;
-    constexpr int NQ = M16 ? 2 : 4;  // distinct column quads of a 32-column block among a lane's four
+    constexpr int QPB = M16 ? 2 : 4;  // quads (4 consecutive n of one m) a lane holds per block
+    constexpr int NQ = M16 ? 1 : 4;   // distinct column positions among them
     // The epilogue stages EPI_STRIPS 32-row strips of a wave's tile at once (all of it for 2-byte
     // outputs), padded so that the transposing writes do not collide on banks.
     constexpr int ROW_BYTES = C::WTN * OB;
     constexpr int PITCH = ROW_BYTES + (OB == 2 ? 8 : 16);
     constexpr int EPI_STRIPS = (OB == 2 || MI == 1) ? MI : MI / 2;
     constexpr int WAVE_BYTES = EPI_STRIPS * 32 * PITCH;
-    constexpr int SMEM_BYTES = C::LDS_BYTES > WAVE_BYTES * NW ? C::LDS_BYTES : WAVE_BYTES * NW;
-    static_assert(SMEM_BYTES + 4 * (BM + 2 * BN) <= 160 * 1024, "LDS");
+    // The epilogue operands of the tile (token scales, weight scales, bias) are staged behind the waves' transpose
+    // buffers, in memory that belongs to the K-tile stages while the main loop runs.
+    constexpr int EPI_OPS_OFF = WAVE_BYTES * NW, EPI_OPS_BYTES = 4 * (BM + 2 * BN);
+    constexpr int SMEM_BYTES = C::LDS_BYTES > EPI_OPS_OFF + EPI_OPS_BYTES ? C::LDS_BYTES : EPI_OPS_OFF + EPI_OPS_BYTES;
+    static_assert(SMEM_BYTES + (SPLITK ? 16 : 0) <= 160 * 1024, "LDS");
     __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
-    __shared__ float s_xs[BM], s_ws[BN], s_bias[BN];  // epilogue operands of this tile
+    float *const s_xs = (float *)(smem + EPI_OPS_OFF), *const s_ws = s_xs + BM, *const s_bias = s_ws + BN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -319,19 +335,21 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // but moves no data.
     // load r of tile kt: r < X_LOADS fetches a piece of the X tile, the others a piece of the W tile
     const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
-    auto issue_one = [&](int kt, bool live, int r) {
-        const uint32_t st = smem_base + (kt % S) * C::STAGE_BYTES + wave * 1024;
-        const int kb = (kt_first + kt) * BK;
+    // (sx, sw: the stage of the X and of the W tile that receives tile kt)
+    auto issue_to = [&](int kt, int sx, int sw, bool live, int r) {
         const bool is_x = r < C::X_LOADS;
         const int t = is_x ? r : r - C::X_LOADS;
+        const uint32_t st = smem_base + (is_x ? sx * C::X_STRIDE : C::W_BASE + sw * C::W_STRIDE) + wave * 1024;
+        const int kb = (kt_first + kt) * BK;
         uint32_t vo = live ? (is_x ? xoff[t] : woff[t]) : OOB;
         int so = kb;
         if constexpr (KTAIL) {  // chunks past K are forced out of range per lane
             vo = (kb + (is_x ? xck[t] : wck[t]) < K && vo != OOB) ? vo + (uint32_t)kb : OOB;
             so = 0;
         }
-        dma16(is_x ? rx : rw, st + (is_x ? 0 : C::X_ALLOC) + t * NW * 1024, vo, so);
+        dma16(is_x ? rx : rw, st + t * NW * 1024, vo, so);
     };
+    auto issue_one = [&](int kt, bool live, int r) { issue_to(kt, kt % S, kt % WS, live, r); };  // (prologue: kt is a constant)
     auto issue = [&](int kt, bool live) {
 #pragma unroll
         for (int r = 0; r < C::LOADS; ++r) issue_one(kt, live, r);
@@ -343,7 +361,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) koff[ks] = ((ks * 2 + lhalf) ^ sw) * 16;
     const int xrow_off = (wm * C::WTM + l32) * BK;
-    const int wrow_off = C::X_ALLOC + (wn * C::WTN + l32) * BK;
+    const int wrow_off = (wn * C::WTN + l32) * BK;
     // 16x16x64 form: a fragment is 16 rows x 64 k; lane l fetches the 16 bytes of row l % 16 at k-chunk l / 16 of the
     // k-step (any k order will do as long as both operands use the same one).  The swizzle looks at the low five bits
     // of the row, so the odd 16-row groups have their own chunk offsets.  Which chunk a lane quarter takes is chosen so
@@ -357,25 +375,35 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
 #pragma unroll
         for (int hp = 0; hp < 2; ++hp) koff16[kk][hp] = ((kk * 4 + lchunk) ^ swz<CPR>(hp * 16 + l16)) * 16;
     [[maybe_unused]] const int xrow16 = (wm * C::WTM + l16) * BK;
-    [[maybe_unused]] const int wrow16 = C::X_ALLOC + (wn * C::WTN + l16) * BK;
+    [[maybe_unused]] const int wrow16 = (wn * C::WTN + l16) * BK;
+    // (a wave tile of 48 columns starts on an odd 16-row group of the W tile in every other wave: its column fragments
+    // then take the chunk offsets of the other parity)
+    [[maybe_unused]] int koffw[2][2];
+    {
+        const bool odd = (C::WTN % 32 != 0) && ((wn * (C::WTN / 16)) & 1);
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int hp = 0; hp < 2; ++hp) koffw[kk][hp] = odd ? koff16[kk][hp ^ 1] : koff16[kk][hp];
+    }
 
-    // accumulators: per 32 x 32 block sixteen values per lane, as four quads of 4 consecutive n.
+    // accumulators: per block (32 rows x CB columns) QPB quads of 4 consecutive n per lane.
     //   32x32x32: quad qd holds n = 8 qd + 4 (lane / 32) + e of row m = lane % 32
-    //   16x16x64: quad qd = 2 u + v holds n = 16 v + 4 (lane / 16) + e of row m = 16 u + lane % 16
-    v16i acc[M16 ? 1 : MI][M16 ? 1 : NI];
-    v4i acc16[M16 ? MI : 1][M16 ? NI : 1][4];
+    //   16x16x64: quad qd holds n = 4 (lane / 16) + e of row m = 16 qd + lane % 16
+    v16i acc[M16 ? 1 : MI][M16 ? 1 : NJ];
+    v4i acc16[M16 ? MI : 1][M16 ? NJ : 1][2];
     if constexpr (M16) {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
-                for (int qd = 0; qd < 4; ++qd) acc16[i][j][qd] = (v4i)0;
+                for (int qd = 0; qd < 2; ++qd) acc16[i][j][qd] = (v4i)0;
     } else {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
     }
@@ -388,15 +416,15 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         if constexpr (M16) acc16[i][j][qd] += v;
         else acc[i][j][4 * qd] += v.x, acc[i][j][4 * qd + 1] += v.y, acc[i][j][4 * qd + 2] += v.z, acc[i][j][4 * qd + 3] += v.w;
     };
-    auto quad_m = [&](int qd) { return M16 ? (qd >> 1) * 16 + l16 : l32; };              // row inside the 32-row strip
-    auto quad_n = [&](int qd) { return M16 ? (qd & 1) * 16 + lq * 4 : qd * 8 + lhalf * 4; };  // first column inside the block
-    auto quad_c = [&](int qd) constexpr { return M16 ? (qd & 1) : qd; };                  // which of the NQ column quads
+    auto quad_m = [&](int qd) { return M16 ? qd * 16 + l16 : l32; };              // row inside the 32-row strip
+    auto quad_n = [&](int qd) { return M16 ? lq * 4 : qd * 8 + lhalf * 4; };      // first column inside the block
+    auto quad_c = [&](int qd) constexpr { return M16 ? 0 : qd; };                 // which of the NQ column positions
 
-    // Fragment registers per phase.  32x32x32: MI + NI fragments of one k-step of 32.  16x16x64: a phase is one half of
-    // the wave tile's rows (MI fragments of 16 rows) against all 2 NI column fragments for a k-step of 64; phases 0, 1
+    // Fragment registers per phase.  32x32x32: MI + NJ fragments of one k-step of 32.  16x16x64: a phase is one half of
+    // the wave tile's rows (MI fragments of 16 rows) against all NJ column fragments for a k-step of 64; phases 0, 1
     // share the column fragments of k-step 0, phases 2, 3 those of k-step 1.
-    constexpr int XF = MI, WF = M16 ? 2 * NI : NI;
-    constexpr int MN = M16 ? MI * 2 * NI : MI * NI;  // MFMAs per phase
+    constexpr int XF = MI, WF = NJ;
+    constexpr int MN = MI * NJ;  // MFMAs per phase
     auto load_x = [&](const char *st, int ph, v4i (&xf)[XF]) {
         if constexpr (M16) {
             const int h = ph & 1, kk = (ph >> 1) & 1;
@@ -414,23 +442,23 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         if constexpr (M16) {
             const int kk = (ph >> 1) & 1;
 #pragma unroll
-            for (int jj = 0; jj < WF; ++jj) wf[jj] = *(const v4i *)(st + wrow16 + jj * 16 * BK + koff16[kk][jj & 1]);
+            for (int jj = 0; jj < WF; ++jj) wf[jj] = *(const v4i *)(st + wrow16 + jj * 16 * BK + koffw[kk][jj & 1]);
         } else {
 #pragma unroll
-            for (int j = 0; j < NI; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ph]);
+            for (int j = 0; j < NJ; ++j) wf[j] = *(const v4i *)(st + wrow_off + j * 32 * BK + koff[ph]);
         }
     };
-    auto load_frags = [&](const char *st, int ph, v4i (&xf)[XF], v4i (&wf)[WF]) {
-        load_w(st, ph, wf);
-        load_x(st, ph, xf);
+    auto load_frags = [&](const char *xst, const char *wst, int ph, v4i (&xf)[XF], v4i (&wf)[WF]) {
+        load_w(wst, ph, wf);
+        load_x(xst, ph, xf);
     };
     auto mma_one = [&](const v4i (&xf)[XF], const v4i (&wf)[WF], int ph, int r) {
         if constexpr (M16) {
             const int jj = r / MI, t = r % MI, ii = (ph & 1) * MI + t;  // a column fragment is done with after MI MFMAs
-            v4i &a = acc16[ii >> 1][jj >> 1][(ii & 1) * 2 + (jj & 1)];
+            v4i &a = acc16[ii >> 1][jj][ii & 1];
             a = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[jj], xf[t], a, 0, 0, 0);
         } else {
-            const int i = r / NI, j = r % NI;
+            const int i = r / NJ, j = r % NJ;
             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[j], xf[i], acc[i][j], 0, 0, 0);
         }
     };
@@ -453,11 +481,14 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         return c;
     };
     static_assert(SPREAD_DMA || cut(KS) == C::LOADS, "the split has to cover every load of a tile");
+    // W one stage ahead: the X tile goes out first behind the barrier (all of it), the W tile, which has a K-tile more
+    // to land, in the phases after; at any barrier the loads that may still be in flight are that one W tile's
+    static_assert(!ASYM || (!SPREAD_DMA && cut(1) == C::X_LOADS), "X behind the barrier, W in the phases that follow");
 #pragma unroll
     for (int s = 0; s < PRE; ++s) {
         if (!SPREAD_DMA && s == PRE - 1) {
 #pragma unroll
-            for (int r = 0; r < cut(1); ++r) issue_one(s, s < KT, r);  // the rest follows inside the loop
+            for (int r = 0; r < (ASYM ? C::LOADS : cut(1)); ++r) issue_one(s, s < KT, r);  // the rest follows inside the loop
         } else {
             issue(s, s < KT);
         }
@@ -489,7 +520,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         }
     }
 
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(SPREAD_DMA ? (PRE - 1) * C::LOADS : cut(1)));  // younger tiles may be in flight
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(SPREAD_DMA ? (PRE - 1) * C::LOADS : (ASYM ? C::LOADS : cut(1))));  // younger tiles may be in flight
     __builtin_amdgcn_s_barrier();  // tile 0 is in LDS for everyone (no fence: nothing else has been written)
 
     // Fragments are double-buffered in registers: the LDS reads of k-step s+1 are issued before
@@ -498,14 +529,19 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // (its last fragments are in registers), so the stage of tile kt is refilled with tile kt+S
     // right away, and tile kt+1 is known to have landed, so its first fragments can be fetched.
     v4i xa[XF] = {}, wa[WF] = {}, xb[XF] = {}, wb[WF] = {};
-    if (KT > 0) load_frags(smem, 0, xa, wa);
+    if (KT > 0) load_frags(smem, smem + C::W_BASE, 0, xa, wa);
     // Drain scalar loads (kernel arguments) here: a scalar load still pending at the loop header
     // would turn every LDS wait inside the loop into a full lgkmcnt(0).
     __builtin_amdgcn_s_waitcnt(0xC07F);
 
+    int ix = 0, iw = 0;  // kt % S, kt % WS: the stages that hold tile kt
     for (int kt = 0; kt < KT; ++kt) {
-        const char *st = smem + (kt % S) * C::STAGE_BYTES;
-        const char *nx = smem + ((kt + 1) % S) * C::STAGE_BYTES;
+        if constexpr (!ASYM) iw = ix;  // (one index: the W tile then sits at a constant distance from its X tile)
+        const int ix1 = ix + 1 == S ? 0 : ix + 1, iw1 = ASYM ? (iw + 1 == WS ? 0 : iw + 1) : ix1;      // ... tile kt + 1
+        const int ixp = ix == 0 ? S - 1 : ix - 1, iwp = ASYM ? (iw == 0 ? WS - 1 : iw - 1) : ixp;      // ... held tile kt - 1
+        const char *xst = smem + ix * C::X_STRIDE, *xnx = smem + ix1 * C::X_STRIDE;
+        const char *wst = ASYM ? smem + C::W_BASE + iw * C::W_STRIDE : xst + C::W_BASE;
+        const char *wnx = ASYM ? smem + C::W_BASE + iw1 * C::W_STRIDE : xnx + C::W_BASE;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const bool last = ks == KS - 1;
@@ -513,7 +549,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                 // my part of tile kt+1 has landed and my LDS reads of tile kt have returned; what may
                 // still be in flight are the younger tiles (and, spread, the part of the newest one
                 // that the earlier phases of this iteration have issued)
-                constexpr int YOUNGER = SPREAD_DMA ? (S - 3) * C::LOADS + (KS - 1) * C::LOADS / KS : 0;
+                constexpr int YOUNGER = SPREAD_DMA ? (S - 3) * C::LOADS + (KS - 1) * C::LOADS / KS : (ASYM ? C::W_LOADS : 0);
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(YOUNGER) & 0xF0FF);
                 __builtin_amdgcn_s_barrier();
             }
@@ -523,18 +559,20 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
             v4i(&wc)[WF] = (!M16 && (ks & 1)) ? wb : wa;
             v4i(&wn_)[WF] = (M16 || (ks & 1)) ? wa : wb;
             // past the last tile the next-fragment reads fetch stale LDS that nobody uses
-            const char *fsrc = last ? nx : st;
+            const char *fx = last ? xnx : xst, *fw = last ? wnx : wst;
             const int fks = last ? 0 : ks + 1;
             // 32x32x32: the next phase's fragments are requested in front of this phase's MFMAs.  16x16x64: one fragment
             // behind each of the first MFMAs instead (a 16-cycle MFMA covers three or four other instructions, not a
             // burst of eight LDS reads with their address arithmetic, and the two waves of a SIMD run in step).
-            if constexpr (!M16) load_frags(fsrc, fks, xn, wn_);
+            if constexpr (!M16) load_frags(fx, fw, fks, xn, wn_);
             __builtin_amdgcn_sched_barrier(0);
             // the tile being fetched: two stages refill the stage that this iteration's barrier frees
             // (tile kt+2) from the last phase on and finish in the following phases of the next iteration
-            const int ft = SPREAD_DMA ? kt + S - 1 : (last ? kt + S : kt + S - 1);
-            const bool live = ft < KT;
-            (void)live;
+            // (the stage freed by the previous barrier, or from the last phase on by this iteration's: each operand's
+            // tile is the one its stage count puts there)
+            const bool behind = !SPREAD_DMA && last;
+            const int ftx = kt + S - (behind ? 0 : 1), ftw = kt + WS - (behind ? 0 : 1);
+            const int fsx = behind ? ix : ixp, fsw = behind ? iw : iwp;
             // this phase's share of its loads
             const int la = SPREAD_DMA ? ks * C::LOADS / KS : (last ? 0 : cut(ks + 1));
             const int lb = SPREAD_DMA ? (ks + 1) * C::LOADS / KS : (last ? cut(1) : cut(ks + 2));
@@ -547,15 +585,18 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                     const int kk = (fks >> 1) & 1;
                     if ((ks & 1) && r % MI == MI - 1) {  // the k-step ends with this phase: the column fragment is free
                         const int jj = r / MI;
-                        wn_[jj] = *(const v4i *)(fsrc + wrow16 + jj * 16 * BK + koff16[kk][jj & 1]);
+                        wn_[jj] = *(const v4i *)(fw + wrow16 + jj * 16 * BK + koffw[kk][jj & 1]);
                     } else if (l0 == l1 && frag < XF) {  // a slot with nothing else to issue takes a row fragment
                         const int ii = (fks & 1) * MI + frag;
-                        xn[frag] = *(const v4i *)(fsrc + xrow16 + ii * 16 * BK + koff16[kk][ii & 1]);
+                        xn[frag] = *(const v4i *)(fx + xrow16 + ii * 16 * BK + koff16[kk][ii & 1]);
                         ++frag;
                     }
                 }
 #pragma unroll
-                for (int l = l0; l < l1; ++l) issue_one(ft, live, l);
+                for (int l = l0; l < l1; ++l) {
+                    const int ft = l < C::X_LOADS ? ftx : ftw;
+                    issue_to(ft, fsx, fsw, ft < KT, l);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (M16) {  // (a phase with fewer free slots than row fragments)
@@ -564,18 +605,20 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                 for (int f = 0; f < XF; ++f) {
                     if (f >= frag) {
                         const int ii = (fks & 1) * MI + f;
-                        xn[f] = *(const v4i *)(fsrc + xrow16 + ii * 16 * BK + koff16[kk][ii & 1]);
+                        xn[f] = *(const v4i *)(fx + xrow16 + ii * 16 * BK + koff16[kk][ii & 1]);
                     }
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        ix = ix1, iw = iw1;
     }
 
     // ---- epilogue ----------------------------------------------------------------------
     // The loads issued past the last tile move no data from memory but still zero-fill their LDS
     // destination: they must have landed before the stages are reused.
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __builtin_amdgcn_s_barrier();  // every wave is done with the stages: the epilogue operands may go where they were
     if constexpr (SPLITK) {
         // Every slice leaves its sums in memory (in register order: thread t of the workgroup writes 16 bytes at
         // 16 (q NT + t) of its block for its q-th group of four) and counts itself in; the slice that arrives
@@ -586,12 +629,13 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         // invalidate, which a release/acquire fence pair at agent scope would cost every workgroup on the XCD.
         __shared__ unsigned s_arrived;
         const int T = tiles_m * tiles_n, tile = __builtin_amdgcn_readfirstlane((int)blockIdx.x % T);
-        constexpr int QUADS = MI * NI * 4;
+        constexpr int QUADS = MI * NJ * QPB;
+        static_assert(QUADS % 4 == 0, "the partial sums are read back four quads at a time");
         int *mine = g.partials + ((int64_t)slice * T + tile) * (BM * BN);
 #pragma unroll
         for (int qd = 0; qd < QUADS; ++qd) {
-            const int i = qd / (NI * 4), j = qd / 4 % NI;
-            const v4i o = quad_of(i, j, qd % 4);
+            const int i = qd / (NJ * QPB), j = qd / QPB % NJ;
+            const v4i o = quad_of(i, j, qd % QPB);
             // (s_nop 1: a 16-byte store reads its data registers after it has issued, and the two wait states that keep a
             // following vector instruction from overwriting them are the compiler's job, which it cannot do for an
             // instruction it does not see)
@@ -616,8 +660,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                              : "memory");
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int qd = q0 + u, i = qd / (NI * 4), j = qd / 4 % NI;
-                    quad_add(i, j, qd % 4, v[u]);
+                    const int qd = q0 + u, i = qd / (NJ * QPB), j = qd / QPB % NJ;
+                    quad_add(i, j, qd % QPB, v[u]);
                 }
             }
         }
@@ -656,20 +700,20 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // the activation scales of the lane's rows of strip i: one row, or (16x16x64) one per 16-row half
     auto strip_scales = [&](int i, float (&xs2)[2]) {
         xs2[0] = s_xs[wm * C::WTM + i * 32 + quad_m(0)];
-        xs2[1] = M16 ? s_xs[wm * C::WTM + i * 32 + quad_m(2)] : xs2[0];
+        xs2[1] = M16 ? s_xs[wm * C::WTM + i * 32 + quad_m(1)] : xs2[0];
     };
     auto convert_strip = [&](int i, char *dst_rows, const auto &wr, const auto &br, auto ORDER, auto ROW, auto BIAS) {
         float xs2[2];
         strip_scales(i, xs2);
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
+        for (int j = 0; j < NJ; ++j) {
 #pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int nl = j * 32 + quad_n(qd);  // first of 4 consecutive n held by this lane
+            for (int qd = 0; qd < QPB; ++qd) {
+                const int nl = j * CB + quad_n(qd);  // first of 4 consecutive n held by this lane
                 const v4i q4 = quad_of(i, j, qd);
                 const int a4[4] = {q4.x, q4.y, q4.z, q4.w};
                 epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value>(
-                    a4, xs2[qd >> 1], wr[j][quad_c(qd)], br[j][quad_c(qd)], dst_rows + quad_m(qd) * PITCH + nl * OB);
+                    a4, xs2[M16 ? qd : 0], wr[j][quad_c(qd)], br[j][quad_c(qd)], dst_rows + quad_m(qd) * PITCH + nl * OB);
             }
         }
     };
@@ -683,17 +727,17 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // the instructions a wave executes are contiguous in memory (the epilogue runs once per wave,
     // straight from a cold instruction cache).
     // With more than 8 waves a wave has fewer registers than the accumulators plus the operands of
-    // all its columns need: the column operands are then fetched per 32-column block, and a block is
+    // all its columns need: the column operands are then fetched per column block, and a block is
     // converted for all staged strips before the next one is fetched.
     // (the variant with a low-rank side branch needs registers for its operands: per-block fetches as well)
     constexpr bool PRELOAD_ALL = C::NT <= 512 && !SIDE;
     auto run_epilogue = [&](auto ORDER, auto ROW, auto BIAS) {
-        constexpr int NPRE = PRELOAD_ALL ? NI : 1;
+        constexpr int NPRE = PRELOAD_ALL ? NJ : 1;
         float4 wr[NPRE][NQ], br[NPRE][NQ];
         auto fetch_cols = [&](int j, float4 (&wj)[NQ], float4 (&bj)[NQ]) __attribute__((always_inline)) {
 #pragma unroll
             for (int c = 0; c < NQ; ++c) {
-                const int nl = wn * C::WTN + j * 32 + quad_n(c);  // (16x16x64: quads 0 and 1 are the two distinct ones)
+                const int nl = wn * C::WTN + j * CB + quad_n(c);
                 if constexpr (decltype(ROW)::value) wj[c] = *(const float4 *)&s_ws[nl];
                 else wj[c] = make_float4(s_ws[0], s_ws[0], s_ws[0], s_ws[0]);
                 if constexpr (decltype(BIAS)::value) bj[c] = *(const float4 *)&s_bias[nl];
@@ -702,7 +746,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         };
         if constexpr (OUT != OUT_I32 && PRELOAD_ALL) {
 #pragma unroll
-            for (int j = 0; j < NI; ++j) fetch_cols(j, wr[j], br[j]);
+            for (int j = 0; j < NJ; ++j) fetch_cols(j, wr[j], br[j]);
         }
 #pragma unroll
         for (int i0 = 0; i0 < MI; i0 += EPI_STRIPS) {
@@ -712,10 +756,10 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                 char *rows = ebuf + is * 32 * PITCH;
                 if constexpr (OUT == OUT_I32) {
 #pragma unroll
-                    for (int j = 0; j < NI; ++j)
+                    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-                        for (int qd = 0; qd < 4; ++qd) {
-                            const int nl = j * 32 + quad_n(qd);
+                        for (int qd = 0; qd < QPB; ++qd) {
+                            const int nl = j * CB + quad_n(qd);
                             *(v4i *)(rows + quad_m(qd) * PITCH + nl * 4) = quad_of(i, j, qd);
                         }
                 } else if constexpr (PRELOAD_ALL) {
@@ -724,15 +768,15 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
             }
             if constexpr (OUT != OUT_I32 && !PRELOAD_ALL) {
 #pragma unroll
-                for (int j = 0; j < NI; ++j) {
+                for (int j = 0; j < NJ; ++j) {
                     fetch_cols(j, wr[0], br[0]);
-                    // side branch: the rank-r product of this 32 x 32 block on the matrix cores, with the same
+                    // side branch: the rank-r product of this block on the matrix cores, with the same
                     // operand roles as the main product (rows n from side_b, columns m from side_t), so that
                     // the result has the accumulators' layout
-                    // (16x16x64 form: four 16 x 16 products per block, a lane's fragment being 4 ranks of one row)
+                    // (16x16x64 form: two 16 x 16 products per block, a lane's fragment being 4 ranks of one row)
                     constexpr int RMAX = 64;
                     [[maybe_unused]] v4i bfr[M16 ? 1 : RMAX / 16];
-                    [[maybe_unused]] v2i bfr16[M16 ? 2 : 1][RMAX / 16];
+                    [[maybe_unused]] v2i bfr16[RMAX / 16];
                     if constexpr (SIDE && !M16) {
                         const int n = min(n0 + wn * C::WTN + j * 32 + l32, gN - 1);
 #pragma unroll
@@ -741,14 +785,11 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                                 bfr[ks] = *(const v4i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lhalf * 8) * 2);
                     }
                     if constexpr (SIDE && M16) {
+                        const int n = min(n0 + wn * C::WTN + j * 16 + l16, gN - 1);
 #pragma unroll
-                        for (int v = 0; v < 2; ++v) {
-                            const int n = min(n0 + wn * C::WTN + j * 32 + v * 16 + l16, gN - 1);
-#pragma unroll
-                            for (int ks = 0; ks < RMAX / 16; ++ks)
-                                if (ks * 16 < g.side_rank)
-                                    bfr16[v][ks] = *(const v2i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lq * 4) * 2);
-                        }
+                        for (int ks = 0; ks < RMAX / 16; ++ks)
+                            if (ks * 16 < g.side_rank)
+                                bfr16[ks] = *(const v2i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lq * 4) * 2);
                     }
 #pragma unroll
                     for (int is = 0; is < EPI_STRIPS; ++is) {
@@ -780,32 +821,29 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
 #pragma unroll
                             for (int u = 0; u < 2; ++u) {
                                 const int m = min(m0 + wm * C::WTM + i * 32 + u * 16 + l16, gM - 1);
-                                v4f sacc[2] = {(v4f)0.0f, (v4f)0.0f};
+                                v4f sacc = (v4f)0.0f;
 #pragma unroll
                                 for (int ks = 0; ks < RMAX / 16; ++ks) {
                                     if (ks * 16 < g.side_rank) {
                                         const v2i tfr = *(const v2i *)((const char *)g.side_t + ((int64_t)m * g.side_rank + ks * 16 + lq * 4) * 2);
-#pragma unroll
-                                        for (int v = 0; v < 2; ++v) sacc[v] = side_mfma16<OUT>(bfr16[v][ks], tfr, sacc[v]);
+                                        sacc = side_mfma16<OUT>(bfr16[ks], tfr, sacc);
                                     }
                                 }
 #pragma unroll
-                                for (int v = 0; v < 2; ++v)
-#pragma unroll
-                                    for (int e = 0; e < 4; ++e) {
-                                        float y = round_to_dtype<SDT>(sacc[v][e]);
-                                        if (g.side_has_alpha) y = round_to_dtype<SDT>(y * g.side_alpha);
-                                        sd[4 * (u * 2 + v) + e] = y;
-                                    }
+                                for (int e = 0; e < 4; ++e) {
+                                    float y = round_to_dtype<SDT>(sacc[e]);
+                                    if (g.side_has_alpha) y = round_to_dtype<SDT>(y * g.side_alpha);
+                                    sd[4 * u + e] = y;
+                                }
                             }
                         }
 #pragma unroll
-                        for (int qd = 0; qd < 4; ++qd) {
-                            const int nl = j * 32 + quad_n(qd);
+                        for (int qd = 0; qd < QPB; ++qd) {
+                            const int nl = j * CB + quad_n(qd);
                             const v4i q4 = quad_of(i, j, qd);
                             const int a4[4] = {q4.x, q4.y, q4.z, q4.w};
                             epilogue_quad<OUT, decltype(ORDER)::value, decltype(ROW)::value, decltype(BIAS)::value, SIDE>(
-                                a4, xs2[qd >> 1], wr[0][quad_c(qd)], br[0][quad_c(qd)], ebuf + (is * 32 + quad_m(qd)) * PITCH + nl * OB,
+                                a4, xs2[M16 ? qd : 0], wr[0][quad_c(qd)], br[0][quad_c(qd)], ebuf + (is * 32 + quad_m(qd)) * PITCH + nl * OB,
                                 SIDE ? &sd[4 * qd] : nullptr);
                         }
                     }
@@ -900,11 +938,17 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
 // reach 4.9), so the clock settles higher.  The shorter instruction covers fewer other instructions, which is why that form
 // deals its LDS reads out one by one; the 128 x 128 tile and the few-tile configurations (one wave per SIMD, bound by the
 // global->LDS path) lose more to that than they gain and keep the 32x32x32 form.
-using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400, 16>;  // 8 waves, 2 x 64 KB stages, one workgroup per CU; refill in two halves (2-3 % faster than one burst)
-using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6, 0, 16>;  // 8 waves of 64 x 96, 2 x 56 KB stages: fills 256 CUs where 256 x 256 leaves a partial round
+#ifndef I8F_WST
+#define I8F_WST 3
+#endif
+using CfgBig = Cfg<256, 256, 128, 2, 4, 2, 6, 0x4400, 16, I8F_WST>;  // 8 waves, 2 X and 3 W stages of 32 KB (all of the LDS), one workgroup per CU
+using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6, 0x4300, 16, I8F_WST>;  // 8 waves of 64 x 96, 2 x 32 + 3 x 24 KB: fills 256 CUs where 256 x 256 leaves a partial round
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU (10 % slower with the 16x16x64 MFMA: 32x32x32)
 using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8, 0, 16>;  // 12 waves of 96 x 64, 2 x 72 KB stages
 using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8, 0, 16>;  // 12 waves of 64 x 96, the same transposed
+// (A 288 x 192 tile of twelve 96 x 48 waves, which covers 4608 x 3072 in exactly 256 workgroups, was measured and is not
+// kept: 42.9 us against 37.7 us for the 216 tiles of 256 x 256.  It moves 11 % more bytes per multiply-accumulate through a
+// load path that is already the bound, and with all 256 CUs multiplying the clock settles 8 % lower.)
 // Outputs of few tiles: about one workgroup per CU, so nothing hides the latency of the global->LDS
 // loads (the weight comes from HBM: a model's weights are far larger than the caches) but the loads in
 // flight; four stages instead of two, and the largest tile that still gives 192 workgroups.
