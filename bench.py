@@ -205,6 +205,16 @@ def extras(L, dev, quick=False):
                                           "cold_operands_median_us": round(tc["median_us"], 2), "cold_operands_tops": round(tops_c, 1),
                                           "cold_operands_frac_of_int8_peak": round(tops_c / PEAK_INT8_TOPS, 4),
                                           "tile": "%dx%d" % L.gemm_tile(M, N, K)[:2]}
+    # the vendor library's int8 product on the same box and operands (torch._int_mm = hipBLASLt: int32 result, no
+    # epilogue, so it does less than the launch above), warm loop like the first figure; bench-only, not product code
+    try:
+        wt = wq.t()
+        t_v = time_kernel(lambda i: torch._int_mm(q, wt), max(10, iters // 4), burst=8)
+        out["target_gemm_4608x3072x3072"]["vendor_int_mm_median_us"] = round(t_v["median_us"], 2)
+        out["target_gemm_4608x3072x3072"]["vendor_int_mm_note"] = "torch._int_mm(q, w.T): int32 accumulators only, no dequantisation epilogue"
+    except Exception as e:   # a torch build without the routine says so in the line
+        out["target_gemm_4608x3072x3072"]["vendor_int_mm_median_us"] = None
+        out["target_gemm_4608x3072x3072"]["vendor_int_mm_note"] = f"torch._int_mm unavailable: {type(e).__name__}"
     del cq, cw, cy
 
     # fused rotate + quant at the same shape, cycling 8 buffer sets (> 256 MB in total), bursts of 8

@@ -281,23 +281,37 @@ def _bias_arg(bias, N, device):
 
 
 _SPLITK_WORKSPACES = {}
+_SPLITK_COUNTER_BYTES = 4096
 
 
 def _splitk_workspace(t: torch.Tensor, M: int, N: int, K: int):
-    """The K-split workspace of (device, current stream) for shapes that can use one (a long K and few output
-    tiles), else None.  Allocated and zeroed once; launches on one stream run one after the other, so they can share
-    it.  None while a graph is being captured and there is none yet (memory allocated during a capture belongs to
-    the graph)."""
+    """The K-split workspace for shapes that can use one (a long K and few output tiles), else None.
+
+    The library's contract is one launch at a time per workspace (launches that overlap in time race on the partial
+    sums).  Eager calls: one workspace per (device, stream), allocated and zeroed once and kept until
+    clear_splitk_workspaces(); launches on one stream run one after the other, so they can share it.  While the
+    stream is capturing a graph the eager workspace is never used (a replay of the graph on another stream could
+    overlap eager calls on this one): the call gets a workspace of its own from the graph's memory pool, with a
+    fill kernel in front of it that clears the arrival words on every replay, and the memory goes back to the pool
+    of the graph when the call returns (later nodes of the same graph run after this one)."""
     if K < 10240 or M * N > 128 * 128 * 128:
         return None
+    nbytes = lib().i8f_linear_w8a8_workspace_bytes()
+    if torch.cuda.is_current_stream_capturing():
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=t.device)
+        ws[:_SPLITK_COUNTER_BYTES].zero_()
+        return ws
     key = (t.device.index, torch.cuda.current_stream(t.device).cuda_stream)
     ws = _SPLITK_WORKSPACES.get(key)
     if ws is None:
-        if torch.cuda.is_current_stream_capturing():
-            return None
-        ws = torch.zeros(lib().i8f_linear_w8a8_workspace_bytes(), dtype=torch.uint8, device=t.device)
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=t.device)
         _SPLITK_WORKSPACES[key] = ws
     return ws
+
+
+def clear_splitk_workspaces() -> None:
+    """Drop the cached K-split workspaces (16 MB per device and stream that used one); the next call allocates anew."""
+    _SPLITK_WORKSPACES.clear()
 
 
 def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None, addend=None):
@@ -340,6 +354,16 @@ def lora_side_fusable(M: int, N: int, K: int, rank: int, out_dtype, side_dtype) 
     """Whether linear_w8a8_lora takes this problem (else: a side tensor and linear_w8a8(addend=...))."""
     return (out_dtype in (torch.bfloat16, torch.float16) and side_dtype == out_dtype and 0 < rank <= 64
             and K % 128 == 0 and N % 8 == 0 and M > 0)
+
+
+def lora_side_pays(M: int, N: int, K: int) -> bool:
+    """Whether the side branch inside the epilogue is the cheaper way to add a low-rank product to this GEMM.  The
+    fused form exists for the eight-wave tiles: a problem whose plain GEMM takes a twelve-wave tile (288 x 256 or
+    256 x 288, e.g. 4608 x 12288 x 3072) would fall back to 256 x 256 tiles and lose more than the [M,N] side tensor
+    costs (measured 202 us fused against 199 us with a side tensor added in the epilogue), so such problems form
+    the side tensor with torch and add it in the epilogue."""
+    bm, bn, _stages = gemm_tile(M, N, K)
+    return (bm, bn) not in ((288, 256), (256, 288))
 
 
 def linear_w8a8_lora(a, a_scale, w, w_scale, bias, side_t, side_b, alpha=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None):

@@ -135,12 +135,23 @@ def _is_call(node, *targets):
     return node.op == "call_function" and node.target in targets
 
 
+def _meta_shape(node):
+    v = node.meta.get("example_value", node.meta.get("val")) if isinstance(node, torch.fx.Node) else None
+    return None if v is None else tuple(v.shape)
+
+
 def _through_views(node):
-    """The producer of `node` behind shape-only steps that have no other user."""
+    """The producer of `node` behind shape-only steps that have no other user and only regroup the LEADING
+    dimensions: a step whose traced shapes do not show the same last dimension on both sides (a view that splits or
+    merges the feature dimension, or a graph without shape metadata) ends the walk."""
     while isinstance(node, torch.fx.Node) and len(node.users) == 1 and (
             (node.op == "call_method" and node.target in _VIEW_METHODS)
             or _is_call(node, torch.reshape, torch.flatten)):
-        node = node.args[0]
+        src = node.args[0]
+        out_shape, in_shape = _meta_shape(node), _meta_shape(src)
+        if not out_shape or not in_shape or out_shape[-1] != in_shape[-1]:
+            break
+        node = src
     return node
 
 
@@ -173,13 +184,18 @@ def _vectors_broadcast_over_tokens(x, scale, shift) -> bool:
     def meta(n):
         return n.meta.get("example_value", n.meta.get("val"))
 
-    def shape(n):
-        v = meta(n)
-        return None if v is None else tuple(v.shape)
-    xs, ss, ts = shape(x), shape(scale), shape(shift)
-    if xs is None or ss is None or ts is None or ss != ts or len(xs) < 2:
+    if any(not isinstance(n, torch.fx.Node) or meta(n) is None for n in (x, scale, shift)):
         return False
-    if not (meta(x).dtype == meta(scale).dtype == meta(shift).dtype):   # mixed dtypes promote in torch: leave them to it
+    return modulation_broadcasts_over_tokens(meta(x), meta(scale), meta(shift))
+
+
+def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
+    """Whether (1 + scale) * x + shift can run inside the quantiser: scale and shift of x's dtype and of one shape,
+    [K] or [.., 1, K] against x [.., T, K] with the same leading dimensions, i.e. one vector per leading index,
+    shared by the T rows that are consecutive rows of the flattened activations.  (Mixed dtypes promote in torch,
+    other shapes broadcast differently: those stay torch expressions.)"""
+    xs, ss, ts = tuple(x.shape), tuple(scale.shape), tuple(shift.shape)
+    if ss != ts or len(xs) < 2 or not (x.dtype == scale.dtype == shift.dtype):
         return False
     if len(ss) == 1:
         return ss[0] == xs[-1]
@@ -201,6 +217,9 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         src = _through_views(x_in)
         if not isinstance(src, torch.fx.Node):
             continue
+        x_shape = _meta_shape(x_in)
+        if x_shape is None:
+            continue
         h = _match_gelu(src)
         new_args = None
         if h is not None:
@@ -211,11 +230,18 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
                 new_args = (m[0], _lib.PRO_MODULATE, m[1], m[2])
         if new_args is None:
             continue
+        # The fused operator returns the leading shape of h, the original one that of x_in: the same when nothing
+        # sat between them; a layer that flattened h to 2-D gets its 2-D result back by a reshape; anything else
+        # (a direct caller with another regrouping of the rows) is left alone.
+        h_shape = _meta_shape(new_args[0])
+        if h_shape is None or h_shape[-1] != x_shape[-1]:
+            continue
+        if h_shape != x_shape and len(x_shape) != 2:
+            continue
         with gm.graph.inserting_before(node):
             fused = gm.graph.call_function(torch.ops.i8f.int8_linear_prologue,
                                            (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order))
-            # the layer flattened its input to 2-D and restores the leading shape itself: so does the operator
-            restored = gm.graph.call_method("reshape", (fused, -1, _out_features(weight)))
+            restored = fused if h_shape == x_shape else gm.graph.call_method("reshape", (fused, -1, _out_features(weight)))
         node.replace_all_uses_with(restored)
         gm.graph.erase_node(node)
         n_fused += 1

@@ -29,7 +29,9 @@
 #pragma once
 
 #include "i8f_common.hpp"
+#include "splitk_protocol.h"
 #include <algorithm>
+#include <atomic>
 
 namespace i8f {
 namespace gemm {
@@ -87,7 +89,8 @@ struct GemmArgs {
     // K split over `splits` workgroups per tile (1: none): partial sums and per-tile arrival counters in caller memory
     int splits;
     int *partials;          // [splits][tiles][BM * BN] int32, in the register order of the kernel
-    unsigned *arrivals;     // [tiles], zero before the launch and zero again after it
+    unsigned *arrivals;     // [tiles] arrival words (splitk_protocol.h); any contents before the launch, zero after it
+    unsigned splitk_tag;    // names this launch in the arrival words
 };
 
 // SPLIT_ (two-stage configurations): how a wave's loads of one K-tile are dealt over the phases that
@@ -643,7 +646,15 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == 0) s_arrived = __hip_atomic_fetch_add(g.arrivals + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) {
+            unsigned word = __hip_atomic_load(g.arrivals + tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), next;
+            uint32_t before;
+            do {
+                next = splitk_arrive(word, g.splitk_tag, (uint32_t)g.splits, &before);
+            } while (!__hip_atomic_compare_exchange_strong(g.arrivals + tile, &word, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT));
+            s_arrived = before;
+        }
         __syncthreads();
         if (s_arrived + 1 != (unsigned)g.splits) return;
         for (int o = 0; o < g.splits; ++o) {
@@ -1144,6 +1155,10 @@ int launch(GemmArgs &g, hipStream_t st) {
     int splits = 1;
     if (g.partials && !g.side_t) choose_split(g.M, g.N, g.K, t, splits);
     g.splits = splits;
+    if (splits > 1) {
+        static std::atomic<uint32_t> launches{0};
+        g.splitk_tag = splitk_tag(launches.fetch_add(1, std::memory_order_relaxed));
+    }
     return launch_tile<OUT>(t, g, st);
 }
 

@@ -416,6 +416,10 @@ class Int8TensorwiseOps(manual_cast):
                 rows = x.numel() // max(1, x.shape[-1])
                 fusable = (self._is_quantized and rows > SMALL_BATCH_ROWS and self.lora_A is None
                            and not torch.compiler.is_compiling())
+                if fusable and prologue == _lib.PRO_MODULATE:
+                    # vectors of another dtype or another broadcast pattern are torch's business (as under compile)
+                    fusable = (isinstance(mod_scale, Tensor) and isinstance(mod_shift, Tensor) and x.dim() >= 2
+                               and compile_ops.modulation_broadcasts_over_tokens(x, mod_scale, mod_shift))
                 if not fusable:   # every other path takes the operation as torch would have applied it
                     x = F.gelu(x, approximate="tanh") if prologue == _lib.PRO_GELU_TANH else (1 + mod_scale) * x + mod_shift
                     prologue = _lib.PRO_NONE
@@ -470,7 +474,8 @@ class Int8TensorwiseOps(manual_cast):
                 lora_x = F.linear(x_side.to(lA.dtype), lA)
                 rows = x_2d.shape[0]
                 if (not compiling and rows > SMALL_BATCH_ROWS and lB.dtype == lA.dtype
-                        and _lib.lora_side_fusable(rows, weight.shape[0], weight.shape[1], lA.shape[0], compute_dtype, lA.dtype)):
+                        and _lib.lora_side_fusable(rows, weight.shape[0], weight.shape[1], lA.shape[0], compute_dtype, lA.dtype)
+                        and _lib.lora_side_pays(rows, weight.shape[0], weight.shape[1])):
                     side_factors = (lora_x, lB, self.lora_alpha)
                 else:
                     side = F.linear(lora_x, lB)

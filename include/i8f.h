@@ -150,7 +150,9 @@ int i8f_quant_tensorwise(const void *x, int x_dtype, int64_t n, int8_t *q, float
  * the library, one copy per GPU, held until the process ends.  Same results as
  * i8f_quant_tensorwise bit for bit.
  * I8F_ERR_UNSUPPORTED for n > 2^32 elements.  Calls that overlap in time on one
- * GPU (different streams or threads) race on that array: serialise them.
+ * GPU (different streams or threads) race on that array: serialise them.  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress): make it outside
+ * a stream capture; later calls only launch kernels.
  */
 int i8f_quant_tensorwise_static(const void *x, int x_dtype, int64_t n, int8_t *q, float *scale,
                                 void *stream);
@@ -227,9 +229,15 @@ int i8f_linear_w8a8_add(const int8_t *a, const float *a_scale, const int8_t *w, 
  * sums do not depend on their order); the same Triton launches as i8f_linear_w8a8 (int8_fused_kernel.py:216,
  * 357), whose grids cover the output only.  512 x 3072 x 12288 with weights from HBM: 42 -> 34 us.
  *   workspace        device memory of i8f_linear_w8a8_workspace_bytes() bytes (16 MB + 4 KB), 16-byte aligned,
- *                    whose first 4096 bytes are ZERO before the first call; every call leaves them zero again.
- *                    One workspace serves any number of calls that do not overlap in time (one per stream);
- *                    NULL gives i8f_linear_w8a8_add exactly.
+ *                    whose first 4096 bytes (one arrival word per output tile) are ZERO before the first call;
+ *                    every call that completes leaves them zero again.  Each launch stamps its arrival words
+ *                    with a tag of its own and treats a word with another tag as "nobody has arrived", so the
+ *                    words a launch that never finished (killed, aborted) left behind do not poison the next
+ *                    one.  A captured launch is replayed with the tag it was captured with: a graph whose
+ *                    replays may be aborted should clear the 4096 bytes with a fill kernel in front of the call.
+ *                    One workspace serves any number of calls that do NOT OVERLAP IN TIME (one per stream, and
+ *                    not an eager call next to the replay of a graph that captured the same workspace): calls
+ *                    that overlap race on the partial sums.  NULL gives i8f_linear_w8a8_add exactly.
  * I8F_ERR_INVALID for a workspace that is too small or misaligned.
  */
 int64_t i8f_linear_w8a8_workspace_bytes(void);

@@ -125,6 +125,57 @@ def test_graph_rewrite_leaves_other_producers_alone(pkg):
     assert pkg.compile_ops.fuse_prologues(gm) == 0
 
 
+def test_graph_rewrite_respects_views_and_the_callers_shape(pkg):
+    """A view between the producer and the layer that regroups the FEATURE dimension is not walked through (the
+    quantiser would see rows of another length), and a direct 3-D caller of the operator keeps its 3-D result."""
+    m = _mlp(pkg, k=256, hidden=512)
+    ops = torch.ops.i8f
+
+    class Regrouped(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = m.up
+
+        def forward(self, x):                      # x [4, 24, 128]: gelu on rows of 128, the layer on rows of 256
+            return self.up(F.gelu(x, approximate="tanh").reshape(4, 12, 256))
+
+    gm = torch._dynamo.export(Regrouped())(torch.randn(4, 24, 128).bfloat16()).graph_module
+    assert pkg.compile_ops.fuse_prologues(gm) == 0
+
+    class Direct(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w = torch.nn.Parameter(m.up.weight.data, requires_grad=False)
+            self.ws = torch.nn.Parameter(m.up.weight_scale.data, requires_grad=False)
+
+        def forward(self, x):                      # the operator called on a 3-D tensor, as its schema allows
+            return ops.int8_linear(F.gelu(x, approximate="tanh"), self.w, self.ws, 0.0, None, torch.bfloat16, False, 0)
+
+    x = torch.randn(2, 24, 256).bfloat16()
+    gm = torch._dynamo.export(Direct())(x).graph_module
+    assert pkg.compile_ops.fuse_prologues(gm) == 1
+    outs = [n for n in gm.graph.nodes if n.op == "output"][0].args[0]
+    out = outs[0] if isinstance(outs, (tuple, list)) else outs
+    assert "int8_linear_prologue" in str(out.target), "no reshape to 2-D is put behind a 3-D caller's operator"
+    fake = torch._subclasses.FakeTensorMode()
+    with fake:
+        y = ops.int8_linear_prologue(torch.empty(2, 24, 256, dtype=torch.bfloat16), 2, None, None, torch.empty(512, 256, dtype=torch.int8),
+                                     torch.empty(512, 1), 0.0, None, torch.bfloat16, False, 0)
+    assert tuple(y.shape) == (2, 24, 512)
+
+
+def test_modulation_broadcast_rule(pkg):
+    ok = pkg.compile_ops.modulation_broadcasts_over_tokens
+    x = torch.empty(2, 24, 256, dtype=torch.bfloat16)
+    v = lambda *shape, dt=torch.bfloat16: torch.empty(*shape, dtype=dt)
+    assert ok(x, v(2, 1, 256), v(2, 1, 256)) and ok(x, v(256), v(256))
+    assert not ok(x, v(1, 24, 256), v(1, 24, 256))          # one vector per token of ONE image, broadcast over the batch
+    assert not ok(x, v(1, 1, 256), v(1, 1, 256))            # batch 2 against one pair of vectors: torch broadcasts, rows do not split
+    assert not ok(x, v(2, 1, 256, dt=torch.float32), v(2, 1, 256, dt=torch.float32))
+    assert not ok(x, v(2, 1, 256), v(256))
+    assert ok(torch.empty(1, 24, 256, dtype=torch.bfloat16), v(1, 1, 256), v(1, 1, 256))
+
+
 def _oracle_linear(O, x2d, lin):
     xa, code = O.from_torch(x2d)
     return O.linear_w8a8(xa, code, lin.weight.cpu().numpy(), lin.weight_scale.cpu().numpy().reshape(-1),

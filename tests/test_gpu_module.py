@@ -276,5 +276,12 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
         a = lin(x, prologue=L.PRO_GELU_TANH)
         b = lin(F.gelu(x, approximate="tanh"))
         assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
+    # vectors that torch would broadcast differently, or of another dtype, are left to torch: same result as the
+    # unfused expression (a [1, T, K] vector against a batch of 2 must not be dealt over the rows as if it were [2, 1, K])
+    lin._use_quarot = False
+    per_token = (torch.randn(1, 20, 384, generator=g) * 0.3).bfloat16().to(dev)
+    assert torch.equal(lin(x, prologue=L.PRO_MODULATE, mod_scale=per_token, mod_shift=per_token), lin((1 + per_token) * x + per_token))
+    sc32, sh32 = sc.float(), sh.float()
+    assert torch.equal(lin(x, prologue=L.PRO_MODULATE, mod_scale=sc32, mod_shift=sh32), lin((1 + sc32) * x + sh32))
     small = x[:1, :4]                     # four rows: the W8A16 path applies the operation in torch
     assert torch.equal(lin(small, prologue=L.PRO_GELU_TANH), lin(F.gelu(small, approximate="tanh")))

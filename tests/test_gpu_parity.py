@@ -347,10 +347,42 @@ def test_linear_w8a8_k_split_bit_exact(L, dev, M, N, K, odt):
     assert rc == 0 and torch.equal(plain.view(torch.uint8), got.view(torch.uint8))
 
 
+def test_linear_w8a8_k_split_on_leftover_arrival_words(L, dev):
+    """The arrival words of the K split as launches that never finished would have left them: another launch's tag
+    with every count a slice can leave, counts no slice can leave, all ones.  Every kernel still exits, the result
+    is the oracle's bit for bit, and the words are zero afterwards (a launch stamps the words with its own tag and
+    takes a word with another tag as `nobody has arrived`)."""
+    M, N, K = 64, 3072, 12288    # 64 x 64 tiles, five slices per tile
+    x = acts(M, K)
+    wq = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=G)
+    ws = (torch.rand(N, generator=G) * 0.002 + 0.0005)
+    xa, code = O.from_torch(x)
+    want = O.linear_w8a8(xa, code, wq.numpy(), ws.numpy(), None, O.BF16, O.BF16, 0, L.EPI_TORCH)
+    q, s = L.quant_rowwise(x.to(dev))
+    wd, wsd = wq.to(dev), ws.to(dev)
+    nbytes = L.lib().i8f_linear_w8a8_workspace_bytes()
+    work = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    words = work[:4096].view(torch.int32)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    stale_tag = 0x123456
+    leftovers = [[(stale_tag << 8) | c for c in (1, 2, 3, 4, 5)], [1, 2, 3, 4], [0xff, 0x7fffffff, -1, 0xabcdef07]]
+    for fill in leftovers:
+        words.copy_(torch.tensor([fill[i % len(fill)] for i in range(1024)], dtype=torch.int64).to(torch.int32))
+        out.zero_()
+        rc = L.lib().i8f_linear_w8a8_splitk(q.data_ptr(), s.data_ptr(), wd.data_ptr(), wsd.data_ptr(), 0.0, L.SCALE_ROW, None, L.BF16,
+                                            None, out.data_ptr(), L.BF16, M, N, K, L.EPI_TORCH, work.data_ptr(), nbytes, None)
+        torch.cuda.synchronize()
+        assert rc == 0
+        assert np.array_equal(bits(out), want), f"leftover words {fill[:3]}..."
+        tiles = (N + 63) // 64
+        assert int(words[:tiles].abs().sum()) == 0, "the words of the tiles in use are zero after a completed launch"
+
+
 def test_linear_w8a8_long_k_under_hip_graph_equals_eager(L, dev):
-    """A shape that takes the K split in eager mode, captured in a HIP graph: the Python layer allocates no workspace
-    while a stream is capturing (the capture then runs one workgroup per tile), and with or without the split every
-    replay gives the eager result bit for bit."""
+    """A shape that takes the K split, captured in a HIP graph: while a stream captures, the Python layer gives the
+    call a workspace from the graph's own memory pool with a fill kernel in front that clears the arrival words on
+    every replay (never the eager workspace of the stream), so the split is taken inside the graph too; every replay
+    gives the eager result bit for bit, with eager split launches between the replays."""
     M, N, K = 64, 1024, 12288
     q = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=G).to(dev)
     w = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=G).to(dev)
@@ -359,8 +391,18 @@ def test_linear_w8a8_long_k_under_hip_graph_equals_eager(L, dev):
     eager = L.linear_w8a8(q, s, w, ws)
     static_q = q.clone()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        static_y = L.linear_w8a8(static_q, s, w, ws)
+    seen = []
+    real = L._splitk_workspace
+    try:
+        L._splitk_workspace = lambda *a: seen.append(real(*a)) or seen[-1]
+        with torch.cuda.graph(graph):
+            static_y = L.linear_w8a8(static_q, s, w, ws)
+    finally:
+        L._splitk_workspace = real
+    eager_ws = real(q, M, N, K)
+    assert len(seen) == 1 and seen[0] is not None and seen[0].data_ptr() != eager_ws.data_ptr(), \
+        "the captured call has a workspace of its own"
+    del seen
     for i in range(3):
         q2 = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=G).to(dev)
         want = L.linear_w8a8(q2, s, w, ws)      # eager work (with the split) between the replays
@@ -604,13 +646,25 @@ def test_linear_w8a8_lora_side_branch(L, dev, M, N, K, r, dt, alpha, row):
     if alpha is not None:
         sd = (sd.float() * alpha).to(dt)
     want = (torch.from_numpy(y) + sd.float()).to(dt)
-    ulp = ULP[dt]
-    for ref in (want, unfused.cpu()):
-        d = (got.cpu().float() - ref.float()).abs()
-        # one ulp of the side value (it may round the other way, twice with alpha) plus one of the sum
-        bound = 2 * ulp * (2 * sd.float().abs() + ref.float().abs()) + 1e-6   # (the spacing of the dtype is up to 2 ulp * |v|)
-        assert (d <= bound).all(), f"max excess {(d - bound).max().item()} at {(d - bound).argmax().item()}"
-        assert (d != 0).float().mean().item() <= 0.01
+    # Element by element: the result is round(y + s') where s' is the reference's side value or a NEIGHBOUR of it in the
+    # dtype (one step when the rank-r sum rounds the other way, two with alpha, whose product is rounded again): nothing
+    # else is allowed, and all but 1 % of the elements take the reference's side value itself.
+    steps = 1 if alpha is None else 2
+    yt = torch.from_numpy(y)
+    for side_ref, ref in ((sd, want), (side.cpu().to(dt), unfused.cpu())):
+        ok = torch.zeros(got.shape, dtype=torch.bool)
+        for k in range(-steps, steps + 1):
+            ok |= _raw16((yt + step_16(side_ref, k).float()).to(dt)) == _raw16(got.cpu())
+        assert ok.all(), f"{(~ok).sum().item()} elements are not y + (side value or a neighbour), first at {(~ok).flatten().nonzero()[0].item()}"
+        assert (_raw16(got.cpu()) != _raw16(ref)).float().mean().item() <= 0.01
+
+
+def step_16(t, k):
+    """t (bfloat16 / float16) moved k representable values up (k < 0: down), through zero if need be."""
+    b = t.contiguous().view(torch.int16).to(torch.int32)
+    o = torch.where(b < 0, -(b & 0x7fff), b) + k          # sign-magnitude patterns as ordered integers
+    b2 = torch.where(o < 0, (-o) | 0x8000, o)
+    return torch.where(b2 >= 0x8000, b2 - 0x10000, b2).to(torch.int16).view(t.dtype)
 
 
 # ------------------------------------------------------------------ small batch W8A16 (a8)
@@ -649,7 +703,15 @@ def test_small_m_w8a16_within_tolerance(L, dev, M, N, K, dt):
     xa, code = O.from_torch(x)
     ref = O.to_f32(O.linear_w8a16(xa, code, wq.numpy(), ws.numpy(), O.from_torch(bias)[0], code), code)
     got = L.linear_w8a16_small_m(x.to(dev), wq.to(dev), ws.to(dev), bias.to(dev)).float().cpu().numpy()
-    assert (np.abs(got - ref) <= w8a16_bound(x, wq, ws, ref, dt)).all()
+    err = np.abs(got - ref)
+    assert (err <= w8a16_bound(x, wq, ws, ref, dt)).all()
+    # The worst case above grows with K; rounding errors of a binary32 accumulation add up like a random walk, so
+    # all but a few elements also meet the bound with sqrt(K) in place of K (a kernel that is off by a unit in the
+    # last place everywhere passes the first bound at K = 3072 and fails this one) ...
+    tight = spacing(ref, dt) + (w8a16_bound(x, wq, ws, ref, dt) - spacing(ref, dt)) / np.sqrt(K)
+    assert (err <= tight).mean() >= 0.995
+    if dt != torch.float32:   # ... and a 16-bit result differs from the reference's only where a sum sat next to a rounding boundary
+        assert (err != 0).mean() <= 0.10 + 2.0 / err.size
     got_t = L.linear_w8a16_small_m(x.to(dev), wq.to(dev), 0.004, None).float().cpu().numpy()
     ref_t = O.to_f32(O.linear_w8a16(xa, code, wq.numpy(), np.float32(0.004)), code)
     assert (np.abs(got_t - ref_t) <= w8a16_bound(x, wq, torch.full((N,), 0.004), ref_t, dt)).all()
