@@ -466,6 +466,26 @@ def target_only(L, dev, mode, steps, warmup):
             "frac_of_int8_peak": round(ops / t["median_us"] / 1e6 / PEAK_INT8_TOPS, 4)}
 
 
+def quant_only(L, dev, mode, steps, warmup):
+    """Nothing but launches of the per-row quantiser at the north-star shape (4608 x 3072 bf16), with (`rot`) or without
+    (`plain`) the 128-block rotation, over 8 buffer sets (> 256 MB), for profilers."""
+    M, K, sets = 4608, 3072, 8
+    g = torch.Generator().manual_seed(99)
+    xs = [_acts(g, M, K, 0.01, 20.0).to(dev) for _ in range(sets)]
+    qs = [torch.empty(M, K, dtype=torch.int8, device=dev) for _ in range(sets)]
+    ss = [torch.empty(M, 1, dtype=torch.float32, device=dev) for _ in range(sets)]
+    lib, ptr, stream = L.lib(), L._ptr, L._stream(xs[0])
+    qargs = [(ptr(xs[i]), L.BF16, M, K, K, 128 if mode == "rot" else 0, ptr(qs[i]), ptr(ss[i]), stream) for i in range(sets)]
+
+    def call(i):
+        rc = lib.i8f_quant_rowwise(*qargs[i])
+        assert rc == 0, rc
+    t = time_kernel(call, iters=max(1, steps // sets), warmup=warmup, sets=sets, burst=sets)
+    qbytes = M * K * 3 + 4 * M
+    return {"kernel": "quant16_kernel", "shape": "4608x3072 bf16", "rotation": mode == "rot", "median_us": round(t["median_us"], 2),
+            "min_us": round(t["min_us"], 2), "frac_of_hbm_peak": round(qbytes / t["median_us"] / 1e3 / PEAK_HBM_GBS, 4)}
+
+
 # --------------------------------------------------------------------------- CPU baseline
 def cpu_baseline(reps=3):
     """The reference's torch CPU path on config 1.  A 512-row probe sizes the sample: the whole
@@ -507,6 +527,8 @@ def main():
     ap.add_argument("--target-only", choices=("warm", "cold"),
                     help="profiling aid: launch nothing but the north-star GEMM (4608x3072x3072) on warm or cold operands, "
                          "print its timing and exit")
+    ap.add_argument("--quant-only", choices=("rot", "plain"),
+                    help="profiling aid: launch nothing but the per-row quantiser at 4608x3072 bf16, with or without rotation")
     ap.add_argument("--zero-operands", action="store_true",
                     help="diagnostic: all-zero activations and weights (same instructions, no switching in the multipliers), "
                          "to show what the power limit costs; the line says data = zeros and is not a benchmark result")
@@ -524,6 +546,9 @@ def main():
 
     if a.target_only:
         print(json.dumps(target_only(L, dev, a.target_only, a.steps, a.warmup)))
+        return
+    if a.quant_only:
+        print(json.dumps(quant_only(L, dev, a.quant_only, a.steps, a.warmup)))
         return
     step = MlpStep(L, dev)
     if a.zero_operands:

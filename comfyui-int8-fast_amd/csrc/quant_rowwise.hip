@@ -283,16 +283,13 @@ __device__ __forceinline__ void rotate_run16(float (&v)[16], float s0, float s1,
     dpp_fmac16<2>(v, s2);   // row_half_mirror
     const float h = hadamard_entry<DT>() * (s0 * s1 * s2);
 #pragma unroll
-    for (int j = 0; j < 16; j += 2) {
-        const float a = v[j] * h, b = v[j + 1] * h;
-        if constexpr (DT == I8F_BF16) {  // one packed conversion rounds two values
-            const uint32_t pk = f32x2_to_bf16x2_bits(a, b);
-            v[j] = __uint_as_float(pk << 16);
-            v[j + 1] = __uint_as_float(pk & 0xffff0000u);
-        } else {
-            v[j] = round_to_dtype<DT>(a);
-            v[j + 1] = round_to_dtype<DT>(b);
-        }
+    for (int j = 0; j < 16; ++j) {
+        const float a = v[j] * h;
+        // bfloat16: the packed conversion with a zero in the low half leaves the rounded value in the high half, which
+        // IS its binary32 form: one instruction rounds and widens (two values per conversion would need two more
+        // instructions to pull them apart again)
+        if constexpr (DT == I8F_BF16) v[j] = __uint_as_float(f32x2_to_bf16x2_bits(0.0f, a));
+        else v[j] = round_to_dtype<DT>(a);
     }
 }
 
@@ -302,14 +299,50 @@ __device__ __forceinline__ float max3_abs(float m, float a, float b) {
     return r;
 }
 
-__device__ __forceinline__ uint32_t quant4_magic(float a, float b, float c, float d, float inv) {
+// scale = max(amax / 127, 1e-30) and inv = 1 / scale, both correctly rounded, for an amax that is a value of a 16-bit
+// dtype, without the division sequence (22 instructions of a wave's fixed work become 8):
+//   amax / 127 = fma(r, y, q) with y = RN(1 / 127), q = RN(amax y), r = amax - 127 q (exact): Markstein's correction,
+//     which gives the correctly rounded quotient for every finite bfloat16 and binary16 amax whose quotient is not
+//     below the 1e-30 floor (every such value is checked on the host by the test suite);
+//   1 / scale = fma(e, y0, y0) with y0 the hardware reciprocal (1 ulp) and e = 1 - scale y0: correctly rounded unless
+//     the significand of scale is all ones (Markstein), which takes the division.
+__device__ __forceinline__ void scale_and_inverse16(float amax, float &scale, float &inv) {
+    const float y = 0x1.020408p-7f;  // RN(1 / 127)
+    const float q = amax * y;
+    const float r = __builtin_fmaf(-127.0f, q, amax);
+    float s = __builtin_fmaf(r, y, q);
+    s = s < 1e-30f ? 1e-30f : s;
+    const float y0 = __builtin_amdgcn_rcpf(s);
+    const float e = __builtin_fmaf(-s, y0, 1.0f);
+    float iv = __builtin_fmaf(e, y0, y0);
+    // (every lane holds the same scale: a scalar test and a branch that is practically never taken)
+    if (__builtin_expect((__builtin_amdgcn_readfirstlane(__float_as_uint(s)) & 0x7fffffu) == 0x7fffffu, 0)) iv = 1.0f / s;
+    scale = s;
+    inv = iv;
+}
+
+// Sixteen values of one run to sixteen int8 in four dwords.  p + 1.5 * 2^23 leaves the rounded integer in the low byte
+// of the sum; the additions after the first of each dword write that byte straight into its place (an SDWA destination
+// select with the other bytes preserved), so nothing is left to shuffle: 32 instructions per run instead of 44.  An
+// instruction that writes part of a register must not be followed at once by a reader of that register: the four dwords
+// are worked on in turn, which puts three instructions between any two that touch the same one.
+__device__ __forceinline__ uint4 quant16_magic(const float (&v)[16], float inv) {
+    float p[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) p[j] = v[j] * inv;
     const float M = 12582912.0f;
-    const uint32_t ua = __float_as_uint(a * inv + M), ub = __float_as_uint(b * inv + M);
-    const uint32_t uc = __float_as_uint(c * inv + M), ud = __float_as_uint(d * inv + M);
-    // low bytes of the four sums: {ua.b0, ub.b0} and {uc.b0, ud.b0}, then the two halves
-    const uint32_t lo = __builtin_amdgcn_perm(ub, ua, 0x0c0c0400u);
-    const uint32_t hi = __builtin_amdgcn_perm(ud, uc, 0x04000c0cu);
-    return lo | hi;
+    uint32_t o0, o1, o2, o3;
+#define I8F_SDWA_ADD(d, s, b) "v_add_f32_sdwa %" #d ", %" #s ", %20 dst_sel:BYTE_" #b " dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+    asm("v_add_f32 %0, %4, %20\n\tv_add_f32 %1, %8, %20\n\tv_add_f32 %2, %12, %20\n\tv_add_f32 %3, %16, %20\n\t"
+        I8F_SDWA_ADD(0, 5, 1) I8F_SDWA_ADD(1, 9, 1) I8F_SDWA_ADD(2, 13, 1) I8F_SDWA_ADD(3, 17, 1)
+        I8F_SDWA_ADD(0, 6, 2) I8F_SDWA_ADD(1, 10, 2) I8F_SDWA_ADD(2, 14, 2) I8F_SDWA_ADD(3, 18, 2)
+        I8F_SDWA_ADD(0, 7, 3) I8F_SDWA_ADD(1, 11, 3) I8F_SDWA_ADD(2, 15, 3) I8F_SDWA_ADD(3, 19, 3)
+        "s_nop 0"
+        : "=&v"(o0), "=&v"(o1), "=&v"(o2), "=&v"(o3)
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]), "v"(p[8]), "v"(p[9]),
+          "v"(p[10]), "v"(p[11]), "v"(p[12]), "v"(p[13]), "v"(p[14]), "v"(p[15]), "v"(M));
+#undef I8F_SDWA_ADD
+    return make_uint4(o0, o1, o2, o3);
 }
 
 // WPR waves share a row (1 or 4); each lane holds RUNS runs of 16 elements; one row per wave or group of
@@ -317,16 +350,22 @@ __device__ __forceinline__ uint32_t quant4_magic(float a, float b, float c, floa
 // fewer, longer-lived waves ramp up and drain more slowly).  FULL: every lane's runs exist and every row of
 // the grid exists (K = 16 RUNS 64 WPR, M a multiple of the rows of a workgroup), so nothing is tested or
 // zero-filled: 3 % at 4608 x 3072.
-template <int DT, bool ROT, int WPR, int RUNS, bool FULL, int PRO = I8F_PRO_NONE>
-__global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x, int64_t M, int64_t K,
-                                                       int64_t ldx_bytes, int8_t *__restrict__ q,
-                                                       float *__restrict__ scale, const Prologue pro) {
+// SEG > 1 (with WPR = 1): a row is cut into SEG contiguous segments of whole 128-blocks, one wave each, which share
+// only the row maximum: units of half a row, for rows that would otherwise leave some SIMDs with a whole row more
+// than others.
+template <int DT, bool ROT, int WPR, int RUNS, bool FULL, int PRO, int SEG>
+__device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t M, int64_t K, int64_t ldx_bytes,
+                                             int8_t *__restrict__ q, float *__restrict__ scale, const Prologue &pro,
+                                             int64_t first_row) {
+    static_assert(SEG == 1 || WPR == 1, "segments are for the one-wave-per-row form");
     constexpr int TPR = 64 * WPR;
-    constexpr int ROWS = 256 / TPR;  // the workgroup has ROWS * TPR threads: 256, or 192 with three waves to a row
+    constexpr int ROWS = 256 / (TPR * SEG);  // rows per workgroup
     const int t = threadIdx.x % TPR;
-    const int rb = threadIdx.x / TPR;
-    const int64_t m = (int64_t)blockIdx.x * ROWS + rb;
-    const int nruns = (int)(K / 16);
+    const int unit = threadIdx.x / TPR;
+    const int rb = unit / SEG, sg = unit % SEG;
+    const int64_t m = first_row + rb;
+    const int nruns = (int)(K / 16) / SEG;   // runs of this wave's segment (of the row if SEG == 1)
+    const int64_t seg_run = (int64_t)sg * nruns;  // first run of the segment
     // run held by this lane inside its group of 8: lanes 4..7 take runs 7..4
     const int p = t ^ (((t >> 2) & 1) * 3);
     const float s0 = (p & 1) ? -1.0f : 1.0f, s1 = (p & 2) ? -1.0f : 1.0f, s2 = (p & 4) ? -1.0f : 1.0f;
@@ -339,8 +378,8 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
         for (int r = 0; r < RUNS; ++r) {
             const int R = r * TPR + p;
             if (FULL || (ok && R < nruns)) {
-                raw[r][0] = *(const uint4 *)(xrow + (int64_t)R * 32);
-                raw[r][1] = *(const uint4 *)(xrow + (int64_t)R * 32 + 16);
+                raw[r][0] = *(const uint4 *)(xrow + (seg_run + R) * 32);
+                raw[r][1] = *(const uint4 *)(xrow + (seg_run + R) * 32 + 16);
             } else {
                 raw[r][0] = make_uint4(0, 0, 0, 0);
                 raw[r][1] = make_uint4(0, 0, 0, 0);
@@ -358,7 +397,7 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
             if constexpr (PRO == I8F_PRO_MODULATE) {
                 // the vectors of this row's group, same 16 columns (they come from cache: every row of the group reads them)
                 const int R = r * TPR + p;
-                const int64_t off = (vrow * K + (FULL || R < nruns ? R : 0) * 16) * 2;
+                const int64_t off = (vrow * K + (seg_run + (FULL || R < nruns ? R : 0)) * 16) * 2;
                 float sv[16], tv[16];
                 expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), sv);
                 expand16<DT>(*(const uint4 *)((const char *)pro.t + off), *(const uint4 *)((const char *)pro.t + off + 16), tv);
@@ -373,18 +412,17 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
             for (int j = 0; j < 16; j += 2) amax = max3_abs(amax, v[r][j], v[r][j + 1]);
         }
         amax = wave_max(amax);
-        if constexpr (WPR > 1) {
-            __shared__ float red[ROWS][WPR];
-            if ((t & 63) == 0) red[rb][t / 64] = amax;
+        if constexpr (WPR * SEG > 1) {
+            __shared__ float red[ROWS][WPR * SEG];
+            if ((t & 63) == 0) red[rb][sg * WPR + t / 64] = amax;
             __syncthreads();
             amax = red[rb][0];
 #pragma unroll
-            for (int w = 1; w < WPR; ++w) amax = fmaxf(amax, red[rb][w]);
+            for (int w = 1; w < WPR * SEG; ++w) amax = fmaxf(amax, red[rb][w]);
         }
 
-        float s = amax / 127.0f;
-        s = s < 1e-30f ? 1e-30f : s;
-        const float inv = 1.0f / s;
+        float s, inv;
+        scale_and_inverse16(amax, s, inv);
 
         if (FULL || m < M) {
             int8_t *qrow = q + m * K;
@@ -392,23 +430,53 @@ __global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x
             for (int r = 0; r < RUNS; ++r) {
                 const int R = r * TPR + p;
                 if (FULL || R < nruns) {
-                    uint4 o;
-                    o.x = quant4_magic(v[r][0], v[r][1], v[r][2], v[r][3], inv);
-                    o.y = quant4_magic(v[r][4], v[r][5], v[r][6], v[r][7], inv);
-                    o.z = quant4_magic(v[r][8], v[r][9], v[r][10], v[r][11], inv);
-                    o.w = quant4_magic(v[r][12], v[r][13], v[r][14], v[r][15], inv);
-                    stream_store16(qrow + (int64_t)R * 16, o);
+                    stream_store16(qrow + (seg_run + R) * 16, quant16_magic(v[r], inv));
                 }
             }
-            if (t == 0) scale[m] = s;
+            if (t == 0 && sg == 0) scale[m] = s;
         }
     }
+}
+
+template <int DT, bool ROT, int WPR, int RUNS, bool FULL, int PRO = I8F_PRO_NONE>
+__global__ __launch_bounds__(256) void quant16_kernel(const char *__restrict__ x, int64_t M, int64_t K,
+                                                       int64_t ldx_bytes, int8_t *__restrict__ q,
+                                                       float *__restrict__ scale, const Prologue pro) {
+    quant16_body<DT, ROT, WPR, RUNS, FULL, PRO, 1>(x, M, K, ldx_bytes, q, scale, pro, (int64_t)blockIdx.x * (256 / (64 * WPR)));
+}
+
+// The rotating quantiser is bound by the vector ALUs of the SIMDs that get the most rows.  1 024 SIMDs take a multiple
+// of 1 024 rows evenly, one wave per row; up to 512 rows beyond that would put a whole extra row on as many SIMDs
+// while the others idle, so those rows go as half rows (two waves to a row, two rows to a workgroup): every SIMD gets
+// at most half a row more.  One launch: the first main_blocks workgroups take four whole rows each, the others two
+// rows in halves.
+constexpr int TAIL_SEG = 2;  // (quarter rows measured the same as half rows: twice the waves, each with a wave's fixed work)
+template <int DT, bool ROT, int RUNS>
+__global__ __launch_bounds__(256) void quant16_tail_kernel(const char *__restrict__ x, int64_t M, int64_t K,
+                                                            int64_t ldx_bytes, int8_t *__restrict__ q,
+                                                            float *__restrict__ scale, int main_blocks) {
+    const Prologue none{};
+    if ((int)blockIdx.x < main_blocks)
+        quant16_body<DT, ROT, 1, RUNS, true, I8F_PRO_NONE, 1>(x, M, K, ldx_bytes, q, scale, none, (int64_t)blockIdx.x * 4);
+    else
+        quant16_body<DT, ROT, 1, (RUNS + TAIL_SEG - 1) / TAIL_SEG, false, I8F_PRO_NONE, TAIL_SEG>(
+            x, M, K, ldx_bytes, q, scale, none, (int64_t)main_blocks * 4 + ((int64_t)blockIdx.x - main_blocks) * (4 / TAIL_SEG));
 }
 
 template <int DT, bool ROT, int WPR, int RUNS, int PRO = I8F_PRO_NONE>
 int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st, const Prologue &pro = Prologue{}) {
     constexpr int ROWS = 256 / (64 * WPR);
     const int64_t blocks = (M + ROWS - 1) / ROWS;
+    if constexpr (ROT && PRO == I8F_PRO_NONE && WPR == 1) {
+        // whole rows for every SIMD, then the rest (at most half a row per SIMD) in half rows of whole 128-blocks
+        const int64_t rest = M % 1024;
+        if (K == (int64_t)RUNS * 64 * 16 && M % 4 == 0 && M >= 1024 && rest > 0 && rest <= 512 && (K / 16) % (8 * TAIL_SEG) == 0) {
+            const int main_blocks = (int)((M - rest) / 4);
+            hipLaunchKernelGGL((quant16_tail_kernel<DT, ROT, RUNS>), dim3((unsigned)(main_blocks + rest * TAIL_SEG / 4)), dim3(256), 0, st,
+                               (const char *)x, M, K, ldx * 2, q, scale, main_blocks);
+            return check_launch();
+        }
+    }
     if (PRO == I8F_PRO_NONE && K == (int64_t)RUNS * 64 * WPR * 16 && M % ROWS == 0)
         hipLaunchKernelGGL((quant16_kernel<DT, ROT, WPR, RUNS, PRO == I8F_PRO_NONE, PRO>), dim3((unsigned)blocks), dim3(ROWS * 64 * WPR), 0, st,
                            (const char *)x, M, K, ldx * 2, q, scale, pro);

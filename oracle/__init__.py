@@ -51,6 +51,8 @@ def lib() -> ctypes.CDLL:
         L.orc_linear_w8a16.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i64]
         L.orc_sr_delta.argtypes = [vp, vp, i32, vp, i64, i64, vp]
         L.orc_merge_i8.argtypes = [vp, vp, i64, vp]
+        L.orc_scale_by_127_mismatches.argtypes = [vp, i64, vp]
+        L.orc_scale_by_127_mismatches.restype = i64
         L.orc_quotient_by_reciprocal_mismatches.argtypes = [vp, vp, i64, vp]
         L.orc_quotient_by_reciprocal_mismatches.restype = i64
         L.orc_lora_delta.argtypes = [vp, vp, i64, i64, i64, f32, vp]
@@ -278,6 +280,14 @@ def sr_delta(x, scale, noise):
     dq = np.empty((N, K), dtype=np.int8)
     _chk(lib().orc_sr_delta(_p(x), _p(scale), mode, _p(noise), N, K, _p(dq)), "sr_delta")
     return dq
+
+
+def scale_by_127_mismatches(a):
+    """(count, first index or -1) of values whose fma-corrected product with 1/127 differs from max(a / 127, 1e-30)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    first = ctypes.c_int64(-1)
+    n = lib().orc_scale_by_127_mismatches(_p(a), a.size, ctypes.byref(first))
+    return int(n), int(first.value)
 
 
 def quotient_by_reciprocal_mismatches(a, b):

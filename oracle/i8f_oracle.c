@@ -494,6 +494,30 @@ int orc_sr_delta(const float *x, const float *scale, int scale_mode, const float
 }
 
 /*
+ * Check of an arithmetic identity that the HIP quantiser for 16-bit inputs relies on (no counterpart in the reference,
+ * which divides, int8_quant.py:21,29): with y = 1/127 correctly rounded, q = a*y followed by ONE correction
+ * fma(fma(-127, q, a), y, q), clamped below at 1e-30, equals max(a / 127, 1e-30).  Returns how many of the n values
+ * disagree (bit patterns compared) and stores the index of the first in *first_bad.
+ */
+int64_t orc_scale_by_127_mismatches(const float *a, int64_t n, int64_t *first_bad) {
+    int64_t bad = 0;
+    const float y = 1.0f / 127.0f;
+    for (int64_t i = 0; i < n; ++i) {
+        float q = a[i] * y;
+        const float r = fmaf(-127.0f, q, a[i]);
+        q = fmaf(r, y, q);
+        if (q < 1e-30f) q = 1e-30f;
+        float t = a[i] / 127.0f;
+        if (t < 1e-30f) t = 1e-30f;
+        if (memcmp(&q, &t, 4) != 0) {
+            if (bad == 0 && first_bad) *first_bad = i;
+            ++bad;
+        }
+    }
+    return bad;
+}
+
+/*
  * Check of an arithmetic identity that the HIP merge kernels rely on (no counterpart in the reference, which
  * divides): with y = 1/b correctly rounded, q = a*y followed by two corrections q = fma(fma(-b, q, a), y, q)
  * is the correctly rounded a/b as long as nothing over- or underflows.  Returns how many of the n pairs

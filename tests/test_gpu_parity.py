@@ -46,6 +46,8 @@ QUANT_CASES = [
     (8, 3072, torch.float32, True), (8, 3072, torch.float16, True), (5, 24576, torch.float32, True),
     (6, 40960, torch.float32, True), (2, 70000, torch.bfloat16, False), (3, 66048, torch.bfloat16, True),
     (4, 384, torch.bfloat16, True), (1, 128, torch.float32, True), (257, 512, torch.float16, False), (1, 8, torch.bfloat16, False),
+    # row counts just beyond a multiple of 1024: the rows beyond it are quantised as half rows by two waves each
+    (4608, 3072, torch.bfloat16, True), (1536, 1024, torch.float16, True), (1028, 2048, torch.bfloat16, True), (2052, 4096, torch.bfloat16, True),
 ]
 
 
@@ -59,6 +61,28 @@ def test_quant_rowwise_bit_exact(L, dev, M, K, dt, rot):
     q, s = L.quant_rowwise(x.to(dev), rotate=rot)
     assert np.array_equal(q.cpu().numpy(), qo)
     assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_quant_rowwise_every_possible_row_maximum(L, dev, dt):
+    """The 16-bit quantiser takes its scale and the reciprocal of the scale without the division sequence; the row
+    maximum is a value of the dtype, so every case there is gets a row of its own: each finite positive pattern as
+    the maximum of a row of 128 values (fractions of it, both signs, the maximum at a varying position), and scales
+    and int8 are the oracle's bit for bit."""
+    if dt == torch.bfloat16:
+        amax = (torch.arange(1, 0x7F80, dtype=torch.int32) << 16).view(torch.float32)
+    else:
+        amax = torch.arange(1, 0x7C00, dtype=torch.int16).view(torch.float16).float()
+    M, K = amax.numel(), 128
+    frac = torch.rand(M, K, generator=G) * 2 - 1
+    x = (frac * amax[:, None]).to(dt)
+    x[torch.arange(M), torch.arange(M) % K] = amax.to(dt) * torch.where(torch.arange(M) % 2 == 0, 1.0, -1.0).to(dt)
+    xa, code = O.from_torch(x)
+    qo, so = O.quant_rowwise(xa, code, 0)
+    q, s = L.quant_rowwise(x.to(dev))
+    bad = (s.cpu().numpy().view(np.uint32) != so.view(np.uint32)).reshape(-1)
+    assert not bad.any(), f"{bad.sum()} scales differ, first for a row maximum of {amax[int(bad.argmax())].item()!r}"
+    assert np.array_equal(q.cpu().numpy(), qo)
 
 
 PROLOGUE_CASES = [

@@ -364,6 +364,19 @@ def test_sr_delta_special_cases():
     assert abs(O.sr_delta(xs, scale, noise).astype(np.float64).mean() - 1.2) < 5e-3
 
 
+def test_row_scale_without_a_division_is_the_division_for_every_16_bit_maximum():
+    """The HIP quantiser for bfloat16 / binary16 rows takes amax / 127 as fma(fma(-127, q, amax), y, q), q = amax y,
+    y = RN(1/127).  amax is a value of the row's dtype, so every case there is can be checked: all finite
+    non-negative patterns of both dtypes (and, for good measure, 4 M random binary32 values)."""
+    bf = (np.arange(0, 0x7F80, dtype=np.uint32) << 16).view(np.float32)
+    h = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    assert O.scale_by_127_mismatches(bf) == (0, -1)
+    assert O.scale_by_127_mismatches(h) == (0, -1)
+    rng = np.random.default_rng(5)
+    r32 = rng.integers(0, 0x7F000000, 4_000_000, dtype=np.int64).astype(np.uint32).view(np.float32)
+    assert O.scale_by_127_mismatches(r32) == (0, -1)
+
+
 def test_quotient_by_reciprocal_is_the_correctly_rounded_division():
     """The HIP merge kernels compute delta / scale as q = delta * y, twice q += fma(-scale, q, delta) * y with
     y = 1 / scale, where 2^-20 <= scale <= 2^20 and 2^-102 <= |delta| <= 2^80 (everything else takes the division).
