@@ -282,7 +282,15 @@ int launch(const SmallMArgs &a, hipStream_t st) {
     const size_t es = dtype_size(DT);
     const bool vec = a.K % 16 == 0 && (uintptr_t)a.w % 16 == 0 && (uintptr_t)a.x % 16 == 0 && (a.ldx * es) % 16 == 0;
     if constexpr (DT != I8F_F32) {
-        if (vec && a.K < (1ll << 30)) return launch_lds<DT, 2, 8>(a, st);
+        if (vec && a.K < (1ll << 30)) {
+            // Workgroups of two 16-column blocks, unless that leaves CUs without one: then one block each, twice as
+            // many workgroups (3072 x 12288: 192 instead of 96, 18.4 -> 13.1 us with the weight from HBM).  Beyond one
+            // workgroup per CU the two-block form is the faster one at every size measured (it fetches the activations
+            // once for both blocks).
+            const int64_t blocks = (a.N + 15) / 16;
+            if ((blocks + 1) / 2 < 256) return launch_lds<DT, 1, 8>(a, st);
+            return launch_lds<DT, 2, 8>(a, st);
+        }
     }
     dim3 grid((unsigned)((a.N + 3) / 4));
     if (vec) hipLaunchKernelGGL((small_m_kernel<DT, true>), grid, dim3(256), 0, st, a);

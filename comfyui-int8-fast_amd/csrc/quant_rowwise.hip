@@ -467,7 +467,7 @@ template <int DT, bool ROT, int WPR, int RUNS, int PRO = I8F_PRO_NONE>
 int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st, const Prologue &pro = Prologue{}) {
     constexpr int ROWS = 256 / (64 * WPR);
     const int64_t blocks = (M + ROWS - 1) / ROWS;
-    if constexpr (ROT && PRO == I8F_PRO_NONE && WPR == 1) {
+    if constexpr (ROT && PRO == I8F_PRO_NONE && WPR == 1) {  // (the quantiser without rotation is not bound by the vector ALUs: the split costs it 2 %)
         // whole rows for every SIMD, then the rest (at most half a row per SIMD) in half rows of whole 128-blocks
         const int64_t rest = M % 1024;
         if (K == (int64_t)RUNS * 64 * 16 && M % 4 == 0 && M >= 1024 && rest > 0 && rest <= 512 && (K / 16) % (8 * TAIL_SEG) == 0) {
