@@ -24,6 +24,7 @@ import torch
 from . import _lib, compile_ops, dynamic_lora, int8_fused_kernel, int8_quant, nodes, quarot  # noqa: F401
 from .int8_fused_kernel import (  # noqa: F401
     hip_int8_linear,
+    hip_int8_linear_pair,
     hip_int8_linear_per_row,
     hip_quantize_rowwise,
     triton_int8_linear,
@@ -35,6 +36,7 @@ from .int8_quant import (  # noqa: F401
     INT8MergedLoRAPatchAdapter,
     Int8TensorwiseOps,
     dequantize,
+    forward_pair,
     int8_forward_dynamic,
     int8_forward_dynamic_per_row,
     quantize_int8,

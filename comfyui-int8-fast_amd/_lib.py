@@ -53,6 +53,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_last_hip_error.restype = i32
     L.i8f_quant_rowwise.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, vp]
     L.i8f_rotate128.argtypes = [vp, i32, i64, i64, i64, vp, vp]
+    L.i8f_quant_rowwise_grouped.argtypes = [vp, i32, i32, i64, i32, vp]
     L.i8f_quant_rowwise_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, i32, vp, vp, vp]
     L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
     L.i8f_quant_tensorwise_workspace_bytes.restype = i64
@@ -70,7 +71,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_lora",
+    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -78,7 +79,7 @@ def lib() -> ctypes.CDLL:
 
 
 EXPORTS = (
-    "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_rotate128",
+    "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue",
     "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
@@ -201,6 +202,36 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
                                                     _ptr(mod_shift), rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s),
                                                     _stream(x)), "i8f_quant_rowwise_prologue")
     return q, s
+
+
+class _QuantGroup(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_void_p), ("M", ctypes.c_int64), ("ldx", ctypes.c_int64), ("q", ctypes.c_void_p),
+                ("scale", ctypes.c_void_p)]
+
+
+def quant_rowwise_grouped(xs, rotate: bool = False):
+    """quant_rowwise for several [M_i, K] tensors of one dtype, one width and one device in a single launch
+    -> [(int8 [M_i,K], float32 [M_i,1]), ...], bit-identical to the separate calls."""
+    xs = list(xs)
+    if not xs:
+        return []
+    for i, x in enumerate(xs):
+        _dev(x, f"xs[{i}]")
+        xs[i] = _rows(x, f"xs[{i}]")
+    K, dt, device = xs[0].shape[1], xs[0].dtype, xs[0].device
+    if any(x.shape[1] != K or x.dtype != dt or x.device != device for x in xs):
+        raise ValueError("the tensors of a group launch share their width, dtype and device")
+    if rotate and K % 128:
+        raise ValueError(f"rotation needs K % 128 == 0, got K={K}")
+    outs = [(torch.empty((x.shape[0], K), dtype=torch.int8, device=device), torch.empty((x.shape[0], 1), dtype=torch.float32, device=device))
+            for x in xs]
+    groups = (_QuantGroup * len(xs))()
+    for g, x, (q, s) in zip(groups, xs, outs):
+        g.x, g.M, g.ldx, g.q, g.scale = x.data_ptr(), x.shape[0], (x.stride(0) if x.shape[0] > 1 else K), q.data_ptr(), s.data_ptr()
+    with _on(device):
+        _check(lib().i8f_quant_rowwise_grouped(ctypes.byref(groups), len(xs), dtype_code(dt), K, 128 if rotate else 0, _stream(xs[0])),
+               "i8f_quant_rowwise_grouped")
+    return outs
 
 
 def quant_tensorwise(x: torch.Tensor, static_scratch: bool = False):

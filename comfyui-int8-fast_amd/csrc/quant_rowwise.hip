@@ -463,6 +463,47 @@ __global__ __launch_bounds__(256) void quant16_tail_kernel(const char *__restric
             x, M, K, ldx_bytes, q, scale, none, (int64_t)main_blocks * 4 + ((int64_t)blockIdx.x - main_blocks) * (4 / TAIL_SEG));
 }
 
+// Several row blocks of one width in one launch (the image and the text tokens of a transformer block, each with
+// its own tensors): workgroup b belongs to the group whose range of workgroups holds b.  Launches of a few
+// microseconds cost as much in the gap between kernels as in the kernel, so two 5 us launches become one of 7.
+constexpr int MAX_GROUPS = 8;
+struct GroupedArgs {
+    const char *x[MAX_GROUPS];
+    int8_t *q[MAX_GROUPS];
+    float *scale[MAX_GROUPS];
+    int64_t M[MAX_GROUPS], ldx_bytes[MAX_GROUPS];
+    int first_block[MAX_GROUPS + 1];   // first workgroup of each group; [n] = all workgroups
+    int n;
+};
+
+template <int DT, bool ROT, int WPR, int RUNS>
+__global__ __launch_bounds__(256) void quant16_grouped_kernel(const GroupedArgs g, int64_t K) {
+    int grp = 0;
+#pragma unroll
+    for (int i = 1; i < MAX_GROUPS; ++i)
+        if (i < g.n && (int)blockIdx.x >= g.first_block[i]) grp = i;
+    grp = __builtin_amdgcn_readfirstlane(grp);
+    const Prologue none{};
+    quant16_body<DT, ROT, WPR, RUNS, false, I8F_PRO_NONE, 1>(g.x[grp], g.M[grp], K, g.ldx_bytes[grp], g.q[grp], g.scale[grp], none,
+                                                            (int64_t)((int)blockIdx.x - g.first_block[grp]) * (256 / (64 * WPR)));
+}
+
+template <int DT, bool ROT, int WPR, int RUNS>
+int launch16_grouped(const GroupedArgs &g, int64_t K, hipStream_t st) {
+    hipLaunchKernelGGL((quant16_grouped_kernel<DT, ROT, WPR, RUNS>), dim3((unsigned)g.first_block[g.n]), dim3(256), 0, st, g, K);
+    return check_launch();
+}
+
+template <int DT, bool ROT, int WPR>
+int pick_runs16_grouped(int runs, const GroupedArgs &g, int64_t K, hipStream_t st) {
+    switch (runs) {
+    case 1: return launch16_grouped<DT, ROT, WPR, 1>(g, K, st);
+    case 2: return launch16_grouped<DT, ROT, WPR, 2>(g, K, st);
+    case 3: return launch16_grouped<DT, ROT, WPR, 3>(g, K, st);
+    default: return launch16_grouped<DT, ROT, WPR, 4>(g, K, st);
+    }
+}
+
 template <int DT, bool ROT, int WPR, int RUNS, int PRO = I8F_PRO_NONE>
 int launch16(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float *scale, hipStream_t st, const Prologue &pro = Prologue{}) {
     constexpr int ROWS = 256 / (64 * WPR);
@@ -721,6 +762,52 @@ extern "C" int i8f_quant_rowwise(const void *x, int x_dtype, int64_t M, int64_t 
     case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st);
     default: return dispatch_rot<I8F_F32>(rot, x, M, K, ldx, q, scale, st);
     }
+}
+
+extern "C" int i8f_quant_rowwise_grouped(const i8f_quant_group *groups, int n_groups, int x_dtype, int64_t K,
+                                         int rotate_block, void *stream) {
+    using namespace i8f;
+    if (n_groups < 0 || (n_groups > 0 && !groups) || K < 0 || !valid_dtype(x_dtype)) return I8F_ERR_INVALID;
+    if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
+    if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
+    bool one_launch = x_dtype != I8F_F32 && n_groups >= 2 && n_groups <= MAX_GROUPS && K % 16 == 0 && K >= 16 && K <= 16 * 64 * 4 * 4;
+    int64_t blocks = 0;
+    const int wpr = K / 16 <= 64 * 4 ? 1 : 4;
+    for (int i = 0; i < n_groups; ++i) {
+        const i8f_quant_group &g = groups[i];
+        if (g.M < 0 || (g.M > 0 && (!g.scale || g.ldx < K || (K > 0 && (!g.x || !g.q))))) return I8F_ERR_INVALID;
+        if (g.M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
+        one_launch = one_launch && (uintptr_t)g.x % 16 == 0 && (g.ldx * 2) % 16 == 0 && (uintptr_t)g.q % 16 == 0;
+        blocks += (g.M + 4 / wpr - 1) / (4 / wpr);
+    }
+    if (!one_launch || blocks > 0x7fffffff) {  // shapes without a grouped kernel: one launch per group, same results
+        for (int i = 0; i < n_groups; ++i)
+            if (int rc = i8f_quant_rowwise(groups[i].x, x_dtype, groups[i].M, K, groups[i].ldx, rotate_block, groups[i].q,
+                                           groups[i].scale, stream))
+                return rc;
+        return I8F_OK;
+    }
+    if (blocks == 0) return I8F_OK;
+    if (int rc = check_device()) return rc;
+    GroupedArgs ga{};
+    ga.n = n_groups;
+    int at = 0;
+    for (int i = 0; i < n_groups; ++i) {
+        ga.x[i] = (const char *)groups[i].x, ga.q[i] = groups[i].q, ga.scale[i] = groups[i].scale;
+        ga.M[i] = groups[i].M, ga.ldx_bytes[i] = groups[i].ldx * 2;
+        ga.first_block[i] = at;
+        at += (int)((groups[i].M + 4 / wpr - 1) / (4 / wpr));
+    }
+    ga.first_block[n_groups] = at;
+    hipStream_t st = (hipStream_t)stream;
+    const bool rot = rotate_block != 0;
+    const int64_t nruns = K / 16;
+    const int runs = wpr == 1 ? (int)((nruns + 63) / 64) : (int)((nruns + 255) / 256);
+#define I8F_GROUPED(DT)                                                                                              \
+    (wpr == 1 ? (rot ? pick_runs16_grouped<DT, true, 1>(runs, ga, K, st) : pick_runs16_grouped<DT, false, 1>(runs, ga, K, st)) \
+              : (rot ? pick_runs16_grouped<DT, true, 4>(runs, ga, K, st) : pick_runs16_grouped<DT, false, 4>(runs, ga, K, st)))
+    return x_dtype == I8F_BF16 ? I8F_GROUPED(I8F_BF16) : I8F_GROUPED(I8F_F16);
+#undef I8F_GROUPED
 }
 
 extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, int prologue,

@@ -94,6 +94,37 @@ def int8_forward_dynamic_per_row(x: Tensor, weight: Tensor, weight_scale: Tensor
                                    prologue=prologue, side=side)
 
 
+def forward_pair(layers, xs):
+    """Linear.forward for several quantised layers of one shape at once, e.g. the same projection of the image and of
+    the text stream of a double-stream block: [layer(x) for layer, x in zip(layers, xs)], with the activations of all
+    streams quantised by ONE kernel launch where the layers allow it (W8A8 path on every stream: more than 16 rows,
+    quantised weights on the inputs' device, no dynamic LoRA, no managed casting, the same rotation flag, inputs of one
+    width and one 16-bit dtype, eager mode).  Anything else falls back to the layers' own forward; results are
+    bit-identical either way."""
+    layers, xs = list(layers), list(xs)
+    ok = len(layers) >= 2 and len(layers) == len(xs) and not torch.compiler.is_compiling()
+    if ok:
+        x0 = xs[0]
+        rot = bool(getattr(layers[0], "_use_quarot", False))
+        for lin, x in zip(layers, xs):
+            managed = lin.comfy_cast_weights or len(lin.weight_function) > 0 or len(lin.bias_function) > 0
+            ok = ok and (getattr(lin, "_is_quantized", False) and not managed and lin.lora_A is None and x.is_cuda
+                         and lin.weight.device == x.device and (lin.bias is None or lin.bias.device == x.device)
+                         and x.dtype == x0.dtype and x.dtype in (torch.float16, torch.bfloat16) and x.shape[-1] == x0.shape[-1]
+                         and x.device == x0.device and x.numel() // max(1, x.shape[-1]) > SMALL_BATCH_ROWS
+                         and bool(getattr(lin, "_use_quarot", False)) == rot)
+    if not ok:
+        return [lin(x) for lin, x in zip(layers, xs)]
+    scales = []
+    for lin in layers:
+        ws = lin._get_weight_scale()
+        if isinstance(ws, Tensor) and ws.device != xs[0].device:
+            ws = ws.to(xs[0].device, non_blocking=True)
+        scales.append(ws)
+    return int8_fused_kernel.hip_int8_linear_pair(xs, [lin.weight for lin in layers], scales, [lin.bias for lin in layers],
+                                                  xs[0].dtype, rotate=rot)
+
+
 # --------------------------------------------------------------------------- LoRA delta reconstruction
 def reconstruct_lora_diff(weights, target_shape, device, dtype, strength):
     """Float delta of a LoRA / LoHA / LoKr patch and its scalar multiplier (int8_quant.py:128-208).

@@ -107,6 +107,25 @@ int i8f_quant_rowwise(const void *x, int x_dtype, int64_t M, int64_t K, int64_t 
                       int rotate_block, int8_t *q, float *scale, void *stream);
 
 /*
+ * i8f_quant_rowwise for several row blocks of one width K and one dtype in ONE launch: group i is an
+ * independent i8f_quant_rowwise(x, x_dtype, M, K, ldx, rotate_block, q, scale).  No counterpart in the reference,
+ * whose operator quantises one layer's input at a time (int8_fused_kernel.py:55-73); it is for callers that hold
+ * the inputs of two layers at once -- the image and the text tokens of a double-stream transformer block, which
+ * have their own weights and therefore their own linear layers -- where kernels of a few microseconds cost as
+ * much in the gaps between launches as in themselves.  Results are those of the separate calls bit for bit.
+ * The array of groups is read on the host during the call.  Up to 8 groups of 16-bit activations with 16-byte
+ * aligned rows and K % 16 == 0 (K <= 16384) take one launch; anything else is launched group by group.
+ */
+typedef struct i8f_quant_group {
+    const void *x;   /* [M,K] of x_dtype, row stride ldx elements */
+    int64_t M, ldx;
+    int8_t *q;       /* [M,K] int8, contiguous */
+    float *scale;    /* [M] */
+} i8f_quant_group;
+int i8f_quant_rowwise_grouped(const i8f_quant_group *groups, int n_groups, int x_dtype, int64_t K,
+                              int rotate_block, void *stream);
+
+/*
  * i8f_quant_rowwise with the elementwise operation in front of the linear layer
  * applied on the fly.  The reference gets this fusion from torch.compile, which
  * fuses the producer of the activations into its traceable Triton quantiser

@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 19
+    assert len(names) == 20
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -51,6 +51,16 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_quant_rowwise(one, L.BF16, 4, 256, 128, 0, one, one, null) == INVALID     # ldx < K
     assert lib.i8f_quant_rowwise(null, L.BF16, 4, 256, 256, 0, one, one, null) == INVALID    # NULL input
     assert lib.i8f_quant_rowwise(null, L.BF16, 0, 256, 256, 0, null, null, null) == 0        # empty: nothing to do
+    groups = (L._QuantGroup * 2)()
+    groups[0].x, groups[0].M, groups[0].ldx, groups[0].q, groups[0].scale = 16, 4, 256, 16, 16
+    groups[1].x, groups[1].M, groups[1].ldx, groups[1].q, groups[1].scale = 16, 4, 128, 16, 16    # ldx < K
+    assert lib.i8f_quant_rowwise_grouped(ctypes.byref(groups), 2, L.BF16, 256, 0, null) == INVALID
+    groups[1].ldx, groups[1].q = 256, None                                                          # NULL output
+    assert lib.i8f_quant_rowwise_grouped(ctypes.byref(groups), 2, L.BF16, 256, 0, null) == INVALID
+    assert lib.i8f_quant_rowwise_grouped(ctypes.byref(groups), 2, L.BF16, 200, 128, null) == INVALID
+    assert lib.i8f_quant_rowwise_grouped(ctypes.byref(groups), 2, 9, 256, 0, null) == INVALID
+    assert lib.i8f_quant_rowwise_grouped(null, 1, L.BF16, 256, 0, null) == INVALID
+    assert lib.i8f_quant_rowwise_grouped(null, 0, L.BF16, 256, 0, null) == 0
     assert lib.i8f_rotate128(one, L.F32, 4, 100, 100, one, null) == INVALID
     # K-split workspace: too small, misaligned; the size is what the header says (16 MB + 4 KB)
     nbytes = lib.i8f_linear_w8a8_workspace_bytes()

@@ -285,3 +285,27 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
     assert torch.equal(lin(x, prologue=L.PRO_MODULATE, mod_scale=sc32, mod_shift=sh32), lin((1 + sc32) * x + sh32))
     small = x[:1, :4]                     # four rows: the W8A16 path applies the operation in torch
     assert torch.equal(lin(small, prologue=L.PRO_GELU_TANH), lin(F.gelu(small, approximate="tanh")))
+
+
+@pytest.mark.parametrize("quarot", [False, True])
+def test_forward_pair_equals_the_layers_own_forward(pkg, dev, quarot):
+    """forward_pair: the same projection of two token streams with their own weights, activations quantised in one
+    launch, bit-identical to calling each layer; layers that cannot share the launch (a small batch) fall back."""
+    g = torch.Generator().manual_seed(31)
+
+    def layer(n, k):
+        lin = pkg.Int8TensorwiseOps.Linear(k, n, bias=True)
+        lin._load_from_state_dict({"l.weight": torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g),
+                                   "l.weight_scale": torch.rand(n, 1, generator=g) * 0.002 + 1e-3,
+                                   "l.bias": torch.randn(n, generator=g).bfloat16()}, "l.", {}, True, [], [], [])
+        lin._use_quarot = quarot
+        return lin.to(dev)
+    img, txt = layer(192, 384), layer(192, 384)
+    x_img = torch.randn(2, 100, 384, generator=g).bfloat16().to(dev)
+    x_txt = torch.randn(2, 20, 384, generator=g).bfloat16().to(dev)
+    y_img, y_txt = pkg.forward_pair([img, txt], [x_img, x_txt])
+    assert y_img.shape == (2, 100, 192) and y_txt.shape == (2, 20, 192)
+    assert torch.equal(y_img, img(x_img)) and torch.equal(y_txt, txt(x_txt))
+    small = x_txt[:1, :3]                                  # three rows: that stream takes the W8A16 path, so no shared launch
+    y_img2, y_small = pkg.forward_pair([img, txt], [x_img, small])
+    assert torch.equal(y_img2, y_img) and torch.equal(y_small, txt(small))

@@ -85,6 +85,33 @@ def test_quant_rowwise_every_possible_row_maximum(L, dev, dt):
     assert np.array_equal(q.cpu().numpy(), qo)
 
 
+@pytest.mark.parametrize("rot,dt,K", [(False, torch.bfloat16, 3072), (True, torch.bfloat16, 3072), (True, torch.float16, 1024),
+                                       (False, torch.bfloat16, 12288), (False, torch.float16, 200), (False, torch.float32, 256)])
+def test_quant_rowwise_grouped_equals_separate_calls_and_the_oracle(L, dev, rot, dt, K):
+    """Several row blocks in one launch (i8f_quant_rowwise_grouped): every group's int8 and scales are the oracle's and
+    those of a launch of its own, for row counts that do and do not fill a workgroup, an empty group, a strided group,
+    and the shapes (binary32, odd widths) that the entry point launches group by group."""
+    Ms = [130, 0, 33, 4, 257]
+    xs = [acts(M, K, dt) for M in Ms]
+    wide = acts(19, K + 16, dt)
+    dev_xs = [x.to(dev) for x in xs] + [wide.to(dev)[:, :K]]
+    xs.append(wide[:, :K].contiguous())
+    got = L.quant_rowwise_grouped(dev_xs, rotate=rot)
+    assert len(got) == len(xs)
+    for x, xd, (q, s) in zip(xs, dev_xs, got):
+        if x.shape[0] == 0:
+            assert q.shape == (0, K) and s.shape == (0, 1)
+            continue
+        xa, code = O.from_torch(x)
+        qo, so = O.quant_rowwise(xa, code, 128 if rot else 0)
+        assert np.array_equal(q.cpu().numpy(), qo)
+        assert np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+        q1, s1 = L.quant_rowwise(xd, rotate=rot)
+        assert torch.equal(q1, q) and torch.equal(s1, s)
+    with pytest.raises(ValueError):
+        L.quant_rowwise_grouped([dev_xs[0], dev_xs[0][:, : K // 2]])
+
+
 PROLOGUE_CASES = [
     # M, K, dtype, rotate, vectors
     (64, 3072, torch.bfloat16, False, 1), (48, 3072, torch.bfloat16, True, 2), (12, 12288, torch.bfloat16, False, 3),
