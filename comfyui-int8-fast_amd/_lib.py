@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libi8f_gfx950.so")
 BF16, F16, F32 = 0, 1, 2
 SCALE_TENSOR, SCALE_ROW = 0, 1
 EPI_TORCH, EPI_FUSED = 0, 1
-PRO_NONE, PRO_MODULATE, PRO_GELU_TANH = 0, 1, 2
+PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE = 0, 1, 2, 3
 
 _DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
 
@@ -167,7 +167,8 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
     """x [M,K] (bf16/fp16/fp32, cuda) -> (int8 [M,K], float32 [M,1]); rotate=True applies the 128-block Hadamard first.
     prologue applies an elementwise operation while the rows are read: PRO_GELU_TANH, or PRO_MODULATE with
     mod_scale / mod_shift of x's dtype, [V,K] (or [K]): (1 + mod_scale) * x + mod_shift, M // V consecutive rows
-    to a vector."""
+    to a vector, or PRO_SILU_GATE with the gate operand as mod_scale (x's dtype, [M,K], or [V,K] like the vectors
+    above): silu(x) * mod_scale."""
     _dev(x, "x")
     x = _rows(x, "x")
     M, K = x.shape
@@ -177,8 +178,10 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
     s = torch.empty((M, 1), dtype=torch.float32, device=x.device)
     ldx = x.stride(0) if M > 1 else K
     rows_per_vec = 1
-    if prologue == PRO_MODULATE:
+    if prologue in (PRO_MODULATE, PRO_SILU_GATE):
         vecs = []
+        if prologue == PRO_SILU_GATE:
+            mod_shift = mod_scale      # one operand: the gate
         for name, v in (("mod_scale", mod_scale), ("mod_shift", mod_shift)):
             _dev(v, name)
             if v.dtype != x.dtype or v.device != x.device or v.numel() % max(K, 1) or v.shape[-1] != K:

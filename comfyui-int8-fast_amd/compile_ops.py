@@ -19,8 +19,8 @@ the namespace `i8f` with a shape-only ("fake") implementation:
 dispatcher overhead per layer.  A weight scale is passed either as a tensor or, for the
 single-scale layout, as a float beside a `None` tensor.
 
-`fuse_prologues(graph_module)` rewrites a traced graph so that `gelu(x, approximate="tanh")` and
-`(1 + scale) * x + shift` feeding an `int8_linear` become its prologue, and `backend(inner)` is a
+`fuse_prologues(graph_module)` rewrites a traced graph so that `gelu(x, approximate="tanh")`,
+`(1 + scale) * x + shift` and `silu(a) * b` feeding an `int8_linear` become its prologue, and `backend(inner)` is a
 torch.compile backend that applies the rewrite and hands the graph to `inner` ("inductor" by default):
 
     model = torch.compile(model, backend=compile_ops.backend())
@@ -110,8 +110,9 @@ def _(x, weight, weight_scale, weight_scale_value, bias, rotate):
 def int8_linear_prologue(x: Tensor, prologue: int, mod_scale: Optional[Tensor], mod_shift: Optional[Tensor],
                          weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
                          bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int) -> Tensor:
-    """int8_linear on prologue(x): tanh-GELU, or (1 + mod_scale) * x + mod_shift with one pair of vectors per
-    group of consecutive rows; the transformed activations exist only inside the quantiser."""
+    """int8_linear on prologue(x): tanh-GELU, (1 + mod_scale) * x + mod_shift with one pair of vectors per
+    group of consecutive rows, or silu(x) * mod_scale with a gate operand of x's shape; the transformed activations
+    exist only inside the quantiser."""
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
                               mod_shift=mod_shift)
@@ -162,6 +163,21 @@ def _match_gelu(node):
     return node.args[0] if approx == "tanh" else None
 
 
+def _match_silu_gate(node):
+    """silu(a) * b in either operand order (a, b of one shape and dtype by the traced metadata) -> (a, b) nodes."""
+    if not (_is_call(node, operator.mul, torch.mul) and len(node.users) == 1 and len(node.args) == 2):
+        return None
+    for act, gate in (node.args, node.args[::-1]):
+        if not (isinstance(act, torch.fx.Node) and isinstance(gate, torch.fx.Node) and len(act.users) == 1
+                and _is_call(act, torch.nn.functional.silu)):
+            continue
+        a = act.args[0]
+        va, vb = (n.meta.get("example_value", n.meta.get("val")) if isinstance(n, torch.fx.Node) else None for n in (a, gate))
+        if va is not None and vb is not None and tuple(va.shape) == tuple(vb.shape) and va.dtype == vb.dtype:
+            return a, gate
+    return None
+
+
 def _match_modulate(node):
     """(1 + scale) * x + shift in any operand order -> (x, scale, shift) nodes."""
     if not (_is_call(node, operator.add, torch.add) and len(node.users) == 1 and len(node.args) == 2):
@@ -203,8 +219,8 @@ def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
 
 
 def fuse_prologues(gm: torch.fx.GraphModule) -> int:
-    """Rewrite int8_linear(gelu_tanh(h)) and int8_linear((1 + s) * h + t) (no dynamic-LoRA addend, producer used
-    nowhere else) into int8_linear_prologue(h, ...).  Returns the number of layers rewritten."""
+    """Rewrite int8_linear(gelu_tanh(h)), int8_linear((1 + s) * h + t) and int8_linear(silu(h) * g) (no dynamic-LoRA
+    addend, producer used nowhere else) into int8_linear_prologue(h, ...).  Returns the number of layers rewritten."""
     n_fused = 0
     targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
     for node in list(gm.graph.nodes):
@@ -226,8 +242,11 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
             new_args = (h, _lib.PRO_GELU_TANH, None, None)
         else:
             m = _match_modulate(src)
+            g = _match_silu_gate(src) if m is None else None
             if m is not None and _vectors_broadcast_over_tokens(*m):
                 new_args = (m[0], _lib.PRO_MODULATE, m[1], m[2])
+            elif g is not None:
+                new_args = (g[0], _lib.PRO_SILU_GATE, g[1], None)
         if new_args is None:
             continue
         # The fused operator returns the leading shape of h, the original one that of x_in: the same when nothing

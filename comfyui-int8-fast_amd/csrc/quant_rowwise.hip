@@ -39,6 +39,9 @@ struct Elem {
 //                                                     rows_per_vec rows, in x's dtype.  Evaluated as
 //                                                     torch evaluates the three tensor operations in
 //                                                     x's dtype: each result rounded to that dtype.
+//   I8F_PRO_SILU_GATE  v = silu(x) * g[k]             gated activation of a SwiGLU feed-forward; g like s above (one
+//                                                     row of g per row of x when rows_per_vec = 1); silu in binary32
+//                                                     rounded to x's dtype, then the product rounded to x's dtype.
 //   I8F_PRO_GELU_TANH  v = gelu(x), tanh form         0.5 x (1 + tanh(b (x + 0.044715 x^3))), b = sqrt(2/pi),
 //                                                     evaluated in binary32 and rounded once to x's dtype,
 //                                                     tanh(u) = 1 - 2 / (exp(2u) + 1) on the hardware's
@@ -58,9 +61,16 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a));
 }
 
+// x / (1 + exp(-x)) on the hardware's exp2 and reciprocal (a few binary32 ulp); exp2 overflowing to +inf gives x * 0
+__device__ __forceinline__ float silu_f32(float x) {
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
+
 template <int DT, int PRO>
 __device__ __forceinline__ float apply_prologue(float x, float s, float t) {
-    if constexpr (PRO == I8F_PRO_MODULATE) {
+    if constexpr (PRO == I8F_PRO_SILU_GATE) {
+        return round_to_dtype<DT>(round_to_dtype<DT>(silu_f32(x)) * s);
+    } else if constexpr (PRO == I8F_PRO_MODULATE) {
         const float a = round_to_dtype<DT>(1.0f + s);
         const float b = round_to_dtype<DT>(a * x);
         return round_to_dtype<DT>(b + t);
@@ -390,7 +400,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
         float v[RUNS][16];
         float amax = 0.0f;
         [[maybe_unused]] int64_t vrow = 0;  // the row's pair of modulation vectors (M < 2^31: a 32-bit division)
-        if constexpr (PRO == I8F_PRO_MODULATE) vrow = (uint32_t)(FULL || m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
+        if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_SILU_GATE) vrow = (uint32_t)(FULL || m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
             expand16<DT>(raw[r][0], raw[r][1], v[r]);
@@ -403,6 +413,13 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
                 expand16<DT>(*(const uint4 *)((const char *)pro.t + off), *(const uint4 *)((const char *)pro.t + off + 16), tv);
 #pragma unroll
                 for (int j = 0; j < 16; ++j) v[r][j] = FULL || R < nruns ? apply_prologue<DT, PRO>(v[r][j], sv[j], tv[j]) : 0.0f;
+            } else if constexpr (PRO == I8F_PRO_SILU_GATE) {
+                const int R = r * TPR + p;
+                const int64_t off = (vrow * K + (seg_run + (FULL || R < nruns ? R : 0)) * 16) * 2;
+                float gv[16];
+                expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), gv);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v[r][j] = FULL || R < nruns ? apply_prologue<DT, PRO>(v[r][j], gv[j], 0.0f) : 0.0f;
             } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) v[r][j] = apply_prologue<DT, PRO>(v[r][j], 0.0f, 0.0f);
@@ -570,10 +587,11 @@ __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__r
     const int64_t base = m * ldx;
     __shared__ float red[4];
     // element k of this row after the prologue
-    const int64_t vbase = PRO == I8F_PRO_MODULATE ? (m / pro.rows_per_vec) * K : 0;
+    const int64_t vbase = (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_SILU_GATE) ? (m / pro.rows_per_vec) * K : 0;
     auto element = [&](int64_t k) {
         const float xv = load_as_f32<DT>(x, base + k);
-        if constexpr (PRO == I8F_PRO_MODULATE) return apply_prologue<DT, PRO>(xv, load_as_f32<DT>(pro.s, vbase + k), load_as_f32<DT>(pro.t, vbase + k));
+        if constexpr (PRO == I8F_PRO_SILU_GATE) return apply_prologue<DT, PRO>(xv, load_as_f32<DT>(pro.s, vbase + k), 0.0f);
+        else if constexpr (PRO == I8F_PRO_MODULATE) return apply_prologue<DT, PRO>(xv, load_as_f32<DT>(pro.s, vbase + k), load_as_f32<DT>(pro.t, vbase + k));
         else return apply_prologue<DT, PRO>(xv, 0.0f, 0.0f);
     };
 
@@ -707,6 +725,7 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
     const size_t es = dtype_size(DT);
     bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) && ((uintptr_t)q % 8 == 0);
     if constexpr (PRO == I8F_PRO_MODULATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0 && (uintptr_t)pro.t % 16 == 0;
+    if constexpr (PRO == I8F_PRO_SILU_GATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0;
     const int64_t nchunks = K / EPC;
     if constexpr (DT != I8F_F32) {
         const int64_t nruns = K / 16;
@@ -737,6 +756,9 @@ int dispatch_rot(bool rot, const void *x, int64_t M, int64_t K, int64_t ldx, int
     case I8F_PRO_GELU_TANH:
         return rot ? dispatch<DT, true, I8F_PRO_GELU_TANH>(x, M, K, ldx, q, scale, st, pro)
                    : dispatch<DT, false, I8F_PRO_GELU_TANH>(x, M, K, ldx, q, scale, st, pro);
+    case I8F_PRO_SILU_GATE:
+        return rot ? dispatch<DT, true, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro)
+                   : dispatch<DT, false, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro);
     default: return rot ? dispatch<DT, true>(x, M, K, ldx, q, scale, st) : dispatch<DT, false>(x, M, K, ldx, q, scale, st);
     }
 }
@@ -815,7 +837,7 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
                                           int rotate_block, int8_t *q, float *scale, void *stream) {
     using namespace i8f;
     if (prologue == I8F_PRO_NONE) return i8f_quant_rowwise(x, x_dtype, M, K, ldx, rotate_block, q, scale, stream);
-    if (prologue != I8F_PRO_MODULATE && prologue != I8F_PRO_GELU_TANH) return I8F_ERR_INVALID;
+    if (prologue != I8F_PRO_MODULATE && prologue != I8F_PRO_GELU_TANH && prologue != I8F_PRO_SILU_GATE) return I8F_ERR_INVALID;
     if (M < 0 || K < 0 || !valid_dtype(x_dtype)) return I8F_ERR_INVALID;
     if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
     if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
@@ -823,6 +845,7 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
     if (!scale || ldx < K) return I8F_ERR_INVALID;
     if (K > 0 && (!x || !q)) return I8F_ERR_INVALID;
     if (prologue == I8F_PRO_MODULATE && (rows_per_vec <= 0 || (K > 0 && (!mod_scale || !mod_shift)))) return I8F_ERR_INVALID;
+    if (prologue == I8F_PRO_SILU_GATE && (rows_per_vec <= 0 || (K > 0 && !mod_scale))) return I8F_ERR_INVALID;
     if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
     if (int rc = check_device()) return rc;
     if (rows_per_vec > 0x7fffffff) rows_per_vec = 0x7fffffff;  // M itself is below 2^31

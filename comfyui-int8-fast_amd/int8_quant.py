@@ -438,8 +438,9 @@ class Int8TensorwiseOps(manual_cast):
         def forward(self, x: Tensor, prologue: int = _lib.PRO_NONE, mod_scale: Tensor | None = None,
                     mod_shift: Tensor | None = None) -> Tensor:
             """The reference's forward(x) (int8_quant.py:703-778).  The optional arguments name the elementwise
-            operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, or _lib.PRO_MODULATE with
-            (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension -- which the W8A8 path
+            operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, _lib.PRO_MODULATE with
+            (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension, or _lib.PRO_SILU_GATE with
+            silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8 path
             then applies inside its quantiser instead of in a pass of its own (under torch.compile the graph
             rewrite of compile_ops does this without the caller's help)."""
             managed = self.comfy_cast_weights or len(self.weight_function) > 0 or len(self.bias_function) > 0
@@ -447,12 +448,19 @@ class Int8TensorwiseOps(manual_cast):
                 rows = x.numel() // max(1, x.shape[-1])
                 fusable = (self._is_quantized and rows > SMALL_BATCH_ROWS and self.lora_A is None
                            and not torch.compiler.is_compiling())
+                if fusable and prologue == _lib.PRO_SILU_GATE:   # the gate operand has x's shape and dtype, or torch does it
+                    fusable = isinstance(mod_scale, Tensor) and mod_scale.shape == x.shape and mod_scale.dtype == x.dtype
                 if fusable and prologue == _lib.PRO_MODULATE:
                     # vectors of another dtype or another broadcast pattern are torch's business (as under compile)
                     fusable = (isinstance(mod_scale, Tensor) and isinstance(mod_shift, Tensor) and x.dim() >= 2
                                and compile_ops.modulation_broadcasts_over_tokens(x, mod_scale, mod_shift))
                 if not fusable:   # every other path takes the operation as torch would have applied it
-                    x = F.gelu(x, approximate="tanh") if prologue == _lib.PRO_GELU_TANH else (1 + mod_scale) * x + mod_shift
+                    if prologue == _lib.PRO_GELU_TANH:
+                        x = F.gelu(x, approximate="tanh")
+                    elif prologue == _lib.PRO_SILU_GATE:
+                        x = F.silu(x) * mod_scale
+                    else:
+                        x = (1 + mod_scale) * x + mod_shift
                     prologue = _lib.PRO_NONE
 
             if not self._is_quantized:

@@ -76,8 +76,11 @@ typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
  *                      block's qkv and MLP projections; the three tensor operations
  *                      are each rounded to x's dtype, as torch's eager kernels do
  *   I8F_PRO_GELU_TANH  gelu(x, approximate="tanh") in binary32, rounded once to x's dtype
+ *   I8F_PRO_SILU_GATE  silu(x) * g[k], the gated activation in front of the down projection of a
+ *                      SwiGLU feed-forward (w2(silu(w1 x) * w3 x)): silu in binary32 rounded to x's
+ *                      dtype, then the product rounded to x's dtype, as torch's two eager kernels do
  */
-typedef enum i8f_prologue { I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2 } i8f_prologue;
+typedef enum i8f_prologue { I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2, I8F_PRO_SILU_GATE = 3 } i8f_prologue;
 
 /* Library version (I8F_VERSION of the build). */
 int i8f_version(void);
@@ -134,10 +137,12 @@ int i8f_quant_rowwise_grouped(const i8f_quant_group *groups, int n_groups, int x
  *   prologue      i8f_prologue
  *   mod_scale, mod_shift   I8F_PRO_MODULATE: [ceil(M / rows_per_vec), K] of x_dtype,
  *                 contiguous; row m uses vector m / rows_per_vec (one pair of vectors
- *                 per image of a batch); ignored otherwise
+ *                 per image of a batch).  I8F_PRO_SILU_GATE: mod_scale is the gate operand g,
+ *                 same layout (rows_per_vec = 1 for a gate tensor of x's shape), mod_shift
+ *                 is ignored.  Both ignored otherwise.
  * I8F_PRO_MODULATE is bit-identical to torch's three eager operations followed by
- * i8f_quant_rowwise; I8F_PRO_GELU_TANH agrees with torch's gelu to the last bits of
- * binary32 before the rounding to x_dtype (tests state the tolerance).
+ * i8f_quant_rowwise; I8F_PRO_GELU_TANH and I8F_PRO_SILU_GATE agree with torch's gelu / silu
+ * to the last bits of binary32 before the rounding to x_dtype (tests state the tolerance).
  */
 int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                                int prologue, const void *mod_scale, const void *mod_shift,

@@ -166,7 +166,7 @@ def quant_tensorwise(x, dtype_code):
     return q, s
 
 
-PRO_MODULATE, PRO_GELU_TANH = 1, 2
+PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE = 1, 2, 3
 
 
 def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
@@ -177,6 +177,9 @@ def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
     if kind == PRO_MODULATE:
         s, t = _arr(s, dtype_code).reshape(-1, K), _arr(t, dtype_code).reshape(-1, K)
         assert s.shape == t.shape and s.shape[0] * rows_per_vec >= M
+    elif kind == PRO_SILU_GATE:
+        s, t = _arr(s, dtype_code).reshape(-1, K), None
+        assert s.shape[0] * rows_per_vec >= M
     out = np.empty((M, K), dtype=x.dtype)
     _chk(lib().orc_prologue(_p(x), dtype_code, M, K, K, kind, _p(s) if s is not None else None,
                             _p(t) if t is not None else None, rows_per_vec, _p(out)), "prologue")

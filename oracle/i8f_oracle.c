@@ -255,13 +255,19 @@ int orc_quant_rowwise(const void *x, int dtype, int64_t M, int64_t K, int64_t ld
  *   kind 2  gelu(x, approximate="tanh") = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
  *           in binary32, rounded once to dtype (the tanh is the C library's: a
  *           tolerance reference in the last binary32 bits, not a bit pattern)
+ *   kind 3  silu(x) * g[k]: x / (1 + exp(-x)) in binary32 rounded to dtype, then the
+ *           product rounded to dtype (torch's silu and mul kernels; the gated activation of a
+ *           SwiGLU feed-forward, e.g. the z-image family the loader names,
+ *           int8_unet_loader.py:60-93); g is s, laid out like s of kind 1; expf is the C
+ *           library's: a tolerance reference like kind 2
  * out is [M,K] of dtype, contiguous.  Followed by orc_quant_rowwise it is the
  * oracle of the fused quantiser.
  */
 int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, int kind,
                  const void *s, const void *t, int64_t rows_per_vec, void *out) {
-    if (M < 0 || K < 0 || ldx < K || (kind != 1 && kind != 2)) return -1;
+    if (M < 0 || K < 0 || ldx < K || (kind != 1 && kind != 2 && kind != 3)) return -1;
     if (kind == 1 && (rows_per_vec <= 0 || !s || !t)) return -1;
+    if (kind == 3 && (rows_per_vec <= 0 || !s)) return -1;
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; ++m) {
         for (int64_t k = 0; k < K; ++k) {
@@ -272,6 +278,12 @@ int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, in
                 const float a = round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype);
                 const float b = round_to_dtype(a * xv, dtype);
                 v = b + load_as_f32(t, dtype, vi);
+            } else if (kind == 3) {
+                /* silu(x) * g as two tensor operations: x / (1 + exp(-x)) in binary32, rounded to the dtype, then
+                 * the product with the gate value, rounded again by the store below */
+                const size_t vi = (size_t)((m / rows_per_vec) * K + k);
+                const float a = round_to_dtype(xv / (1.0f + expf(-xv)), dtype);
+                v = a * load_as_f32(s, dtype, vi);
             } else {
                 const float kBeta = 0.7978845608028654f, kKappa = 0.044715f;
                 const float x3 = xv * xv * xv;

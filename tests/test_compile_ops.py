@@ -164,6 +164,44 @@ def test_graph_rewrite_respects_views_and_the_callers_shape(pkg):
     assert tuple(y.shape) == (2, 24, 512)
 
 
+def test_graph_rewrite_moves_the_swiglu_gate_into_the_quantiser(pkg):
+    """w2(silu(w1 x) * w3 x): the product feeding the down projection becomes its prologue, in either operand order;
+    a gate of another shape (broadcast by torch) is left alone."""
+    g = torch.Generator().manual_seed(12)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class SwiGlu(torch.nn.Module):
+        def __init__(self, flip):
+            super().__init__()
+            self.w1, self.w3, self.w2, self.flip = lin(512, 256), lin(512, 256), lin(256, 512), flip
+
+        def forward(self, x):
+            a, b = self.w1(x), self.w3(x)
+            return self.w2(b * F.silu(a) if self.flip else F.silu(a) * b)
+
+    x = torch.randn(2, 24, 256).bfloat16()
+    for flip in (False, True):
+        gm = torch._dynamo.export(SwiGlu(flip))(x).graph_module
+        assert pkg.compile_ops.fuse_prologues(gm) == 1
+        fused = [n for n in gm.graph.nodes if n.op == "call_function" and "int8_linear_prologue" in str(n.target)]
+        assert len(fused) == 1 and fused[0].args[1] == pkg._lib.PRO_SILU_GATE and fused[0].args[3] is None
+        assert not any("silu" in str(n.target) for n in gm.graph.nodes if n.op == "call_function")
+
+    class Broadcast(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w1, self.w2 = lin(512, 256), lin(256, 512)
+
+        def forward(self, x, gate):                      # gate [512]: not a tensor of the activation's shape
+            return self.w2(F.silu(self.w1(x)) * gate)
+    gm = torch._dynamo.export(Broadcast())(x, torch.randn(512).bfloat16()).graph_module
+    assert pkg.compile_ops.fuse_prologues(gm) == 0
+
+
 def test_modulation_broadcast_rule(pkg):
     ok = pkg.compile_ops.modulation_broadcasts_over_tokens
     x = torch.empty(2, 24, 256, dtype=torch.bfloat16)

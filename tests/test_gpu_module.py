@@ -276,6 +276,10 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
         a = lin(x, prologue=L.PRO_GELU_TANH)
         b = lin(F.gelu(x, approximate="tanh"))
         assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
+        gate = torch.randn(2, 20, 384, generator=g).bfloat16().to(dev)
+        a = lin(x, prologue=L.PRO_SILU_GATE, mod_scale=gate)
+        b = lin(F.silu(x) * gate)
+        assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
     # vectors that torch would broadcast differently, or of another dtype, are left to torch: same result as the
     # unfused expression (a [1, T, K] vector against a batch of 2 must not be dealt over the rows as if it were [2, 1, K])
     lin._use_quarot = False

@@ -155,6 +155,29 @@ def test_quant_rowwise_gelu_prologue_within_tolerance(L, dev, M, K, dt, rot, V):
         assert (np.abs(s.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
 
 
+@pytest.mark.parametrize("M,K,dt,rot,V", PROLOGUE_CASES)
+def test_quant_rowwise_silu_gate_prologue_within_tolerance(L, dev, M, K, dt, rot, V):
+    """silu(a) * b inside the quantiser (the gated activation in front of a SwiGLU down projection) against the oracle
+    (C expf) and against torch's silu and mul on the device followed by the plain quantiser; same bar as the GELU
+    prologue: scales within 2 ulp of the dtype, int8 at most 1 apart, at least 99.9 % equal (99 % with rotation)."""
+    a = (acts(M, K, dt).float() * 0.5).to(dt)
+    b = torch.randn(M, K, generator=G).to(dt)
+    aa, code = O.from_torch(a)
+    qo, so = O.quant_rowwise(O.prologue(aa, code, O.PRO_SILU_GATE, O.from_torch(b)[0], rows_per_vec=1), code, 128 if rot else 0)
+    q, s = L.quant_rowwise(a.to(dev), rotate=rot, prologue=L.PRO_SILU_GATE, mod_scale=b.to(dev))
+    q2, s2 = L.quant_rowwise(torch.nn.functional.silu(a.to(dev)) * b.to(dev), rotate=rot)
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-22}[dt]
+    for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+        d = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() <= (1e-2 if rot else 1e-3)
+        assert (np.abs(s.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
+    if M % V == 0 and V > 1:   # one gate row per group of rows (the vector form)
+        bv = torch.randn(V, K, generator=G).to(dt)
+        qa, sa = L.quant_rowwise(a.to(dev), rotate=rot, prologue=L.PRO_SILU_GATE, mod_scale=bv.to(dev))
+        qb, sb = L.quant_rowwise(a.to(dev), rotate=rot, prologue=L.PRO_SILU_GATE, mod_scale=bv.repeat_interleave(M // V, 0).to(dev))
+        assert torch.equal(qa, qb) and torch.equal(sa, sb)
+
+
 TENSORWISE_CASES = [
     # shape, dtype
     ((3072, 3072), torch.bfloat16), ((3072, 3072), torch.float32), ((1, 1), torch.float32), ((7,), torch.float16),

@@ -503,3 +503,28 @@ def test_prologue_gelu_tanh_agrees_with_torch(dt):
     assert (np.abs(got - w) <= ulp * np.abs(w) + 2.0**-23 * np.abs(x.float().numpy())).all()
     assert (got != w).mean() < (1e-2 if dt != torch.float32 else 0.5)
     assert got[0, 4] == 20.0 and got[0, 5] == 0.0 and got[0, 0] == 0.0
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+def test_prologue_silu_gate_agrees_with_torch(dt):
+    """silu(a) * b as torch's two eager kernels compute it: the oracle divides by 1 + expf(-a) with the C library's
+    expf, torch with its own vectorised exp, so the activated value may differ in the last bit of binary32, i.e. now
+    and then by one unit in the last place of the dtype before the product; the product of equal activations is equal."""
+    g = torch.Generator().manual_seed(33)
+    a = (torch.randn(64, 512, generator=g) * 3).to(dt)
+    b = torch.randn(64, 512, generator=g).to(dt)
+    a[0, :8] = torch.tensor([0.0, -0.0, 1e-6, -1e-6, 20.0, -20.0, 100.0, -100.0]).to(dt)
+    want = torch.nn.functional.silu(a) * b
+    got = O.to_f32(O.prologue(O.from_torch(a)[0], O.from_torch(a)[1], O.PRO_SILU_GATE, O.from_torch(b)[0], rows_per_vec=1), O.from_torch(a)[1])
+    w = want.float().numpy()
+    ulp = {torch.bfloat16: 2.0**-7, torch.float16: 2.0**-10, torch.float32: 2.0**-22}[dt]
+    # one unit of the activated value, carried through the product and its rounding
+    assert (np.abs(got - w) <= 2 * ulp * np.abs(w) + 1e-30).all()
+    assert (got != w).mean() < (1e-2 if dt != torch.float32 else 0.5)
+    assert got[0, 0] == 0.0 and got[0, 4] == np.float32((torch.tensor(20.0).to(dt) * b[0, 4]).float())   # silu(0) = 0, silu(20) rounds to 20
+    # one gate row for every three rows of a (the layout the kernel's vector form shares with the modulation)
+    b3 = torch.randn(4, 512, generator=g).to(dt)
+    a3 = a[:12]
+    got3 = O.prologue(O.from_torch(a3)[0], O.from_torch(a3)[1], O.PRO_SILU_GATE, O.from_torch(b3)[0], rows_per_vec=3)
+    want3 = O.prologue(O.from_torch(a3)[0], O.from_torch(a3)[1], O.PRO_SILU_GATE, O.from_torch(b3.repeat_interleave(3, 0))[0], rows_per_vec=1)
+    assert np.array_equal(got3, want3)
