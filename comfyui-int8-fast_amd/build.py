@@ -34,6 +34,7 @@ FLAGS = [
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-mllvm", "-amdgpu-kernarg-preload-count=16",
+    "-DI8F_BUILD_CONTRACT=1",   # i8f_common.hpp refuses to compile without it: a build that bypasses these flags fails
     "-Wall",
     "-Wno-unused-function",
     "-Wno-inline-asm",   # the global->LDS loads name m0 in their clobber list, which clang reports as "reserved"

@@ -957,6 +957,10 @@ using CfgB192 = Cfg<256, 192, 128, 4, 2, 2, 6, 0x4300, 16, I8F_WST>;  // 8 waves
 using CfgMid = Cfg<128, 128, 128, 2, 2, 2, 8>;   // 4 waves, 2 x 32 KB stages, two workgroups per CU (10 % slower with the 16x16x64 MFMA: 32x32x32)
 using CfgTall = Cfg<288, 256, 128, 3, 4, 2, 8, 0, 16>;  // 12 waves of 96 x 64, 2 x 72 KB stages
 using CfgWide = Cfg<256, 288, 128, 4, 3, 2, 8, 0, 16>;  // 12 waves of 64 x 96, the same transposed
+// (Workgroups beyond the tile count that do nothing but touch, a few K-tiles ahead, the W lines the tiles of their XCD are
+// about to request -- they land on the CUs a 216-tile launch leaves idle, since a workgroup of this kernel takes a CU's
+// whole LDS -- were measured and are not kept: 39.8 us against 38.7 us at 4608 x 3072 x 3072, 130.3 against 125.2 us at
+// K = 12288.  The misses they take off the busy CUs do not pay for what their requests add to the XCD's L2 queues.)
 // (A 288 x 192 tile of twelve 96 x 48 waves, which covers 4608 x 3072 in exactly 256 workgroups, was measured and is not
 // kept: 42.9 us against 37.7 us for the 216 tiles of 256 x 256.  It moves 11 % more bytes per multiply-accumulate through a
 // load path that is already the bound, and with all 256 CUs multiplying the clock settles 8 % lower.)

@@ -6,6 +6,20 @@
 // LoRA merge depend on it.
 #pragma once
 
+// The numerical contract and some hand-scheduled assembly depend on how these sources are compiled, so a build with
+// other flags must fail instead of producing a library that is subtly wrong: the build script passes
+// -DI8F_BUILD_CONTRACT=1 together with -ffp-contract=off, -fno-fast-math, -fhip-fp32-correctly-rounded-divide-sqrt and
+// the packed-FP32 feature switched off (the flags a macro cannot see); fast-math and finite-math are seen here.
+#if !defined(I8F_BUILD_CONTRACT) || I8F_BUILD_CONTRACT != 1
+#error "compile these sources with the flags of comfyui-int8-fast_amd/build.py (FLAGS): the results depend on them"
+#endif
+#if defined(__FAST_MATH__) || defined(__FINITE_MATH_ONLY__) && __FINITE_MATH_ONLY__
+#error "fast-math changes the rounding of the quantiser, the epilogue and the merge: build without it"
+#endif
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "this library is written for gfx950 only"
+#endif
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
