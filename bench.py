@@ -641,12 +641,17 @@ def main():
         tg = extra["target_gemm_4608x3072x3072"]
         t_traffic, t_note = gemm_traffic(L, 4608, 3072, 3072)
         t_alg = gemm_algorithmic_bytes(4608, 3072, 3072, bias=False)
+        # headline = operands that are NOT in the memory-side cache (12 operand sets in turn), which is what a layer
+        # inside a model sees; the loop over one operand set is reported beside it
         line["roofline_target"] = {"bound": "mfma", "shape": "M=4608, N=K=3072, W8A8 rowwise, bf16 out", "tile": tg["tile"],
-                                   "ops_per_launch": 2 * 4608 * 3072 * 3072, "avg_launch_us": tg["median_us"],
-                                   "achieved": tg["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": tg["frac_of_int8_peak"],
-                                   "operands": "the same operands in a loop (resident in the 256 MB memory-side cache)",
+                                   "ops_per_launch": 2 * 4608 * 3072 * 3072, "avg_launch_us": tg["cold_operands_median_us"],
+                                   "achieved": tg["cold_operands_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                                   "frac": tg["cold_operands_frac_of_int8_peak"],
+                                   "operands": "12 operand sets in turn (623 MB: none of them in the 256 MB memory-side cache)",
                                    "cold_operands_avg_launch_us": tg["cold_operands_median_us"],
                                    "cold_operands_frac": tg["cold_operands_frac_of_int8_peak"],
+                                   "warm_operands_avg_launch_us": tg["median_us"], "warm_operands_frac": tg["frac_of_int8_peak"],
+                                   "vendor_int_mm_warm_us": tg.get("vendor_int_mm_median_us"),
                                    "traffic": t_traffic, "algorithmic_bytes": t_alg,
                                    "traffic_over_algorithmic": None if t_traffic is None else round(t_traffic / t_alg, 2)}
         if t_note:

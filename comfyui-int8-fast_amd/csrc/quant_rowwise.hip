@@ -137,6 +137,63 @@ __device__ __forceinline__ void rotate_chunk(float (&v)[Elem<DT>::EPC], int lane
     for (int j = 0; j < EPC; ++j) v[j] = round_to_dtype<DT>(v[j] * h);
 }
 
+// binary32 rows: a 128-block is 32 chunks of 4 elements, held by an aligned group of 32 lanes.  Strides 1, 2 of the
+// butterfly stay inside a lane; strides 4 ... 32 pair chunks c and c ^ 1, c ^ 2, c ^ 4, c ^ 8, which DPP reaches as lanes
+// l ^ 1, l ^ 2 (quad permutes), l ^ 7 (mirror of 8 lanes) and l ^ 15 (mirror of a row of 16) if lane l holds chunk
+//   c(l) = (l & 3) ^ (7 if bit 2 of l) ^ (12 if bit 3 of l)     (linear over GF(2): c(l ^ 7) = c(l) ^ 4, c(l ^ 15) = c(l) ^ 8)
+// of its group of 16; stride 64 pairs the two rows of 16 of the group through one lane exchange.  As in rotate_run16 a
+// DPP stage is own + sign * other (one fused multiply-add whose product is exact), which leaves the upper chunk of a
+// pair with the negative of the butterfly's value; both lanes of every later pair carry the same accumulated sign, and
+// the product of the four signs is folded into the final multiplication.  Same fixed-order butterfly, 4 of the 5
+// cross-lane stages without an LDS round trip.
+__device__ __forceinline__ int chunk_of_lane16(int l) { return (l & 3) ^ ((l & 4) ? 7 : 0) ^ ((l & 8) ? 12 : 0); }
+
+#define I8F_DPP_FMAC4(ctrl)                                                                                              \
+    asm volatile("s_nop 1\n\t"                                                                                           \
+                 "v_fmac_f32_dpp %0, %0, %4 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"                        \
+                 "v_fmac_f32_dpp %1, %1, %4 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"                        \
+                 "v_fmac_f32_dpp %2, %2, %4 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"                        \
+                 "v_fmac_f32_dpp %3, %3, %4 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"                        \
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3])                                                       \
+                 : "v"(sign))
+template <int STAGE>
+__device__ __forceinline__ void dpp_fmac4(float (&v)[4], float sign) {
+    if constexpr (STAGE == 0) I8F_DPP_FMAC4("quad_perm:[1,0,3,2]");
+    else if constexpr (STAGE == 1) I8F_DPP_FMAC4("quad_perm:[2,3,0,1]");
+    else if constexpr (STAGE == 2) I8F_DPP_FMAC4("row_half_mirror");
+    else I8F_DPP_FMAC4("row_mirror");
+}
+
+// v: the chunk chunk_of_lane16(lane % 16) + 16 (lane / 16 % 2) of the lane's 128-block
+__device__ __forceinline__ void rotate_chunk_f32(float (&v)[4], int lane) {
+#pragma unroll
+    for (int s = 1; s < 4; s <<= 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if ((j & s) == 0) {
+                const float lo = v[j], hi = v[j + s];
+                v[j] = lo + hi;
+                v[j + s] = lo - hi;
+            }
+        }
+    }
+    const int c = chunk_of_lane16(lane & 15);
+    const float s0 = (c & 1) ? -1.0f : 1.0f, s1 = (c & 2) ? -1.0f : 1.0f, s2 = (c & 4) ? -1.0f : 1.0f, s3 = (c & 8) ? -1.0f : 1.0f;
+    dpp_fmac4<0>(v, s0);
+    dpp_fmac4<1>(v, s1);
+    dpp_fmac4<2>(v, s2);
+    dpp_fmac4<3>(v, s3);
+    const bool upper = (lane & 16) != 0;   // both lanes of this pair carry the same accumulated sign
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float other = __shfl_xor(v[j], 16, 64);
+        v[j] = upper ? (other - v[j]) : (v[j] + other);
+    }
+    const float h = hadamard_entry<I8F_F32>() * (s0 * s1 * s2 * s3);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = v[j] * h;
+}
+
 // TPR threads share a row (64, 256 or 1024); each holds NCH chunks of it.
 template <int DT, bool ROT, int TPR, int NCH>
 __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void quant_rows_kernel(
@@ -152,11 +209,14 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void quant_rows_kernel(
     const bool row_ok = m < M;
     const int nchunks = (int)(K / EPC);
     const char *xrow = x + (row_ok ? m : 0) * ldx_bytes;
+    // which chunk of its step a lane holds: its own, or (rotating binary32 rows) the one that lets DPP pair the lanes
+    constexpr bool DPP32 = ROT && DT == I8F_F32;
+    const int tc = DPP32 ? ((t & ~15) | chunk_of_lane16(t & 15)) : t;
 
     float v[NCH][EPC];
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-        const int c = i * TPR + t;
+        const int c = i * TPR + tc;
         if (row_ok && c < nchunks) {
             load_chunk<DT>(xrow + (int64_t)c * 16, v[i]);
         } else {
@@ -167,7 +227,10 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void quant_rows_kernel(
 
     if constexpr (ROT) {
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) rotate_chunk<DT>(v[i], t);
+        for (int i = 0; i < NCH; ++i) {
+            if constexpr (DPP32) rotate_chunk_f32(v[i], t);
+            else rotate_chunk<DT>(v[i], t);
+        }
     }
 
     float amax = 0.0f;
@@ -194,7 +257,7 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void quant_rows_kernel(
     int8_t *qrow = q + m * K;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-        const int c = i * TPR + t;
+        const int c = i * TPR + tc;
         if (c < nchunks) {
             uint32_t packed[EPC / 4];
 #pragma unroll
