@@ -82,7 +82,9 @@ __device__ __forceinline__ uint32_t f32x2_to_f16x2_bits(float lo, float hi) {
 // value rounded to the storage dtype and widened again
 template <int DT>
 __device__ __forceinline__ float round_to_dtype(float v) {
-    if constexpr (DT == I8F_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+    // bfloat16: the packed conversion with a zero in the low half leaves the rounded value in the high half, which IS
+    // its binary32 form: one instruction rounds and widens
+    if constexpr (DT == I8F_BF16) return __uint_as_float(f32x2_to_bf16x2_bits(0.0f, v));
     else if constexpr (DT == I8F_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
     else return v;
 }
