@@ -390,16 +390,6 @@ def lora_side_fusable(M: int, N: int, K: int, rank: int, out_dtype, side_dtype) 
             and K % 128 == 0 and N % 8 == 0 and M > 0)
 
 
-def lora_side_pays(M: int, N: int, K: int) -> bool:
-    """Whether the side branch inside the epilogue is the cheaper way to add a low-rank product to this GEMM.  The
-    fused form exists for the eight-wave tiles: a problem whose plain GEMM takes a twelve-wave tile (288 x 256 or
-    256 x 288, e.g. 4608 x 12288 x 3072) would fall back to 256 x 256 tiles and lose more than the [M,N] side tensor
-    costs (measured 202 us fused against 199 us with a side tensor added in the epilogue), so such problems form
-    the side tensor with torch and add it in the epilogue."""
-    bm, bn, _stages = gemm_tile(M, N, K)
-    return (bm, bn) not in ((288, 256), (256, 288))
-
-
 def linear_w8a8_lora(a, a_scale, w, w_scale, bias, side_t, side_b, alpha=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None):
     """linear_w8a8 plus the low-rank side branch side_t [M,r] @ side_b [N,r].T (both of out_dtype), formed inside the
     GEMM epilogue: round(y + round(round(side) * alpha)).  A rank that is not a multiple of 16 is padded with zero

@@ -259,12 +259,18 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     // outputs), padded so that the transposing writes do not collide on banks.
     constexpr int ROW_BYTES = C::WTN * OB;
     constexpr int PITCH = ROW_BYTES + (OB == 2 ? 8 : 16);
-    constexpr int EPI_STRIPS = (OB == 2 || MI == 1) ? MI : MI / 2;
+    // (one strip at a time with a side branch, whose operands take the rest of the memory)
+    constexpr int EPI_STRIPS = SIDE ? 1 : ((OB == 2 || MI == 1) ? MI : MI / 2);
     constexpr int WAVE_BYTES = EPI_STRIPS * 32 * PITCH;
     // The epilogue operands of the tile (token scales, weight scales, bias) are staged behind the waves' transpose
     // buffers, in memory that belongs to the K-tile stages while the main loop runs.
     constexpr int EPI_OPS_OFF = WAVE_BYTES * NW, EPI_OPS_BYTES = 4 * (BM + 2 * BN);
-    constexpr int SMEM_BYTES = C::LDS_BYTES > EPI_OPS_OFF + EPI_OPS_BYTES ? C::LDS_BYTES : EPI_OPS_OFF + EPI_OPS_BYTES;
+    // The side branch's operands of the tile, BM rows of side_t and then BN rows of side_b, up to SIDE_RMAX ranks of
+    // 2 bytes per row at a pitch that keeps 16-byte pieces aligned and spreads the rows over the banks.
+    constexpr int SIDE_RMAX = 64, SIDE_PITCH = SIDE_RMAX * 2 + 16;
+    constexpr int SIDE_OFF = EPI_OPS_OFF + EPI_OPS_BYTES, SIDE_BYTES = SIDE ? (BM + BN) * SIDE_PITCH : 0;
+    static_assert(SIDE_OFF % 16 == 0, "16-byte pieces");
+    constexpr int SMEM_BYTES = C::LDS_BYTES > SIDE_OFF + SIDE_BYTES ? C::LDS_BYTES : SIDE_OFF + SIDE_BYTES;
     static_assert(SMEM_BYTES + (SPLITK ? 16 : 0) <= 160 * 1024, "LDS");
     __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
     float *const s_xs = (float *)(smem + EPI_OPS_OFF), *const s_ws = s_xs + BM, *const s_bias = s_ws + BN;
@@ -701,8 +707,21 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
             }
         }
     }
+    if constexpr (SIDE) {
+        // side_t rows m0 ... and side_b rows n0 ... of the tile, 16 bytes (8 ranks) per thread and step; rows beyond
+        // the matrix repeat its last row (their outputs are not stored)
+        const int cpr = g.side_rank >> 3;  // 16-byte pieces per row
+        for (int c = tid; c < (BM + BN) * cpr; c += C::NT) {
+            const int row = c / cpr, cc = c - row * cpr;
+            const char *src = row < BM ? (const char *)g.side_t + (int64_t)min(m0 + row, gM - 1) * g.side_rank * 2
+                                       : (const char *)g.side_b + (int64_t)min(n0 + row - BM, gN - 1) * g.side_rank * 2;
+            *(uint4 *)(smem + SIDE_OFF + row * SIDE_PITCH + cc * 16) = *(const uint4 *)(src + cc * 16);
+        }
+    }
     __syncthreads();  // the stages are dead (reused as per-wave transpose buffers), the operands staged
     char *ebuf = smem + wave * WAVE_BYTES;
+    [[maybe_unused]] const char *const s_side_t = smem + SIDE_OFF + (wm * C::WTM) * SIDE_PITCH;
+    [[maybe_unused]] const char *const s_side_b = smem + SIDE_OFF + (BM + wn * C::WTN) * SIDE_PITCH;
 
     // scale, bias, round: the flags are wave-uniform, so the variant is chosen once
     // scale, bias, round.  The per-column operands (4 consecutive n per lane and MFMA block) are
@@ -789,18 +808,16 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                     [[maybe_unused]] v4i bfr[M16 ? 1 : RMAX / 16];
                     [[maybe_unused]] v2i bfr16[RMAX / 16];
                     if constexpr (SIDE && !M16) {
-                        const int n = min(n0 + wn * C::WTN + j * 32 + l32, gN - 1);
 #pragma unroll
                         for (int ks = 0; ks < RMAX / 16; ++ks)
                             if (ks * 16 < g.side_rank)
-                                bfr[ks] = *(const v4i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lhalf * 8) * 2);
+                                bfr[ks] = *(const v4i *)(s_side_b + (j * 32 + l32) * SIDE_PITCH + (ks * 16 + lhalf * 8) * 2);
                     }
                     if constexpr (SIDE && M16) {
-                        const int n = min(n0 + wn * C::WTN + j * 16 + l16, gN - 1);
 #pragma unroll
                         for (int ks = 0; ks < RMAX / 16; ++ks)
                             if (ks * 16 < g.side_rank)
-                                bfr16[ks] = *(const v2i *)((const char *)g.side_b + ((int64_t)n * g.side_rank + ks * 16 + lq * 4) * 2);
+                                bfr16[ks] = *(const v2i *)(s_side_b + (j * 16 + l16) * SIDE_PITCH + (ks * 16 + lq * 4) * 2);
                     }
 #pragma unroll
                     for (int is = 0; is < EPI_STRIPS; ++is) {
@@ -810,14 +827,13 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                         [[maybe_unused]] float sd[16];
                         constexpr int SDT = OUT == OUT_F16 ? I8F_F16 : I8F_BF16;
                         if constexpr (SIDE && !M16) {
-                            const int m = min(m0 + wm * C::WTM + i * 32 + l32, gM - 1);
                             v16f sacc;
 #pragma unroll
                             for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
 #pragma unroll
                             for (int ks = 0; ks < RMAX / 16; ++ks) {
                                 if (ks * 16 < g.side_rank) {
-                                    const v4i tfr = *(const v4i *)((const char *)g.side_t + ((int64_t)m * g.side_rank + ks * 16 + lhalf * 8) * 2);
+                                    const v4i tfr = *(const v4i *)(s_side_t + (i * 32 + l32) * SIDE_PITCH + (ks * 16 + lhalf * 8) * 2);
                                     sacc = side_mfma<OUT>(bfr[ks], tfr, sacc);
                                 }
                             }
@@ -831,12 +847,11 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                         if constexpr (SIDE && M16) {
 #pragma unroll
                             for (int u = 0; u < 2; ++u) {
-                                const int m = min(m0 + wm * C::WTM + i * 32 + u * 16 + l16, gM - 1);
                                 v4f sacc = (v4f)0.0f;
 #pragma unroll
                                 for (int ks = 0; ks < RMAX / 16; ++ks) {
                                     if (ks * 16 < g.side_rank) {
-                                        const v2i tfr = *(const v2i *)((const char *)g.side_t + ((int64_t)m * g.side_rank + ks * 16 + lq * 4) * 2);
+                                        const v2i tfr = *(const v2i *)(s_side_t + (i * 32 + u * 16 + l16) * SIDE_PITCH + (ks * 16 + lq * 4) * 2);
                                         sacc = side_mfma16<OUT>(bfr16[ks], tfr, sacc);
                                     }
                                 }
@@ -979,7 +994,7 @@ int launch_cfg(GemmArgs &g, hipStream_t st) {
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
     const int flags = (g.row_scale ? 1 : 0) | (g.bias_dtype << 1);  // what the prologue wants to know of the epilogue
     if (g.side_t) {  // validated by the entry point: K % BK == 0 here
-        if constexpr ((OUT == OUT_BF16 || OUT == OUT_F16) && C::NT <= 512) {  // (twelve-wave tiles have no registers to spare for it)
+        if constexpr (OUT == OUT_BF16 || OUT == OUT_F16) {
             hipLaunchKernelGGL((gemm_i8_kernel<C, OUT, false, true>), dim3((unsigned)tiles), dim3(C::NT), 0, st, g.x, g.w, g.M, g.N,
                                g.K, g.tiles_m, g.tiles_n, g.xs, g.ws, g.bias, flags, g);
             return check_launch();
@@ -1155,7 +1170,6 @@ int launch(GemmArgs &g, hipStream_t st) {
         return check_launch();
     }
     Tile t = choose_tile(g.M, g.N);
-    if (g.side_t && (t == TILE_TALL || t == TILE_WIDE)) t = TILE_BIG;  // the side branch exists for the eight-wave tiles
     int splits = 1;
     if (g.partials && !g.side_t) choose_split(g.M, g.N, g.K, t, splits);
     g.splits = splits;

@@ -694,6 +694,8 @@ def test_config4_fused_merge_against_library_product_delta(L, dev):
     (4608, 3072, 3072, 32, torch.bfloat16, None, True), (512, 12288, 3072, 64, torch.bfloat16, 1.25, True),
     (4608, 12288, 3072, 32, torch.bfloat16, None, True), (130, 96, 128, 24, torch.bfloat16, None, False),
     (257, 3080, 640, 8, torch.float16, 2.0, True),
+    # the twelve-wave tiles: 256 x 288 (rank 48), 288 x 256 with a ragged last row and column of tiles
+    (4096, 9216, 256, 48, torch.bfloat16, None, True), (4600, 12280, 128, 16, torch.float16, 0.75, True),
 ])
 def test_linear_w8a8_lora_side_branch(L, dev, M, N, K, r, dt, alpha, row):
     """out = round(y + round(round(t @ B.T) * alpha)) with the rank-r product formed inside the GEMM epilogue, against
