@@ -65,13 +65,14 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a8.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_splitk.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp, i64, vp]
+    L.i8f_linear_w8a8_grouped.argtypes = [vp, i32, i32, i32, i32, i64, i64, i32, vp, i64, vp]
     L.i8f_linear_w8a8_workspace_bytes.argtypes = []
     L.i8f_linear_w8a8_workspace_bytes.restype = i64
     L.i8f_linear_w8a8_lora.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i64, i32, f32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_lora",
+    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -81,7 +82,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue",
-    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
 
@@ -382,6 +383,82 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
                                             0 if work is None else work.numel(), _stream(a)),
                "i8f_linear_w8a8_splitk")
     return out
+
+
+class _LinearGroup(ctypes.Structure):
+    _fields_ = [("a", ctypes.c_void_p), ("a_scale", ctypes.c_void_p), ("w", ctypes.c_void_p), ("w_scale", ctypes.c_void_p),
+                ("w_scale_host", ctypes.c_float), ("bias", ctypes.c_void_p), ("addend", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("M", ctypes.c_int64)]
+
+
+MAX_LINEAR_GROUPS = 4
+
+
+def _addr(t):
+    return None if t is None else t.data_ptr()
+
+
+def linear_w8a8_grouped(problems, out_dtype=torch.bfloat16, order=EPI_TORCH, outs=None):
+    """linear_w8a8 for several problems of one layer shape, each (a, a_scale, w, w_scale, bias) or
+    (a, a_scale, w, w_scale, bias, addend) with its own tensors: the image and the text tokens of a double-stream
+    transformer block through the same projection.  One launch where the library finds that the small problems' tiles
+    fit into the compute units the largest one's last round leaves idle, else one launch per problem; problems that do
+    not share N, K, the scale mode and the bias dtype (or more than MAX_LINEAR_GROUPS of them) are launched one by one
+    from here.  outs: optional list of contiguous [M_i, N] tensors of out_dtype to write into.
+    -> list of outputs, bit-identical to separate linear_w8a8 calls."""
+    problems = [tuple(p) + (None,) * (6 - len(p)) for p in problems]
+    if not problems:
+        return []
+    if outs is not None and len(outs) != len(problems):
+        raise ValueError("outs must hold one tensor per problem")
+    prepared = []
+    for a, a_scale, w, w_scale, bias, addend in problems:
+        a, w = _i8_matrix(a, "a"), _i8_matrix(w, "w")
+        M, K = a.shape
+        N, K2 = w.shape
+        if K != K2:
+            raise ValueError(f"K mismatch: a has {K}, w has {K2}")
+        _dev(a_scale, "a_scale")
+        a_scale = a_scale.reshape(-1).contiguous()
+        if a_scale.numel() != M or a_scale.dtype != torch.float32:
+            raise ValueError("a_scale must be float32 with M elements")
+        ws, ws_host, mode = _scale(w_scale, N, a.device)
+        bias, bcode = _bias_arg(bias, N, a.device)
+        if addend is not None:
+            _dev(addend, "addend")
+            if addend.numel() != M * N or addend.dtype != out_dtype:
+                raise ValueError(f"addend must have {M * N} elements of {out_dtype}")
+            addend = addend.reshape(M, N).contiguous()
+        for name, t in (("w", w), ("a_scale", a_scale), ("addend", addend)):
+            if isinstance(t, torch.Tensor) and t.device != a.device:
+                raise ValueError(f"{name} is on {t.device}, a is on {a.device}")
+        prepared.append((a, a_scale, w, ws, ws_host, mode, bias, bcode, addend, M, N, K))
+    first = prepared[0]
+    bcodes = {p[7] for p in prepared if p[6] is not None}
+    same = (len(prepared) <= MAX_LINEAR_GROUPS and len(bcodes) <= 1
+            and all(p[10] == first[10] and p[11] == first[11] and p[5] == first[5] and p[0].device == first[0].device for p in prepared))
+    if not same:
+        return [linear_w8a8(p[0], p[1], p[2], src[3], p[6], out_dtype, order, None if outs is None else outs[i], addend=p[8])
+                for i, (p, src) in enumerate(zip(prepared, problems))]
+    N, K, mode, device = first[10], first[11], first[5], first[0].device
+    if outs is None:
+        outs = [torch.empty((p[9], N), dtype=out_dtype, device=device) for p in prepared]
+    else:
+        for p, o in zip(prepared, outs):
+            if tuple(o.shape) != (p[9], N) or not o.is_contiguous() or o.dtype != out_dtype or o.device != device:
+                raise ValueError(f"outs: expected a contiguous [{p[9]},{N}] tensor of {out_dtype} on {device}")
+    groups = (_LinearGroup * len(prepared))()
+    for g, p, o in zip(groups, prepared, outs):
+        g.a, g.a_scale, g.w, g.w_scale, g.w_scale_host = _addr(p[0]), _addr(p[1]), _addr(p[2]), _addr(p[3]), p[4]
+        g.bias, g.addend, g.out, g.M = _addr(p[6]), _addr(p[8]), _addr(o), p[9]
+    with _on(device):
+        work = None
+        for p in prepared:   # (used only if the library launches the problems one by one and one of them has a long K)
+            work = work if work is not None else _splitk_workspace(p[0], p[9], N, K)
+        _check(lib().i8f_linear_w8a8_grouped(ctypes.byref(groups), len(prepared), mode, bcodes.pop() if bcodes else 0,
+                                             dtype_code(out_dtype), N, K, order, _ptr(work), 0 if work is None else work.numel(),
+                                             _stream(first[0])), "i8f_linear_w8a8_grouped")
+    return outs
 
 
 def lora_side_fusable(M: int, N: int, K: int, rank: int, out_dtype, side_dtype) -> bool:

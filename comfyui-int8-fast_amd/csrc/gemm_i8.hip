@@ -5,6 +5,9 @@
 namespace i8f {
 namespace gemm {
 template int launch<OUT_BF16>(GemmArgs &, hipStream_t);
+template int launch_group<OUT_BF16>(GemmArgs *, int, hipStream_t);
+extern template int launch_group<OUT_F16>(GemmArgs *, int, hipStream_t);
+extern template int launch_group<OUT_F32>(GemmArgs *, int, hipStream_t);
 extern template int launch<OUT_F16>(GemmArgs &, hipStream_t);
 extern template int launch<OUT_F32>(GemmArgs &, hipStream_t);
 extern template int launch<OUT_I32>(GemmArgs &, hipStream_t);
@@ -92,6 +95,40 @@ extern "C" int i8f_linear_w8a8(const int8_t *a, const float *a_scale, const int8
                                int out_dtype, int64_t M, int64_t N, int64_t K, int order, void *stream) {
     return i8f_linear_w8a8_add(a, a_scale, w, w_scale, w_scale_host, scale_mode, bias, bias_dtype, nullptr, out,
                                out_dtype, M, N, K, order, stream);
+}
+
+extern "C" int i8f_linear_w8a8_grouped(const i8f_linear_group *groups, int n_groups, int scale_mode, int bias_dtype, int out_dtype,
+                                       int64_t N, int64_t K, int order, void *workspace, int64_t workspace_bytes, void *stream) {
+    using namespace i8f;
+    using namespace i8f::gemm;
+    if (n_groups < 0 || (n_groups > 0 && !groups) || N < 0 || K < 0) return I8F_ERR_INVALID;
+    if (workspace && (workspace_bytes < SPLITK_WORKSPACE_BYTES || (uintptr_t)workspace % 16)) return I8F_ERR_INVALID;
+    if (!valid_dtype(out_dtype) || !valid_dtype(bias_dtype)) return I8F_ERR_INVALID;
+    if (scale_mode != I8F_SCALE_TENSOR && scale_mode != I8F_SCALE_ROW) return I8F_ERR_INVALID;
+    if (order != I8F_EPI_TORCH && order != I8F_EPI_FUSED) return I8F_ERR_INVALID;
+    if (n_groups > I8F_MAX_LINEAR_GROUPS) return I8F_ERR_UNSUPPORTED;
+    GemmArgs gs[I8F_MAX_LINEAR_GROUPS];
+    int n = 0;
+    for (int i = 0; i < n_groups; ++i) {
+        const i8f_linear_group &p = groups[i];
+        if (int rc = validate(p.a, p.w, p.M, N, K, p.out)) return rc;
+        if (p.M == 0 || N == 0) continue;
+        if (!p.a_scale || (scale_mode == I8F_SCALE_ROW && !p.w_scale)) return I8F_ERR_INVALID;
+        GemmArgs g{};
+        g.x = p.a, g.w = p.w, g.M = (int)p.M, g.N = (int)N, g.K = (int)K, g.out = p.out;
+        g.xs = p.a_scale, g.ws = p.w_scale, g.ws_host = p.w_scale_host, g.row_scale = scale_mode == I8F_SCALE_ROW;
+        g.bias = p.bias, g.bias_dtype = bias_dtype, g.order = order, g.addend = p.addend;
+        if (workspace) g.arrivals = (unsigned *)workspace, g.partials = (int *)((char *)workspace + SPLITK_COUNTER_BYTES);
+        gs[n++] = g;
+    }
+    if (n == 0) return I8F_OK;
+    if (int rc = check_device()) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (out_dtype) {
+    case I8F_BF16: return launch_group<OUT_BF16>(gs, n, st);
+    case I8F_F16: return launch_group<OUT_F16>(gs, n, st);
+    default: return launch_group<OUT_F32>(gs, n, st);
+    }
 }
 
 extern "C" int i8f_gemm_tile(int64_t M, int64_t N, int64_t K, int *bm, int *bn, int *stages) {

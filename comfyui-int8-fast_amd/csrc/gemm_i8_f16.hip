@@ -4,5 +4,6 @@
 namespace i8f {
 namespace gemm {
 template int launch<OUT_F16>(GemmArgs &, hipStream_t);
+template int launch_group<OUT_F16>(GemmArgs *, int, hipStream_t);
 }  // namespace gemm
 }  // namespace i8f

@@ -242,10 +242,12 @@ __device__ __forceinline__ uint4 add_rounded(uint4 y, uint4 s) {
 // What the prologue needs (operand pointers, sizes, tile counts) comes first in the argument list: the
 // first 16 dwords of the kernel arguments are preloaded into SGPRs at wave launch, the rest (epilogue
 // operands) is fetched by scalar loads that have the whole main loop to land.
+// (The body is shared by the kernel of one problem and the kernel of a group of problems: wg_id is the workgroup's
+// number within its problem, gout / gaddend / ws_host that problem's output, addend and host-side weight scale.)
 template <class C, int OUT, bool KTAIL, bool SIDE = false, bool SPLITK = false>
-__global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
-                                                        const float *gxs, const float *gws, const void *gbias, int flags,
-                                                        const GemmArgs g) {
+__device__ __forceinline__ void gemm_i8_body(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
+                                             const float *gxs, const float *gws, const void *gbias, int flags, const GemmArgs &g,
+                                             const int wg_id, void *gout, const void *gaddend, const float ws_host) {
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NJ = C::NJ, CB = C::CB, CPR = C::CPR;
     constexpr int S = C::STAGES, WS = C::WSTAGES;
     constexpr bool ASYM = WS != S;  // the W tile one stage deeper than the X tile
@@ -285,7 +287,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     int tile_m, tile_n;
     {
         const int T = tiles_m * tiles_n;
-        const int bid = SPLITK ? __builtin_amdgcn_readfirstlane((int)blockIdx.x % T) : (int)blockIdx.x;  // the K slices of a tile are T workgroup ids apart
+        const int bid = SPLITK ? __builtin_amdgcn_readfirstlane(wg_id % T) : wg_id;  // the K slices of a tile are T workgroup ids apart
         const int per = (T + 7) / 8;
         const int tall = (T % 8 == 0) ? 8 : (T % 8);
         const int xcd = bid % 8, loc = bid / 8;
@@ -334,7 +336,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
     const int KT_all = (K + BK - 1) / BK;
     // (integer division runs on the vector ALUs: readfirstlane brings the quotients back to scalar registers, where the
     // K offset of the loads has to be)
-    [[maybe_unused]] const int slice = SPLITK ? __builtin_amdgcn_readfirstlane((int)blockIdx.x / (tiles_m * tiles_n)) : 0;
+    [[maybe_unused]] const int slice = SPLITK ? __builtin_amdgcn_readfirstlane(wg_id / (tiles_m * tiles_n)) : 0;
     const int kt_per = SPLITK ? __builtin_amdgcn_readfirstlane((KT_all + g.splits - 1) / g.splits) : KT_all;
     const int kt_first = slice * kt_per;
     const int KT = SPLITK ? max(min(kt_per, KT_all - kt_first), 0) : KT_all;
@@ -637,7 +639,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         // agree, and the count is taken once this workgroup's stores are acknowledged: no cache-wide write-back or
         // invalidate, which a release/acquire fence pair at agent scope would cost every workgroup on the XCD.
         __shared__ unsigned s_arrived;
-        const int T = tiles_m * tiles_n, tile = __builtin_amdgcn_readfirstlane((int)blockIdx.x % T);
+        const int T = tiles_m * tiles_n, tile = __builtin_amdgcn_readfirstlane(wg_id % T);
         constexpr int QUADS = MI * NJ * QPB;
         static_assert(QUADS % 4 == 0, "the partial sums are read back four quads at a time");
         int *mine = g.partials + ((int64_t)slice * T + tile) * (BM * BN);
@@ -685,7 +687,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         if (tid == 0) __hip_atomic_store(g.arrivals + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     }
     if constexpr (OUT != OUT_I32) {
-        if (!gws) ws_one = g.ws_host;
+        if (!gws) ws_one = ws_host;
 #pragma unroll
         for (int u = 0; u < XS_PER; ++u) {
             const int t = tid + u * C::NT;
@@ -891,8 +893,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                 {
                     const int64_t off = ((int64_t)mm * gN + nn) * OB;
                     uint4 v = val;
-                    if (g.addend) v = add_rounded<OUT>(v, *(const uint4 *)((const char *)g.addend + off));
-                    stream_store16((char *)g.out + off, v);
+                    if (gaddend) v = add_rounded<OUT>(v, *(const uint4 *)((const char *)gaddend + off));
+                    stream_store16((char *)gout + off, v);
                 }
             }
             __builtin_amdgcn_wave_barrier();
@@ -912,6 +914,42 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
         default: run_epilogue(O1{}, T_{}, T_{}); break;
         }
     }
+}
+
+template <class C, int OUT, bool KTAIL, bool SIDE = false, bool SPLITK = false>
+__global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
+                                                        const float *gxs, const float *gws, const void *gbias, int flags,
+                                                        const GemmArgs g) {
+    gemm_i8_body<C, OUT, KTAIL, SIDE, SPLITK>(gx, gw, gM, gN, gK, tiles_m, tiles_n, gxs, gws, gbias, flags, g, (int)blockIdx.x, g.out,
+                                              g.addend, g.ws_host);
+}
+
+// Several problems of one layer shape (N, K, scale mode, dtypes) with their own activations, weights and outputs in
+// one launch: the tiles of a transformer block's image and text stream for the same projection.  Workgroup b
+// belongs to the group whose range of tiles holds b and works as workgroup b - first_tile of that problem.  Where the
+// small problem's tiles fit into the CUs that the large one's last round leaves idle (192 + 24 tiles of 256 x 256 for
+// 4096 and 512 tokens into 3072 columns), the small problem costs nothing.
+constexpr int MAX_GEMM_GROUPS = 4;
+struct GemmGroups {
+    const int8_t *x[MAX_GEMM_GROUPS], *w[MAX_GEMM_GROUPS];
+    const float *xs[MAX_GEMM_GROUPS], *ws[MAX_GEMM_GROUPS];
+    const void *bias[MAX_GEMM_GROUPS], *addend[MAX_GEMM_GROUPS];
+    void *out[MAX_GEMM_GROUPS];
+    float ws_host[MAX_GEMM_GROUPS];
+    int M[MAX_GEMM_GROUPS], tiles_m[MAX_GEMM_GROUPS];
+    int first_tile[MAX_GEMM_GROUPS + 1];  // [n] = all tiles
+    int n;
+};
+
+template <class C, int OUT>
+__global__ __launch_bounds__(C::NT) void gemm_i8_grouped_kernel(int gN, int gK, int tiles_n, int flags, const GemmGroups gg, const GemmArgs g) {
+    int grp = 0;
+#pragma unroll
+    for (int i = 1; i < MAX_GEMM_GROUPS; ++i)
+        if (i < gg.n && (int)blockIdx.x >= gg.first_tile[i]) grp = i;
+    grp = __builtin_amdgcn_readfirstlane(grp);
+    gemm_i8_body<C, OUT, false>(gg.x[grp], gg.w[grp], gg.M[grp], gN, gK, gg.tiles_m[grp], tiles_n, gg.xs[grp], gg.ws[grp], gg.bias[grp],
+                                flags, g, (int)blockIdx.x - gg.first_tile[grp], gg.out[grp], gg.addend[grp], gg.ws_host[grp]);
 }
 
 // ---- slow but shape-agnostic kernel: one thread per output -----------------------------
@@ -1178,6 +1216,110 @@ int launch(GemmArgs &g, hipStream_t st) {
         g.splitk_tag = splitk_tag(launches.fetch_add(1, std::memory_order_relaxed));
     }
     return launch_tile<OUT>(t, g, st);
+}
+
+template <class C, int OUT>
+int launch_cfg_grouped(const GemmArgs *gs, int n, hipStream_t st) {
+    GemmGroups gg{};
+    gg.n = n;
+    const int tiles_n = (gs[0].N + C::BN - 1) / C::BN;
+    int first = 0;
+    for (int i = 0; i < n; ++i) {
+        gg.x[i] = gs[i].x, gg.w[i] = gs[i].w, gg.xs[i] = gs[i].xs, gg.ws[i] = gs[i].ws, gg.bias[i] = gs[i].bias;
+        gg.addend[i] = gs[i].addend, gg.out[i] = gs[i].out, gg.ws_host[i] = gs[i].ws_host, gg.M[i] = gs[i].M;
+        gg.tiles_m[i] = (gs[i].M + C::BM - 1) / C::BM;
+        gg.first_tile[i] = first;
+        first += gg.tiles_m[i] * tiles_n;
+    }
+    for (int i = n; i <= MAX_GEMM_GROUPS; ++i) gg.first_tile[i] = first;
+    const int flags = (gs[0].row_scale ? 1 : 0) | (gs[0].bias_dtype << 1);
+    hipLaunchKernelGGL((gemm_i8_grouped_kernel<C, OUT>), dim3((unsigned)first), dim3(C::NT), 0, st, gs[0].N, gs[0].K, tiles_n, flags, gg, gs[0]);
+    return check_launch();
+}
+
+// Estimated shader cycles of one launch, for the choice between one launch for a group of problems and one launch per
+// problem; the constants are this kernel's measured figures.  A one-workgroup-per-CU tile costs its rounds over the 256
+// CUs times K-tiles times the time of a K-tile (2 970 cycles for 256 x 256, the others in proportion to their area and
+// their relative cost per operation, as choose_tile prices them); the few-tile configurations cost what their busiest
+// CU fetches at 33 bytes per cycle (with the K split: the model of choose_split); every launch 12 000 cycles of launch,
+// prologue and epilogue.
+constexpr int64_t LAUNCH_CYCLES = 12000;
+inline void tile_shape(Tile t, int *bm, int *bn) {
+    int st = 0;
+    switch (t) {
+    case TILE_BIG: tile_dims<CfgBig>(bm, bn, &st); break;
+    case TILE_B192: tile_dims<CfgB192>(bm, bn, &st); break;
+    case TILE_MID: tile_dims<CfgMid>(bm, bn, &st); break;
+    case TILE_TALL: tile_dims<CfgTall>(bm, bn, &st); break;
+    case TILE_WIDE: tile_dims<CfgWide>(bm, bn, &st); break;
+    case TILE_W96: tile_dims<CfgW96>(bm, bn, &st); break;
+    case TILE_MID_DEEP: tile_dims<CfgMidDeep>(bm, bn, &st); break;
+    case TILE_M96_DEEP: tile_dims<CfgM96Deep>(bm, bn, &st); break;
+    case TILE_S64_DEEP: tile_dims<CfgS64Deep>(bm, bn, &st); break;
+    default: tile_dims<CfgT64Deep>(bm, bn, &st); break;
+    }
+}
+inline int64_t ktile_cycles(Tile t) {  // of one K-tile of one tile, one-workgroup-per-CU configurations
+    int bm, bn;
+    tile_shape(t, &bm, &bn);
+    const int per_op = t == TILE_BIG ? 100 : (t == TILE_B192 ? 108 : 102);
+    return 2970ll * bm * bn * per_op / (256 * 256 * 100);
+}
+inline int64_t launch_cycles(int64_t tiles, Tile t, int64_t K) { return (tiles + 255) / 256 * ((K + 127) / 128) * ktile_cycles(t) + LAUNCH_CYCLES; }
+inline int64_t alone_cycles(int64_t M, int64_t N, int64_t K, bool has_workspace) {
+    Tile t = choose_tile(M, N);
+    int splits = 1;
+    if (has_workspace) choose_split(M, N, K, t, splits);
+    int bm, bn;
+    tile_shape(t, &bm, &bn);
+    const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    if (t == TILE_BIG || t == TILE_B192 || t == TILE_TALL || t == TILE_WIDE) return launch_cycles(tiles, t, K);
+    if (t == TILE_MID) return (tiles + 511) / 512 * 2 * ((K + 127) / 128) * (2970ll * 141 / 400) + LAUNCH_CYCLES;
+    if (splits > 1) return ((K / splits) * (bm + bn) + 7ll * splits * bm * bn) / 33 + LAUNCH_CYCLES;
+    return (tiles + 255) / 256 * K * (bm + bn) / 33 + LAUNCH_CYCLES;
+}
+
+// n problems that share N, K, the scale mode, the dtypes and the operation order (gs[i] differ in M and in their
+// pointers).  One launch with the cheapest of the one-workgroup-per-CU tiles where that is estimated to cost less than
+// one launch per problem (the small problems' tiles run on CUs that the large problem's last round would leave idle);
+// else one launch per problem, as launch() would do it.  The results are the same either way.
+template <int OUT>
+int launch_group(GemmArgs *gs, int n, hipStream_t st) {
+    bool together = n >= 2 && n <= MAX_GEMM_GROUPS;
+    for (int i = 0; i < n && together; ++i) {
+        const GemmArgs &g = gs[i];
+        together = (g.K % 128 == 0) && (g.N % 8 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
+                   ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.N * g.K < (1ll << 31)) && ((int64_t)g.M * g.K < (1ll << 31)) &&
+                   (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) && (!g.bias || (uintptr_t)g.bias % 16 == 0) &&
+                   (!g.addend || (uintptr_t)g.addend % 16 == 0) && !g.side_t;
+    }
+    Tile t = TILE_BIG;
+    if (together) {
+        const int64_t N = gs[0].N, K = gs[0].K;
+        int64_t separate = 0;
+        for (int i = 0; i < n; ++i) separate += alone_cycles(gs[i].M, N, K, gs[i].partials != nullptr);
+        int64_t best = -1;
+        for (Tile c : {TILE_BIG, TILE_B192, TILE_TALL, TILE_WIDE}) {
+            int bm, bn;
+            tile_shape(c, &bm, &bn);
+            int64_t tiles = 0;
+            for (int i = 0; i < n; ++i) tiles += ((gs[i].M + bm - 1) / bm) * ((N + bn - 1) / bn);
+            const int64_t cost = launch_cycles(tiles, c, K);
+            if (best < 0 || cost < best) best = cost, t = c;
+        }
+        together = best < separate;
+    }
+    if (!together) {
+        for (int i = 0; i < n; ++i)
+            if (int rc = launch<OUT>(gs[i], st)) return rc;
+        return I8F_OK;
+    }
+    switch (t) {
+    case TILE_BIG: return launch_cfg_grouped<CfgBig, OUT>(gs, n, st);
+    case TILE_B192: return launch_cfg_grouped<CfgB192, OUT>(gs, n, st);
+    case TILE_TALL: return launch_cfg_grouped<CfgTall, OUT>(gs, n, st);
+    default: return launch_cfg_grouped<CfgWide, OUT>(gs, n, st);
+    }
 }
 
 inline int validate(const int8_t *a, const int8_t *w, int64_t M, int64_t N, int64_t K, const void *out) {

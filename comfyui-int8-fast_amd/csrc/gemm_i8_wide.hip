@@ -5,5 +5,6 @@ namespace i8f {
 namespace gemm {
 template int launch<OUT_I32>(GemmArgs &, hipStream_t);
 template int launch<OUT_F32>(GemmArgs &, hipStream_t);
+template int launch_group<OUT_F32>(GemmArgs *, int, hipStream_t);
 }  // namespace gemm
 }  // namespace i8f

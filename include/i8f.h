@@ -271,6 +271,36 @@ int i8f_linear_w8a8_splitk(const int8_t *a, const float *a_scale, const int8_t *
                            int order, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * i8f_linear_w8a8_splitk for several layers of one shape at once: group i is a problem of its own
+ * (activations, weights, scales, bias, addend, output, row count M) and the groups share N, K, the
+ * scale mode, the dtypes and the operation order.  No counterpart in the reference, whose operator
+ * (int8_forward_dynamic*, int8_quant.py:65-118; Int8TensorwiseOps.Linear.forward, :703-778) takes one
+ * layer: a double-stream transformer block runs every projection twice, for its image and for its
+ * text tokens, and the few tiles of the text stream fit into the compute units that the image
+ * stream's last round of tiles leaves idle (4096 and 512 tokens into 3072 columns: 192 + 24 tiles of
+ * 256 x 256 on 256 units), so in one launch the smaller problem costs nothing.  Where the groups'
+ * tiles together need a round more than the largest group alone, or a group has a shape the tiled
+ * kernel does not take, the call launches group by group exactly as i8f_linear_w8a8_splitk would
+ * (workspace: as there, may be NULL).  Results are those of the separate calls bit for bit.
+ * The array of groups is read on the host during the call; at most I8F_MAX_LINEAR_GROUPS groups.
+ */
+#define I8F_MAX_LINEAR_GROUPS 4
+typedef struct i8f_linear_group {
+    const int8_t *a;        /* [M,K] int8 */
+    const float *a_scale;   /* [M] */
+    const int8_t *w;        /* [N,K] int8 */
+    const float *w_scale;   /* [N] (I8F_SCALE_ROW), [1] or NULL (then w_scale_host) */
+    float w_scale_host;
+    const void *bias;       /* [N] of bias_dtype or NULL */
+    const void *addend;     /* [M,N] of out_dtype or NULL */
+    void *out;              /* [M,N] of out_dtype */
+    int64_t M;
+} i8f_linear_group;
+int i8f_linear_w8a8_grouped(const i8f_linear_group *groups, int n_groups, int scale_mode,
+                            int bias_dtype, int out_dtype, int64_t N, int64_t K, int order,
+                            void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * i8f_linear_w8a8 with the second product of the dynamic (unmerged) LoRA side branch
  * computed inside the epilogue on the matrix cores:
  *   out[m,n] = round( i8f_linear_w8a8(...)[m,n] + side[m,n] )

@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 20
+    assert len(names) == 21
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -95,6 +95,25 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 16, 0, 0.0, one, L.F32, 32, 32, 128, 0, null) == UNSUPPORTED
     assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 24, 0, 0.0, one, L.BF16, 32, 32, 128, 0, null) == UNSUPPORTED
     assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 80, 0, 0.0, one, L.BF16, 32, 32, 128, 0, null) == UNSUPPORTED
+    # grouped linear: no groups, a bad mode or dtype, too many groups, a group without output or without scales
+    lg = (L._LinearGroup * 5)()
+    for g in lg:
+        g.a = g.a_scale = g.w = g.w_scale = g.out = one.value
+        g.M = 4
+    assert lib.i8f_linear_w8a8_grouped(null, 0, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == 0
+    assert lib.i8f_linear_w8a8_grouped(null, 2, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == INVALID
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 5, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == INVALID
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, 9, 8, 16, 0, null, 0, null) == INVALID
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 7, null, 0, null) == INVALID
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 0, one, 64, null) == INVALID      # workspace too small
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 5, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == UNSUPPORTED
+    lg[1].out = None
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == INVALID
+    lg[1].out, lg[1].w_scale = one.value, None
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == INVALID
+    lg[1].M = 0   # an empty group is skipped, whatever its pointers
+    lg[0].M = 0
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == 0
     assert lib.i8f_linear_w8a8(one, null, one, one, 1.0, 0, null, 0, one, L.BF16, 4, 4, 4, 0, null) == INVALID            # activation scales missing
     assert lib.i8f_linear_w8a8_add(one, one, one, one, 1.0, 0, null, 0, one, null, L.BF16, 4, 4, 4, 0, null) == INVALID   # no output
     assert lib.i8f_linear_w8a8_add(one, one, one, one, 1.0, 0, null, 0, one, one, 9, 4, 4, 4, 0, null) == INVALID         # bad output dtype

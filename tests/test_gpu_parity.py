@@ -383,6 +383,69 @@ def test_linear_w8a8_bit_exact(L, dev, M, N, K, row, bdt, odt, order):
         assert np.array_equal(bits(got2), want)
 
 
+GROUPED_CASES = [
+    # row counts of the groups, N, K, per-row scales, bias dtype, output dtype, order, residual addend
+    ((4096, 512), 3072, 384, True, torch.bfloat16, torch.bfloat16, 0, False),    # 192 + 24 tiles of 256 x 256: one launch
+    ((4090, 500, 130), 3064, 256, True, torch.float16, torch.float16, 1, True),  # ragged everywhere, three groups, addends
+    ((4096, 512), 9216, 3072, True, torch.bfloat16, torch.bfloat16, 0, False),   # the small group would cost a round: separate launches
+    ((4096, 512), 2304, 256, False, None, torch.float32, 0, False),              # 192 + 24 tiles of 256 x 192, one scale per group
+    ((4032, 288), 4096, 128, True, torch.bfloat16, torch.bfloat16, 0, True),     # 224 + 16 tiles of 288 x 256
+    ((3584, 250), 4608, 128, True, torch.float16, torch.float16, 0, False),      # 224 + 16 tiles of 256 x 288
+    ((512, 4096, 0, 17), 3072, 128, True, torch.bfloat16, torch.bfloat16, 0, False),  # the large group second, an empty one, a tiny one
+    ((300, 200), 512, 200, True, torch.bfloat16, torch.bfloat16, 0, False),      # K not a multiple of 128: separate launches
+]
+
+
+@pytest.mark.parametrize("Ms,N,K,row,bdt,odt,order,add", GROUPED_CASES)
+def test_linear_w8a8_grouped_equals_separate_calls_and_the_oracle(L, dev, Ms, N, K, row, bdt, odt, order, add):
+    """i8f_linear_w8a8_grouped: several problems of one layer shape, each with its own activations, weights, scales, bias
+    and addend, in one launch where the library groups them and group by group where it does not: every output is
+    the oracle's bit for bit and that of a linear_w8a8 call of its own."""
+    ocode = {torch.bfloat16: O.BF16, torch.float16: O.F16, torch.float32: O.F32}[odt]
+    problems, wants = [], []
+    for M in Ms:
+        x = acts(M, K)
+        wf = torch.randn(N, K, generator=G) * 0.02
+        wq, ws = O.quant_rowwise(wf.numpy(), O.F32) if row else O.quant_tensorwise(wf.numpy(), O.F32)
+        bias = None if bdt is None else (torch.randn(N, generator=G) * 0.01).to(bdt)
+        addend = (torch.randn(M, N, generator=G) * 0.3).to(odt) if add else None
+        q, s = L.quant_rowwise(x.to(dev)) if M else (torch.empty(0, K, dtype=torch.int8, device=dev), torch.empty(0, 1, device=dev))
+        ws_arg = torch.from_numpy(ws).to(dev) if row else float(ws[0])
+        problems.append((q, s, torch.from_numpy(wq).to(dev), ws_arg, None if bias is None else bias.to(dev), None if addend is None else addend.to(dev)))
+        if M:
+            xa, code = O.from_torch(x)
+            ba, bcode = (None, O.BF16) if bias is None else O.from_torch(bias)
+            y = O.linear_w8a8(xa, code, wq, ws, ba, bcode, ocode, 0, order)
+            if add:
+                y = O.from_torch((O.to_torch(y, ocode).float() + addend.float()).to(odt))[0]
+            wants.append(y)
+        else:
+            wants.append(None)
+    got = L.linear_w8a8_grouped(problems, odt, order)
+    assert len(got) == len(Ms)
+    for M, p, g, want in zip(Ms, problems, got, wants):
+        assert tuple(g.shape) == (M, N) and g.dtype == odt
+        if M == 0:
+            continue
+        assert np.array_equal(bits(g), want)
+        alone = L.linear_w8a8(p[0], p[1], p[2], p[3], p[4], odt, order, addend=p[5])
+        assert torch.equal(alone, g)
+
+
+def test_linear_w8a8_grouped_mixed_problems_fall_back_to_separate_launches(L, dev):
+    """Problems that do not share N, the scale mode or the bias dtype are launched one by one by the Python layer."""
+    xa, xb = acts(300, 256), acts(40, 256)
+    qa, sa = L.quant_rowwise(xa.to(dev))
+    qb, sb = L.quant_rowwise(xb.to(dev))
+    wa, wb = i8(512, 256).to(dev), i8(264, 256).to(dev)
+    wsa = (torch.rand(512, generator=G) * 0.002 + 0.0005).to(dev)
+    got = L.linear_w8a8_grouped([(qa, sa, wa, wsa, None), (qb, sb, wb, 0.001, (torch.randn(264, generator=G) * 0.1).to(dev))], torch.bfloat16)
+    assert torch.equal(got[0], L.linear_w8a8(qa, sa, wa, wsa, None, torch.bfloat16))
+    assert tuple(got[1].shape) == (40, 264)
+    with pytest.raises(ValueError):
+        L.linear_w8a8_grouped([(qa, sa, wa, wsa, None), (qb, sb, i8(64, 128).to(dev), 0.001, None)], torch.bfloat16)   # K mismatch
+
+
 SPLITK_CASES = [
     # M, N, K, output dtype: few tiles and a long K, where the tile's K range is dealt over several workgroups
     (512, 3072, 12288, torch.bfloat16),   # 128 x 96 tiles, two slices
