@@ -262,6 +262,20 @@ def extras(L, dev, quick=False):
     t_u = time_kernel(mod_unfused, reps, sets=sets, burst=sets)
     out["modulate_quant_4608x3072"] = {"fused_median_us": round(t_f["median_us"], 2), "torch_ops_then_quant_median_us": round(t_u["median_us"], 2),
                                        "fused_gbs": round(qbytes / t_f["median_us"] / 1e3, 1)}
+
+    # the whole adaLN producer of a DiT block, LayerNorm without affine and the modulation, inside the quantiser
+    def norm_fused(i):
+        rc = lib.i8f_quant_rowwise_norm_modulate(ptr(xs[i]), L.BF16, M, K, K, 1e-6, ptr(sc), ptr(sh), M, 0, ptr(qs[i]), ptr(ss[i]), stream)
+        assert rc == 0, rc
+
+    def norm_unfused(i):
+        plain_call((1 + sc) * F.layer_norm(xs[i], (K,), eps=1e-6) + sh, qs[i], ss[i], K)
+
+    t_f = time_kernel(norm_fused, reps, sets=sets, burst=sets)
+    t_u = time_kernel(norm_unfused, reps, sets=sets, burst=sets)
+    out["norm_modulate_quant_4608x3072"] = {"fused_median_us": round(t_f["median_us"], 2), "torch_ops_then_quant_median_us": round(t_u["median_us"], 2),
+                                            "fused_gbs": round(qbytes / t_f["median_us"] / 1e3, 1),
+                                            "note": "layer_norm (no affine) + (1 + scale) * y + shift + quantise: one launch against torch's four kernels and the quantiser"}
     hs = [torch.randn(M, 12288, device=dev).bfloat16() for _ in range(3)]
     hq = [torch.empty(M, 12288, dtype=torch.int8, device=dev) for _ in range(3)]
 

@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libi8f_gfx950.so")
 BF16, F16, F32 = 0, 1, 2
 SCALE_TENSOR, SCALE_ROW = 0, 1
 EPI_TORCH, EPI_FUSED = 0, 1
-PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE = 0, 1, 2, 3
+PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE = 0, 1, 2, 3, 4
 
 _DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
 
@@ -55,6 +55,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_rotate128.argtypes = [vp, i32, i64, i64, i64, vp, vp]
     L.i8f_quant_rowwise_grouped.argtypes = [vp, i32, i32, i64, i32, vp]
     L.i8f_quant_rowwise_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, i32, vp, vp, vp]
+    L.i8f_quant_rowwise_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, i32, vp, vp, vp]
     L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
     L.i8f_quant_tensorwise_workspace_bytes.restype = i64
     L.i8f_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp, vp, i64, vp]
@@ -72,7 +73,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
+    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -81,7 +82,7 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_rotate128",
-    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue",
+    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate",
     "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
@@ -164,12 +165,20 @@ def _scale(ws, N: int, device):
 
 
 # --------------------------------------------------------------------------- entry points
-def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NONE, mod_scale=None, mod_shift=None):
+def norm_modulate_fusable(x: torch.Tensor) -> bool:
+    """Whether the quantiser takes PRO_NORM_MODULATE for these rows (one wavefront holds a row): 16-bit elements,
+    a width of at most 4096 in multiples of 16, 16-byte aligned rows."""
+    return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and x.dim() == 2 and 0 < x.shape[1] <= 4096 and x.shape[1] % 16 == 0
+            and x.stride(1) == 1 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0)
+
+
+def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NONE, mod_scale=None, mod_shift=None, eps: float = 1e-6):
     """x [M,K] (bf16/fp16/fp32, cuda) -> (int8 [M,K], float32 [M,1]); rotate=True applies the 128-block Hadamard first.
     prologue applies an elementwise operation while the rows are read: PRO_GELU_TANH, or PRO_MODULATE with
     mod_scale / mod_shift of x's dtype, [V,K] (or [K]): (1 + mod_scale) * x + mod_shift, M // V consecutive rows
     to a vector, or PRO_SILU_GATE with the gate operand as mod_scale (x's dtype, [M,K], or [V,K] like the vectors
-    above): silu(x) * mod_scale."""
+    above): silu(x) * mod_scale, or PRO_NORM_MODULATE: the modulation applied to layer_norm(x, eps) without affine
+    parameters (see norm_modulate_fusable for the rows it takes)."""
     _dev(x, "x")
     x = _rows(x, "x")
     M, K = x.shape
@@ -179,7 +188,10 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
     s = torch.empty((M, 1), dtype=torch.float32, device=x.device)
     ldx = x.stride(0) if M > 1 else K
     rows_per_vec = 1
-    if prologue in (PRO_MODULATE, PRO_SILU_GATE):
+    if prologue in (PRO_MODULATE, PRO_SILU_GATE, PRO_NORM_MODULATE):
+        if prologue == PRO_NORM_MODULATE and not norm_modulate_fusable(x):
+            raise ValueError("PRO_NORM_MODULATE takes contiguous 16-bit rows of at most 4096 elements in multiples of 16 "
+                             "(see norm_modulate_fusable); normalise with torch and use PRO_MODULATE")
         vecs = []
         if prologue == PRO_SILU_GATE:
             mod_shift = mod_scale      # one operand: the gate
@@ -201,6 +213,10 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
         if prologue == PRO_NONE:
             _check(lib().i8f_quant_rowwise(_ptr(x), dtype_code(x.dtype), M, K, ldx, 128 if rotate else 0, _ptr(q), _ptr(s),
                                            _stream(x)), "i8f_quant_rowwise")
+        elif prologue == PRO_NORM_MODULATE:
+            _check(lib().i8f_quant_rowwise_norm_modulate(_ptr(x), dtype_code(x.dtype), M, K, ldx, float(eps), _ptr(mod_scale),
+                                                         _ptr(mod_shift), rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s),
+                                                         _stream(x)), "i8f_quant_rowwise_norm_modulate")
         else:
             _check(lib().i8f_quant_rowwise_prologue(_ptr(x), dtype_code(x.dtype), M, K, ldx, prologue, _ptr(mod_scale),
                                                     _ptr(mod_shift), rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s),

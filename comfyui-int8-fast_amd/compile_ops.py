@@ -109,19 +109,19 @@ def _(x, weight, weight_scale, weight_scale_value, bias, rotate):
 @torch.library.custom_op(f"{NAMESPACE}::int8_linear_prologue", mutates_args=())
 def int8_linear_prologue(x: Tensor, prologue: int, mod_scale: Optional[Tensor], mod_shift: Optional[Tensor],
                          weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
-                         bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int) -> Tensor:
+                         bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int, eps: float = 1e-6) -> Tensor:
     """int8_linear on prologue(x): tanh-GELU, (1 + mod_scale) * x + mod_shift with one pair of vectors per
-    group of consecutive rows, or silu(x) * mod_scale with a gate operand of x's shape; the transformed activations
-    exist only inside the quantiser."""
+    group of consecutive rows (PRO_NORM_MODULATE: of layer_norm(x, eps) without affine parameters), or
+    silu(x) * mod_scale with a gate operand of x's shape; the transformed activations exist only inside the quantiser."""
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
-                              mod_shift=mod_shift)
+                              mod_shift=mod_shift, eps=eps)
     y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order)
     return y.reshape(*lead, weight.shape[0])
 
 
 @int8_linear_prologue.register_fake
-def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order):
+def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, eps=1e-6):
     return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
 
 
@@ -194,6 +194,27 @@ def _match_modulate(node):
     return None
 
 
+def _match_plain_layer_norm(node):
+    """layer_norm(h, (K,), eps=...) over the last dimension without weight and bias, used nowhere else, on 16-bit rows
+    of a width the normalising quantiser takes -> (h, eps)."""
+    if not (_is_call(node, torch.nn.functional.layer_norm) and len(node.users) == 1):
+        return None
+    names = ("input", "normalized_shape", "weight", "bias", "eps")
+    a = dict(zip(names, node.args))
+    a.update(node.kwargs)
+    h, shape = a.get("input"), a.get("normalized_shape")
+    if a.get("weight") is not None or a.get("bias") is not None or not isinstance(h, torch.fx.Node):
+        return None
+    v = h.meta.get("example_value", h.meta.get("val"))
+    if v is None or v.dtype not in (torch.bfloat16, torch.float16):
+        return None
+    K = int(v.shape[-1])
+    if tuple(int(d) for d in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,))) != (K,) or K % 16 or K > 4096:
+        return None
+    eps = a.get("eps", 1e-5)
+    return (h, float(eps)) if isinstance(eps, (int, float)) else None
+
+
 def _vectors_broadcast_over_tokens(x, scale, shift) -> bool:
     """True if the traced shapes say scale/shift are [.., 1, K] (or [K]) against x [.., T, K]: one vector per
     leading index, shared by the T rows that become consecutive rows of the flattened activations."""
@@ -219,8 +240,9 @@ def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
 
 
 def fuse_prologues(gm: torch.fx.GraphModule) -> int:
-    """Rewrite int8_linear(gelu_tanh(h)), int8_linear((1 + s) * h + t) and int8_linear(silu(h) * g) (no dynamic-LoRA
-    addend, producer used nowhere else) into int8_linear_prologue(h, ...).  Returns the number of layers rewritten."""
+    """Rewrite int8_linear(gelu_tanh(h)), int8_linear((1 + s) * h + t), int8_linear((1 + s) * layer_norm(h) + t) and
+    int8_linear(silu(h) * g) (no dynamic-LoRA addend, producers used nowhere else) into int8_linear_prologue(h, ...).
+    Returns the number of layers rewritten."""
     n_fused = 0
     targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
     for node in list(gm.graph.nodes):
@@ -237,7 +259,7 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         if x_shape is None:
             continue
         h = _match_gelu(src)
-        new_args = None
+        new_args, eps = None, 1e-6
         if h is not None:
             new_args = (h, _lib.PRO_GELU_TANH, None, None)
         else:
@@ -245,6 +267,9 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
             g = _match_silu_gate(src) if m is None else None
             if m is not None and _vectors_broadcast_over_tokens(*m):
                 new_args = (m[0], _lib.PRO_MODULATE, m[1], m[2])
+                ln = _match_plain_layer_norm(m[0])   # the modulated tensor is a LayerNorm without affine: that goes in too
+                if ln is not None:
+                    new_args, eps = (ln[0], _lib.PRO_NORM_MODULATE, m[1], m[2]), ln[1]
             elif g is not None:
                 new_args = (g[0], _lib.PRO_SILU_GATE, g[1], None)
         if new_args is None:
@@ -259,7 +284,7 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
             continue
         with gm.graph.inserting_before(node):
             fused = gm.graph.call_function(torch.ops.i8f.int8_linear_prologue,
-                                           (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order))
+                                           (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order, eps))
             restored = fused if h_shape == x_shape else gm.graph.call_method("reshape", (fused, -1, _out_features(weight)))
         node.replace_all_uses_with(restored)
         gm.graph.erase_node(node)

@@ -48,9 +48,17 @@ struct Elem {
 //                                                     exp2 and reciprocal (a few binary32 ulp).
 struct Prologue {
     int kind;
-    const void *s, *t;       // modulation vectors (MODULATE)
+    const void *s, *t;       // modulation vectors (MODULATE, NORM_MODULATE), gate operand (SILU_GATE)
     int64_t rows_per_vec;    // rows that share one pair of vectors
+    float eps;               // NORM_MODULATE: added to the row's variance
 };
+
+// the sum over the wave in a fixed order (the same in every lane)
+__device__ __forceinline__ float wave_sum_all(float v) {
+#pragma unroll
+    for (int b = 1; b < 64; b <<= 1) v += __shfl_xor(v, b, 64);
+    return v;
+}
 
 // 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3), written as x / (1 + exp(-2u)): five vector instructions and the
 // hardware's exp2 and reciprocal.  exp(-2u) = exp2(x (c1 + c2 x^2)) with c1 = -2 log2(e) sqrt(2/pi), c2 = 0.044715 c1; an
@@ -70,7 +78,7 @@ template <int DT, int PRO>
 __device__ __forceinline__ float apply_prologue(float x, float s, float t) {
     if constexpr (PRO == I8F_PRO_SILU_GATE) {
         return round_to_dtype<DT>(round_to_dtype<DT>(silu_f32(x)) * s);
-    } else if constexpr (PRO == I8F_PRO_MODULATE) {
+    } else if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_NORM_MODULATE) {
         const float a = round_to_dtype<DT>(1.0f + s);
         const float b = round_to_dtype<DT>(a * x);
         return round_to_dtype<DT>(b + t);
@@ -463,11 +471,41 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
         float v[RUNS][16];
         float amax = 0.0f;
         [[maybe_unused]] int64_t vrow = 0;  // the row's pair of modulation vectors (M < 2^31: a 32-bit division)
-        if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_SILU_GATE) vrow = (uint32_t)(FULL || m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
+        if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_SILU_GATE || PRO == I8F_PRO_NORM_MODULATE)
+            vrow = (uint32_t)(FULL || m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
+        if constexpr (PRO == I8F_PRO_NORM_MODULATE) {
+            // LayerNorm without affine over the row, which this wave holds whole: mean, then the variance of the
+            // differences (two passes over registers), y = (x - mean) / sqrt(var + eps) rounded to the dtype.
+            static_assert(WPR == 1 && SEG == 1, "the row's statistics are taken by the one wave that holds it");
+            float sum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < RUNS; ++r) {
+                expand16<DT>(raw[r][0], raw[r][1], v[r]);   // (runs beyond the row are zeros)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) sum += v[r][j];
+            }
+            const float mean = wave_sum_all(sum) / (float)K;
+            float ss = 0.0f;
+#pragma unroll
+            for (int r = 0; r < RUNS; ++r) {
+                const bool in = FULL || r * TPR + p < nruns;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const float d = v[r][j] - mean;
+                    v[r][j] = d;
+                    ss += in ? d * d : 0.0f;
+                }
+            }
+            const float rstd = 1.0f / sqrtf(wave_sum_all(ss) / (float)K + pro.eps);
+#pragma unroll
+            for (int r = 0; r < RUNS; ++r)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v[r][j] = round_to_dtype<DT>(v[r][j] * rstd);
+        }
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
-            expand16<DT>(raw[r][0], raw[r][1], v[r]);
-            if constexpr (PRO == I8F_PRO_MODULATE) {
+            if constexpr (PRO != I8F_PRO_NORM_MODULATE) expand16<DT>(raw[r][0], raw[r][1], v[r]);
+            if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_NORM_MODULATE) {
                 // the vectors of this row's group, same 16 columns (they come from cache: every row of the group reads them)
                 const int R = r * TPR + p;
                 const int64_t off = (vrow * K + (seg_run + (FULL || R < nruns ? R : 0)) * 16) * 2;
@@ -787,16 +825,19 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
     constexpr int EPC = Elem<DT>::EPC;
     const size_t es = dtype_size(DT);
     bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) && ((uintptr_t)q % 8 == 0);
-    if constexpr (PRO == I8F_PRO_MODULATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0 && (uintptr_t)pro.t % 16 == 0;
+    if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_NORM_MODULATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0 && (uintptr_t)pro.t % 16 == 0;
     if constexpr (PRO == I8F_PRO_SILU_GATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0;
     const int64_t nchunks = K / EPC;
     if constexpr (DT != I8F_F32) {
         const int64_t nruns = K / 16;
         if (aligned && K % 16 == 0 && (uintptr_t)q % 16 == 0 && nruns >= 1 && nruns <= 64 * 4 * 4) {
             if (nruns <= 64 * 4) return pick_runs16<DT, ROT, 1, PRO>((int)((nruns + 63) / 64), x, M, K, ldx, q, scale, st, pro);
-            return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
+            if constexpr (PRO != I8F_PRO_NORM_MODULATE) return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
         }
     }
+    // the normalising prologue exists where one wave holds the row: 16-bit rows of up to 4096 aligned elements
+    if constexpr (PRO == I8F_PRO_NORM_MODULATE) return I8F_ERR_UNSUPPORTED;
+    else {
     if constexpr (PRO == I8F_PRO_NONE) {  // the chunked kernels have no prologue form: such shapes take the generic kernel
         if (aligned && nchunks <= 1024 * 8) {
             if (nchunks <= 64 * 8) return pick_nch<DT, ROT, 64>((int)((nchunks + 63) / 64), x, M, K, ldx, q, scale, st);
@@ -807,6 +848,7 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
     hipLaunchKernelGGL((quant_rows_generic_kernel<DT, ROT, PRO>), dim3((unsigned)M), dim3(256), 0, st, x, M, K, ldx,
                        q, scale, pro);
     return check_launch();
+    }
 }
 
 template <int DT>
@@ -822,6 +864,10 @@ int dispatch_rot(bool rot, const void *x, int64_t M, int64_t K, int64_t ldx, int
     case I8F_PRO_SILU_GATE:
         return rot ? dispatch<DT, true, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro)
                    : dispatch<DT, false, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro);
+    case I8F_PRO_NORM_MODULATE:
+        if constexpr (DT == I8F_F32) return I8F_ERR_UNSUPPORTED;
+        else return rot ? dispatch<DT, true, I8F_PRO_NORM_MODULATE>(x, M, K, ldx, q, scale, st, pro)
+                        : dispatch<DT, false, I8F_PRO_NORM_MODULATE>(x, M, K, ldx, q, scale, st, pro);
     default: return rot ? dispatch<DT, true>(x, M, K, ldx, q, scale, st) : dispatch<DT, false>(x, M, K, ldx, q, scale, st);
     }
 }
@@ -912,13 +958,35 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
     if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
     if (int rc = check_device()) return rc;
     if (rows_per_vec > 0x7fffffff) rows_per_vec = 0x7fffffff;  // M itself is below 2^31
-    Prologue pro{prologue, mod_scale, mod_shift, rows_per_vec > 0 ? rows_per_vec : 1};
+    Prologue pro{prologue, mod_scale, mod_shift, rows_per_vec > 0 ? rows_per_vec : 1, 0.0f};
     hipStream_t st = (hipStream_t)stream;
     const bool rot = rotate_block != 0;
     switch (x_dtype) {
     case I8F_BF16: return dispatch_rot<I8F_BF16>(rot, x, M, K, ldx, q, scale, st, pro);
     case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st, pro);
     default: return dispatch_rot<I8F_F32>(rot, x, M, K, ldx, q, scale, st, pro);
+    }
+}
+
+extern "C" int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, float eps,
+                                               const void *mod_scale, const void *mod_shift, int64_t rows_per_vec, int rotate_block,
+                                               int8_t *q, float *scale, void *stream) {
+    using namespace i8f;
+    if (M < 0 || K < 0 || !valid_dtype(x_dtype) || !(eps >= 0.0f)) return I8F_ERR_INVALID;
+    if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
+    if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
+    if (M == 0) return I8F_OK;
+    if (!scale || ldx < K || K == 0 || !x || !q || rows_per_vec <= 0 || !mod_scale || !mod_shift) return I8F_ERR_INVALID;
+    if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
+    if (int rc = check_device()) return rc;
+    if (rows_per_vec > 0x7fffffff) rows_per_vec = 0x7fffffff;
+    Prologue pro{I8F_PRO_NORM_MODULATE, mod_scale, mod_shift, rows_per_vec, eps};
+    hipStream_t st = (hipStream_t)stream;
+    const bool rot = rotate_block != 0;
+    switch (x_dtype) {
+    case I8F_BF16: return dispatch_rot<I8F_BF16>(rot, x, M, K, ldx, q, scale, st, pro);
+    case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st, pro);
+    default: return I8F_ERR_UNSUPPORTED;
     }
 }
 

@@ -34,8 +34,8 @@ def hip_quantize_rowwise(x: torch.Tensor, rotate: bool = False):
 def _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend=None, prologue=None, side=None):
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
-    kind, mod_scale, mod_shift = prologue or (_lib.PRO_NONE, None, None)
-    q, s = _lib.quant_rowwise(x2, rotate=rotate, prologue=kind, mod_scale=mod_scale, mod_shift=mod_shift)
+    kind, mod_scale, mod_shift, eps = (tuple(prologue) + (1e-6,))[:4] if prologue else (_lib.PRO_NONE, None, None, 1e-6)
+    q, s = _lib.quant_rowwise(x2, rotate=rotate, prologue=kind, mod_scale=mod_scale, mod_shift=mod_shift, eps=eps)
     order = DEFAULT_EPILOGUE if order is None else order
     if side is not None:   # (side_t [M,r], side_b [N,r], alpha or None): the low-rank branch formed inside the epilogue
         y = _lib.linear_w8a8_lora(q, s, weight, weight_scale, bias, side[0], side[1], side[2], compute_dtype, order)
@@ -48,8 +48,8 @@ def hip_int8_linear(x, weight, weight_scale, bias=None, compute_dtype=torch.floa
                     addend=None, prologue=None, side=None):
     """W8A8 linear with ONE weight scale (Python float or 1-element tensor).  `addend`, a tensor of the
     output's shape and dtype, is added to the result inside the epilogue (and the sum rounded again).
-    `prologue` = (kind, mod_scale, mod_shift) applies _lib.PRO_GELU_TANH or _lib.PRO_MODULATE to x inside the
-    quantiser.  `side` = (side_t [M,r], side_b [N,r], alpha or None) adds the low-rank product side_t @ side_b.T,
+    `prologue` = (kind, mod_scale, mod_shift[, eps]) applies _lib.PRO_GELU_TANH, _lib.PRO_MODULATE, _lib.PRO_SILU_GATE or
+    _lib.PRO_NORM_MODULATE to x inside the quantiser.  `side` = (side_t [M,r], side_b [N,r], alpha or None) adds the low-rank product side_t @ side_b.T,
     formed inside the epilogue (see _lib.linear_w8a8_lora), instead of a ready-made addend."""
     if isinstance(weight_scale, torch.Tensor) and weight_scale.numel() != 1:
         # the reference's kernel reads element 0 only (int8_fused_kernel.py:153)

@@ -436,12 +436,13 @@ class Int8TensorwiseOps(manual_cast):
 
         # -- forward ------------------------------------------------------------------------
         def forward(self, x: Tensor, prologue: int = _lib.PRO_NONE, mod_scale: Tensor | None = None,
-                    mod_shift: Tensor | None = None) -> Tensor:
+                    mod_shift: Tensor | None = None, eps: float = 1e-6) -> Tensor:
             """The reference's forward(x) (int8_quant.py:703-778).  The optional arguments name the elementwise
             operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, _lib.PRO_MODULATE with
-            (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension, or _lib.PRO_SILU_GATE with
-            silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8 path
-            then applies inside its quantiser instead of in a pass of its own (under torch.compile the graph
+            (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension, _lib.PRO_NORM_MODULATE with
+            the same modulation of layer_norm(x, eps) (no affine parameters: the whole adaLN producer of a DiT
+            block), or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
+            path then applies inside its quantiser instead of in passes of their own (under torch.compile the graph
             rewrite of compile_ops does this without the caller's help)."""
             managed = self.comfy_cast_weights or len(self.weight_function) > 0 or len(self.bias_function) > 0
             if prologue != _lib.PRO_NONE:
@@ -450,10 +451,14 @@ class Int8TensorwiseOps(manual_cast):
                            and not torch.compiler.is_compiling())
                 if fusable and prologue == _lib.PRO_SILU_GATE:   # the gate operand has x's shape and dtype, or torch does it
                     fusable = isinstance(mod_scale, Tensor) and mod_scale.shape == x.shape and mod_scale.dtype == x.dtype
-                if fusable and prologue == _lib.PRO_MODULATE:
+                if fusable and prologue in (_lib.PRO_MODULATE, _lib.PRO_NORM_MODULATE):
                     # vectors of another dtype or another broadcast pattern are torch's business (as under compile)
                     fusable = (isinstance(mod_scale, Tensor) and isinstance(mod_shift, Tensor) and x.dim() >= 2
                                and compile_ops.modulation_broadcasts_over_tokens(x, mod_scale, mod_shift))
+                if prologue == _lib.PRO_NORM_MODULATE and not (fusable and _lib.norm_modulate_fusable(x.reshape(-1, x.shape[-1]))):
+                    # rows the normalising quantiser does not take: torch normalises, the modulation may still be fused
+                    x = F.layer_norm(x, (x.shape[-1],), eps=eps)
+                    prologue = _lib.PRO_MODULATE
                 if not fusable:   # every other path takes the operation as torch would have applied it
                     if prologue == _lib.PRO_GELU_TANH:
                         x = F.gelu(x, approximate="tanh")
@@ -530,7 +535,7 @@ class Int8TensorwiseOps(manual_cast):
                                                   int8_fused_kernel.DEFAULT_EPILOGUE, addend)
                 else:
                     fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
-                    pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift)
+                    pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift, eps)
                     y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=pro,
                             side=side_factors)
             else:

@@ -79,8 +79,12 @@ typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
  *   I8F_PRO_SILU_GATE  silu(x) * g[k], the gated activation in front of the down projection of a
  *                      SwiGLU feed-forward (w2(silu(w1 x) * w3 x)): silu in binary32 rounded to x's
  *                      dtype, then the product rounded to x's dtype, as torch's two eager kernels do
+ *   I8F_PRO_NORM_MODULATE  (1 + s[k]) * layer_norm(x) + t[k] (no affine parameters); taken by
+ *                      i8f_quant_rowwise_norm_modulate only, which carries the epsilon
  */
-typedef enum i8f_prologue { I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2, I8F_PRO_SILU_GATE = 3 } i8f_prologue;
+typedef enum i8f_prologue {
+    I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2, I8F_PRO_SILU_GATE = 3, I8F_PRO_NORM_MODULATE = 4
+} i8f_prologue;
 
 /* Library version (I8F_VERSION of the build). */
 int i8f_version(void);
@@ -148,6 +152,28 @@ int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K,
                                int prologue, const void *mod_scale, const void *mod_shift,
                                int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale,
                                void *stream);
+
+/*
+ * The quantiser with the whole adaLN producer of a DiT block in front of it:
+ *   y = layer_norm(x, eps) without affine parameters, rounded to x's dtype
+ *       (mean and variance of the row in binary32: mean = sum / K, var = sum (x - mean)^2 / K,
+ *        y = (x - mean) * (1 / sqrt(var + eps)))
+ *   z = (1 + s[k]) * y + t[k], three operations each rounded to x's dtype (I8F_PRO_MODULATE)
+ *   then rotation, absmax and int8 as i8f_quant_rowwise.
+ * No counterpart in the reference's files: there the LayerNorm and the modulation are the model's
+ * own torch operations in front of Linear.forward (int8_quant.py:703), fused by torch.compile into
+ * the quantiser's producer (README.md:4,56); here neither y nor z is ever written to memory.
+ * torch's LayerNorm takes its sums in another order and its reciprocal square root from the
+ * hardware, so y agrees with it to the last place of the dtype (tests state the tolerance).
+ *   mod_scale, mod_shift, rows_per_vec: as for I8F_PRO_MODULATE.
+ * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 4096 and x, q and
+ * the vectors are 16-byte aligned (one wavefront holds a row): other callers normalise with their
+ * own kernel and use I8F_PRO_MODULATE.
+ */
+int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                    float eps, const void *mod_scale, const void *mod_shift,
+                                    int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale,
+                                    void *stream);
 
 /*
  * One absmax scale for a whole tensor, then int8 quantisation with it.

@@ -45,6 +45,7 @@ def lib() -> ctypes.CDLL:
         L.orc_quant_rowwise.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp]
         L.orc_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp]
         L.orc_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, vp]
+        L.orc_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, vp]
         L.orc_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp]
         L.orc_epilogue.argtypes = [vp, vp, vp, i32, vp, i32, vp, i32, i64, i64, i32]
         L.orc_linear_w8a8.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i32, vp, i32, vp, i32, i64, i32]
@@ -166,7 +167,7 @@ def quant_tensorwise(x, dtype_code):
     return q, s
 
 
-PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE = 1, 2, 3
+PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE = 1, 2, 3, 4
 
 
 def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
@@ -183,6 +184,18 @@ def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
     out = np.empty((M, K), dtype=x.dtype)
     _chk(lib().orc_prologue(_p(x), dtype_code, M, K, K, kind, _p(s) if s is not None else None,
                             _p(t) if t is not None else None, rows_per_vec, _p(out)), "prologue")
+    return out
+
+
+def norm_modulate(x, dtype_code, eps, s, t, rows_per_vec=1):
+    """(1 + s) * layer_norm(x, eps) + t without affine parameters, every tensor operation rounded to the dtype as
+    torch's eager kernels do; returns the storage array of dtype_code, shape of x."""
+    x = _arr(x, dtype_code)
+    M, K = x.shape
+    s, t = _arr(s, dtype_code).reshape(-1, K), _arr(t, dtype_code).reshape(-1, K)
+    assert s.shape == t.shape and s.shape[0] * rows_per_vec >= M
+    out = np.empty((M, K), dtype=x.dtype)
+    _chk(lib().orc_norm_modulate(_p(x), dtype_code, M, K, K, float(eps), _p(s), _p(t), rows_per_vec, _p(out)), "norm_modulate")
     return out
 
 

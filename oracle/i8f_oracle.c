@@ -297,6 +297,40 @@ int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, in
 }
 
 /*
+ * LayerNorm without affine parameters followed by the adaLN modulation, the producer of a DiT block's
+ * qkv and MLP inputs (the model's own torch operations in front of Linear.forward, int8_quant.py:703):
+ *   y = round((x - mean) * rstd),  mean = sum x / K,  rstd = 1 / sqrt(sum (x - mean)^2 / K + eps)
+ *   z = round(round(round(1 + s) * y) + t)
+ * The row's sums are taken in double (torch's kernels take them in binary32 in their own order; the
+ * difference is far below a unit in the last place of a 16-bit dtype except at rounding boundaries),
+ * mean and rstd are then binary32 values and the elementwise part runs in binary32 as torch's does.
+ */
+int orc_norm_modulate(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, float eps,
+                      const void *s, const void *t, int64_t rows_per_vec, void *out) {
+    if (M < 0 || K <= 0 || ldx < K || rows_per_vec <= 0 || !s || !t) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        double sum = 0.0, ss = 0.0;
+        for (int64_t k = 0; k < K; ++k) sum += (double)load_as_f32(x, dtype, (size_t)(m * ldx + k));
+        const float mean = (float)(sum / (double)K);
+        for (int64_t k = 0; k < K; ++k) {
+            const double d = (double)(load_as_f32(x, dtype, (size_t)(m * ldx + k)) - mean);
+            ss += d * d;
+        }
+        const float var = (float)(ss / (double)K);
+        const float rstd = 1.0f / sqrtf(var + eps);
+        for (int64_t k = 0; k < K; ++k) {
+            const size_t vi = (size_t)((m / rows_per_vec) * K + k);
+            const float y = round_to_dtype((load_as_f32(x, dtype, (size_t)(m * ldx + k)) - mean) * rstd, dtype);
+            const float a = round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype);
+            const float b = round_to_dtype(a * y, dtype);
+            store_from_f32(out, dtype, (size_t)(m * K + k), b + load_as_f32(t, dtype, vi));
+        }
+    }
+    return 0;
+}
+
+/*
  * quantize_int8_tensorwise (int8_quant.py:23-26): one scale for the whole
  * tensor.  Used to prepare the tensorwise weights of BASELINE config 0.
  */

@@ -202,6 +202,43 @@ def test_graph_rewrite_moves_the_swiglu_gate_into_the_quantiser(pkg):
     assert pkg.compile_ops.fuse_prologues(gm) == 0
 
 
+def test_graph_rewrite_moves_layer_norm_and_modulation_into_the_quantiser(pkg):
+    """(1 + scale) * LayerNorm(h) + shift -> linear, the adaLN producer of a DiT block: LayerNorm without affine goes into
+    the quantiser together with the modulation (with its eps); a LayerNorm with affine parameters, one that is used
+    elsewhere too, or rows wider than a wavefront holds stay torch's and only the modulation is fused."""
+    g = torch.Generator().manual_seed(13)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Block(torch.nn.Module):
+        def __init__(self, k, affine=False, reuse=False):
+            super().__init__()
+            self.norm = torch.nn.LayerNorm(k, elementwise_affine=affine, eps=1e-6).bfloat16()
+            self.qkv, self.reuse = lin(64, k), reuse
+
+        def forward(self, x, scale, shift):
+            h = self.norm(x)
+            y = self.qkv((1 + scale) * h + shift)
+            return y + h.sum() if self.reuse else y
+
+    def fused_nodes(mod, k):
+        x, v = torch.randn(2, 24, k).bfloat16(), torch.randn(2, 1, k).bfloat16()
+        gm = torch._dynamo.export(mod)(x, v, v).graph_module
+        assert pkg.compile_ops.fuse_prologues(gm) == 1
+        nodes = [n for n in gm.graph.nodes if n.op == "call_function" and "int8_linear_prologue" in str(n.target)]
+        assert len(nodes) == 1
+        return nodes[0], any("layer_norm" in str(n.target) for n in gm.graph.nodes if n.op == "call_function")
+
+    node, ln_left = fused_nodes(Block(256), 256)
+    assert node.args[1] == pkg._lib.PRO_NORM_MODULATE and not ln_left and abs(node.args[-1] - 1e-6) < 1e-12
+    for mod, k in ((Block(256, affine=True), 256), (Block(256, reuse=True), 256), (Block(8192), 8192)):
+        node, ln_left = fused_nodes(mod, k)
+        assert node.args[1] == pkg._lib.PRO_MODULATE and ln_left
+
+
 def test_modulation_broadcast_rule(pkg):
     ok = pkg.compile_ops.modulation_broadcasts_over_tokens
     x = torch.empty(2, 24, 256, dtype=torch.bfloat16)

@@ -280,6 +280,10 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
         a = lin(x, prologue=L.PRO_SILU_GATE, mod_scale=gate)
         b = lin(F.silu(x) * gate)
         assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
+        a = lin(x, prologue=L.PRO_NORM_MODULATE, mod_scale=sc, mod_shift=sh, eps=1e-6)   # the whole adaLN producer
+        b = lin((1 + sc) * F.layer_norm(x, (384,), eps=1e-6) + sh)
+        assert a.shape == (2, 20, 96) and (a.float() - b.float()).abs().max() <= 2.0**-6 * b.float().abs().max()
+        assert (a != b).float().mean().item() <= 0.2
     # vectors that torch would broadcast differently, or of another dtype, are left to torch: same result as the
     # unfused expression (a [1, T, K] vector against a batch of 2 must not be dealt over the rows as if it were [2, 1, K])
     lin._use_quarot = False
@@ -289,6 +293,12 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
     assert torch.equal(lin(x, prologue=L.PRO_MODULATE, mod_scale=sc32, mod_shift=sh32), lin((1 + sc32) * x + sh32))
     small = x[:1, :4]                     # four rows: the W8A16 path applies the operation in torch
     assert torch.equal(lin(small, prologue=L.PRO_GELU_TANH), lin(F.gelu(small, approximate="tanh")))
+    assert torch.equal(lin(small, prologue=L.PRO_NORM_MODULATE, mod_scale=sc[:1], mod_shift=sh[:1], eps=1e-5),
+                       lin((1 + sc[:1]) * F.layer_norm(small, (384,), eps=1e-5) + sh[:1]))
+    # rows that the normalising quantiser does not take (binary32 here): torch normalises, and the result is that of
+    # the unfused expression
+    x32, sc_, sh_ = x.float(), sc.float(), sh.float()
+    assert torch.equal(lin(x32, prologue=L.PRO_NORM_MODULATE, mod_scale=sc_, mod_shift=sh_), lin((1 + sc_) * F.layer_norm(x32, (384,), eps=1e-6) + sh_))
 
 
 @pytest.mark.parametrize("quarot", [False, True])

@@ -178,6 +178,45 @@ def test_quant_rowwise_silu_gate_prologue_within_tolerance(L, dev, M, K, dt, rot
         assert torch.equal(qa, qb) and torch.equal(sa, sb)
 
 
+@pytest.mark.parametrize("M,K,dt,rot,V,eps", [
+    (64, 3072, torch.bfloat16, False, 1, 1e-6), (48, 3072, torch.bfloat16, True, 2, 1e-6), (33, 4096, torch.float16, False, 3, 1e-5),
+    (10, 1008, torch.bfloat16, False, 2, 1e-6), (6, 384, torch.float16, True, 1, 1e-5), (5, 16, torch.bfloat16, False, 1, 1e-6),
+    (4608, 3072, torch.bfloat16, False, 1, 1e-6),
+])
+def test_quant_rowwise_norm_modulate_prologue_within_tolerance(L, dev, M, K, dt, rot, V, eps):
+    """LayerNorm (no affine) and the adaLN modulation inside the quantiser (i8f_quant_rowwise_norm_modulate) against the
+    oracle (row sums in double) and against torch's layer_norm and three eager operations on the device followed by
+    the plain quantiser.  The kernel takes the row's sums in binary32 in its own order, so a normalised value may land
+    on the other side of a rounding boundary of the dtype: scales within 2 ulp of the dtype, int8 at most 1 apart, at
+    least 99.5 % equal (98 % with rotation, which spreads every such step over 128 values)."""
+    rows = M - M % V
+    x = (acts(rows, K, dt).float() * 3 + 0.25).to(dt)
+    s = (torch.randn(V, K, generator=G) * 0.3).to(dt)
+    t = (torch.randn(V, K, generator=G) * 0.2).to(dt)
+    xa, code = O.from_torch(x)
+    z = O.norm_modulate(xa, code, eps, O.from_torch(s)[0], O.from_torch(t)[0], rows_per_vec=rows // V)
+    qo, so = O.quant_rowwise(z, code, 128 if rot else 0)
+    q, sc = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_NORM_MODULATE, mod_scale=s.to(dev), mod_shift=t.to(dev), eps=eps)
+    xd = x.to(dev).reshape(V, rows // V, K)
+    zt = ((1 + s.to(dev)[:, None]) * torch.nn.functional.layer_norm(xd, (K,), eps=eps) + t.to(dev)[:, None]).reshape(rows, K)
+    q2, s2 = L.quant_rowwise(zt, rotate=rot)
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[dt]
+    for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+        d = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() <= (2e-2 if rot else 5e-3)
+        assert (np.abs(sc.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
+    again = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_NORM_MODULATE, mod_scale=s.to(dev), mod_shift=t.to(dev), eps=eps)
+    assert torch.equal(again[0], q) and torch.equal(again[1], sc)     # fixed order of the sums: launches agree bit for bit
+
+
+def test_quant_rowwise_norm_modulate_refuses_rows_it_does_not_take(L, dev):
+    s = torch.zeros(1, 8192, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError):
+        L.quant_rowwise(torch.zeros(4, 8192, dtype=torch.bfloat16, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s, mod_shift=s)
+    with pytest.raises(ValueError):
+        L.quant_rowwise(torch.zeros(4, 256, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s[:, :256].float(), mod_shift=s[:, :256].float())
+
+
 TENSORWISE_CASES = [
     # shape, dtype
     ((3072, 3072), torch.bfloat16), ((3072, 3072), torch.float32), ((1, 1), torch.float32), ((7,), torch.float16),

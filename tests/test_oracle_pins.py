@@ -528,3 +528,39 @@ def test_prologue_silu_gate_agrees_with_torch(dt):
     got3 = O.prologue(O.from_torch(a3)[0], O.from_torch(a3)[1], O.PRO_SILU_GATE, O.from_torch(b3)[0], rows_per_vec=3)
     want3 = O.prologue(O.from_torch(a3)[0], O.from_torch(a3)[1], O.PRO_SILU_GATE, O.from_torch(b3.repeat_interleave(3, 0))[0], rows_per_vec=1)
     assert np.array_equal(got3, want3)
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_norm_modulate_agrees_with_torch(dt):
+    """(1 + s) * layer_norm(x) + t as torch's eager kernels compute it on 16-bit tensors (LayerNorm without affine in
+    binary32 with its own order of the sums, then three rounded tensor operations).  The oracle takes the row's sums
+    in double, so the normalised value may differ from torch's by one unit in the last place of the dtype at rounding
+    boundaries; that unit is carried through the modulation.  Also pinned: the closed form on a row whose statistics
+    are exact (values +-1: mean 0, variance 1) and the row-group layout of the vectors."""
+    g = torch.Generator().manual_seed(41)
+    M, K, eps = 48, 768, 1e-6
+    x = (torch.randn(M, K, generator=g) * 2 + 0.3).to(dt)
+    x[:, 5] *= 30                                             # an outlier channel, as adaLN inputs have
+    s = (torch.randn(1, K, generator=g) * 0.3).to(dt)
+    t = (torch.randn(1, K, generator=g) * 0.2).to(dt)
+    want = (1 + s) * torch.nn.functional.layer_norm(x, (K,), eps=eps) + t
+    code = O.from_torch(x)[1]
+    got = O.to_f32(O.norm_modulate(O.from_torch(x)[0], code, eps, O.from_torch(s)[0], O.from_torch(t)[0], rows_per_vec=M), code)
+    w = want.float().numpy()
+    ulp = {torch.bfloat16: 2.0**-7, torch.float16: 2.0**-10}[dt]
+    y = torch.nn.functional.layer_norm(x.float(), (K,), eps=eps).numpy()
+    # one unit of the normalised value times the gain, plus the roundings of the product and of the sum
+    bound = ulp * (np.abs(y) * np.abs(1 + s.float().numpy()) + np.abs(w)) + 1e-30
+    assert (np.abs(got - w) <= bound).all()
+    assert (got != w).mean() < 2e-2
+    # exact statistics: +-1 in equal numbers has mean 0 and variance 1, so y = x / sqrt(1 + eps), which rounds to x
+    pm = torch.ones(4, 256)
+    pm[:, ::2] = -1
+    sv, tv = (torch.randn(2, 256, generator=g) * 0.5).to(dt), torch.randn(2, 256, generator=g).to(dt)
+    got2 = O.to_torch(O.norm_modulate(O.from_torch(pm.to(dt))[0], code, 1e-6, O.from_torch(sv)[0], O.from_torch(tv)[0], rows_per_vec=2), code)
+    want2 = ((1 + sv).repeat_interleave(2, 0) * pm.to(dt)) + tv.repeat_interleave(2, 0)
+    assert torch.equal(got2.view(torch.int16), want2.view(torch.int16))
+    # a constant row: variance 0, y = 0 exactly, the result is the shift
+    const = torch.full((1, 64), 3.25).to(dt)
+    got3 = O.to_torch(O.norm_modulate(O.from_torch(const)[0], code, 1e-5, O.from_torch(sv[:1, :64].contiguous())[0], O.from_torch(tv[:1, :64].contiguous())[0]), code)
+    assert torch.equal(got3.view(torch.int16), tv[:1, :64].contiguous().view(torch.int16))
