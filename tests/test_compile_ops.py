@@ -313,6 +313,48 @@ def test_compiled_mlp_with_fused_prologues_equals_the_oracle(pkg, dev, O):
 
 
 @pytest.mark.gpu
+def test_compiled_adaln_block_with_the_layer_norm_in_the_quantiser(pkg, dev, O):
+    """LayerNorm (no affine) -> modulation -> quantised projection compiled with the rewriting backend over inductor:
+    one fused operator, no LayerNorm kernel left, and the output agrees with the oracle's chain (row sums in double)
+    to the rounding of the normalised values: within two bf16 ulps of the output scale, at least 90 % identical."""
+    g = torch.Generator().manual_seed(8)
+    lin = pkg.Int8TensorwiseOps.Linear(512, 192, bias=True)
+    _load(lin, {"weight": torch.randint(-127, 128, (192, 512), dtype=torch.int8, generator=g),
+                "weight_scale": torch.rand(192, 1, generator=g) * 0.002 + 1e-3, "bias": torch.randn(192, generator=g).bfloat16()})
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm, self.qkv = torch.nn.LayerNorm(512, elementwise_affine=False, eps=1e-6), lin
+
+        def forward(self, x, scale, shift):
+            return self.qkv((1 + scale) * self.norm(x) + shift)
+
+    m = Block().to(dev)
+    x = (torch.randn(2, 40, 512, generator=g) * 2 + 0.5).bfloat16()
+    sc, sh = (torch.randn(2, 1, 512, generator=g) * 0.3).bfloat16(), torch.randn(2, 1, 512, generator=g).bfloat16()
+    seen = []
+
+    def counting(gm, inputs):
+        seen.append((sum("int8_linear_prologue" in str(n.target) for n in gm.graph.nodes),
+                     sum("layer_norm" in str(n.target) for n in gm.graph.nodes)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x.to(dev), sc.to(dev), sh.to(dev))
+    assert seen == [(1, 0)]
+    xa, code = O.from_torch(x.reshape(80, 512))
+    z = O.norm_modulate(xa, code, 1e-6, O.from_torch(sc.reshape(2, 512))[0], O.from_torch(sh.reshape(2, 512))[0], rows_per_vec=40)
+    want = O.to_f32(O.linear_w8a8(z, code, lin.weight.cpu().numpy(), lin.weight_scale.cpu().numpy().reshape(-1),
+                                  O.from_torch(lin.bias.cpu())[0], O.BF16, O.BF16, 0), O.BF16).reshape(2, 40, 192)
+    diff = np.abs(got.float().cpu().numpy() - want)
+    assert diff.max() <= 2.0**-7 * np.abs(want).max()
+    assert (diff != 0).mean() < 0.1
+    eager = m(x.to(dev), sc.to(dev), sh.to(dev))       # torch's LayerNorm and modulation, then the layer
+    assert (got.float() - eager.float()).abs().max().item() <= 2.0**-7 * eager.float().abs().max().item()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("rows", [48, 8])
 @pytest.mark.parametrize("scalar_scale", [False, True])
 def test_compiled_forward_equals_eager(pkg, dev, rows, scalar_scale):
