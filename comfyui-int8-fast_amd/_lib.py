@@ -123,7 +123,14 @@ def _ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor):
+    """torch's current stream on t's device as the void * the library takes (the raw handle: building a
+    torch.cuda.Stream object for it costs several microseconds per call)."""
+    if _raw_stream is not None and t.device.index is not None:
+        return ctypes.c_void_p(_raw_stream(t.device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
