@@ -77,15 +77,88 @@ def make_config(i: int, rows: int | None = None) -> dict:
     raise ValueError(i)
 
 
-# HBM-side bytes per GEMM launch come from profiles/gemm_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# figures per shape and tile configuration, with the commands that produced them and the calibration of the
-# counters against a plain copy.  They are a property of (shape, tile configuration), not of this run: a row is
-# used only while the library still picks the tile configuration it was measured with.
+# HBM-side bytes per GEMM launch: measured by this run where rocprofv3 is at hand (live_traffic: two child runs of
+# this file under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`, started before this process touches the GPU, each
+# calibrated on a device copy of known size in the same run), else taken from profiles/gemm_hbm_traffic.txt, the
+# figures of the same procedure per shape and tile configuration (used only while the library still picks the tile
+# configuration a row was measured with).
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_hbm_traffic.txt")
+TRAFFIC_SHAPES = ((4608, 3072, 3072), (4608, 12288, 3072), (4608, 3072, 12288))
+TRAFFIC_LAUNCHES = 6
+TRAFFIC_COPY_BYTES = 20 * 1024 * 1024
+
+
+def traffic_probe(L, dev):
+    """What a child run under rocprofv3 --pmc executes: five device copies of TRAFFIC_COPY_BYTES (the calibration), then
+    TRAFFIC_LAUNCHES launches of the GEMM for each of TRAFFIC_SHAPES in that order, nothing else from this library's
+    GEMM kernel."""
+    src = torch.randint(0, 255, (TRAFFIC_COPY_BYTES,), dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(5):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    g = torch.Generator().manual_seed(5)
+    for (M, N, K) in TRAFFIC_SHAPES:
+        q, s = L.quant_rowwise(_acts(g, M, K, 0.01, 20.0).to(dev))
+        wq, ws = L.quant_rowwise(torch.randn(N, K, device=dev) * 0.02)
+        b = (torch.randn(N, device=dev) * 0.01).bfloat16()
+        y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        torch.cuda.synchronize()
+        for _ in range(TRAFFIC_LAUNCHES):
+            L.linear_w8a8(q, s, wq, ws, b, torch.bfloat16, L.EPI_TORCH, y)
+        torch.cuda.synchronize()
+        del q, s, wq, ws, y
+
+
+def live_traffic():
+    """-> ({(M, N, K): HBM-side bytes per launch}, {"fetch_factor", "write_factor"}, None) measured now, or
+    (None, None, reason).  Must run before this process initialises the GPU (it starts child processes)."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+
+    exe = shutil.which("rocprofv3")
+    if exe is None:
+        return None, None, "rocprofv3 not found"
+    kib = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        out = tempfile.mkdtemp(prefix="i8f_pmc_", dir="/tmp")
+        cmd = [exe, "--pmc", counter, "--output-format", "csv", "-d", out, "-o", "t", "--", sys.executable,
+               os.path.abspath(__file__), "--traffic-probe"]
+        try:
+            p = subprocess.run(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, timeout=180, capture_output=True, text=True)
+        except (subprocess.TimeoutExpired, OSError) as e:
+            shutil.rmtree(out, ignore_errors=True)
+            return None, None, f"rocprofv3 --pmc {counter}: {type(e).__name__}"
+        files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
+        if p.returncode != 0 or not files:
+            shutil.rmtree(out, ignore_errors=True)
+            return None, None, f"rocprofv3 --pmc {counter} failed (exit {p.returncode})"
+        rows = [r for r in csv.DictReader(open(files[0])) if r.get("Counter_Name") == counter]
+        shutil.rmtree(out, ignore_errors=True)
+        rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+        copies = [float(r["Counter_Value"]) for r in rows if "copyBuffer" in r["Kernel_Name"]]
+        gemms = [float(r["Counter_Value"]) for r in rows if "gemm_i8_kernel" in r["Kernel_Name"]]
+        if len(copies) < 3 or len(gemms) != TRAFFIC_LAUNCHES * len(TRAFFIC_SHAPES) or statistics.median(copies) <= 0:
+            return None, None, f"rocprofv3 --pmc {counter}: {len(copies)} copy and {len(gemms)} GEMM dispatches in the trace, not what the probe launches"
+        kib[counter] = (TRAFFIC_COPY_BYTES / 1024 / statistics.median(copies[1:]),
+                        [statistics.median(gemms[i * TRAFFIC_LAUNCHES + 1:(i + 1) * TRAFFIC_LAUNCHES]) for i in range(len(TRAFFIC_SHAPES))])
+    f_fetch, f_write = kib["FETCH_SIZE"][0], kib["WRITE_SIZE"][0]
+    traffic = {shape: int((kib["FETCH_SIZE"][1][i] * f_fetch + kib["WRITE_SIZE"][1][i] * f_write) * 1024)
+               for i, shape in enumerate(TRAFFIC_SHAPES)}
+    return traffic, {"fetch_factor": round(f_fetch, 3), "write_factor": round(f_write, 3)}, None
+
+
+LIVE_TRAFFIC = None   # filled by main() before the GPU is touched
 
 
 def gemm_traffic(L, M, N, K):
-    """HBM-side bytes of one M x N x K GEMM launch from the profile, or None (with the reason)."""
+    """HBM-side bytes of one M x N x K GEMM launch: this run's own measurement, else the profile's, else None (with
+    the reason)."""
+    if LIVE_TRAFFIC is not None and (M, N, K) in LIVE_TRAFFIC:
+        return LIVE_TRAFFIC[(M, N, K)], None
     tile = L.gemm_tile(M, N, K)
     try:
         lines = open(TRAFFIC_FILE).read().splitlines()
@@ -570,12 +643,26 @@ def main():
                          "print its timing and exit")
     ap.add_argument("--quant-only", choices=("rot", "plain"),
                     help="profiling aid: launch nothing but the per-row quantiser at 4608x3072 bf16, with or without rotation")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="what the traffic measurement runs under rocprofv3 --pmc: a few device copies and GEMM launches, no output")
+    ap.add_argument("--no-live-traffic", action="store_true",
+                    help="take the HBM-side bytes of the GEMM launches from profiles/gemm_hbm_traffic.txt instead of measuring them "
+                         "in two child runs under rocprofv3 --pmc")
     ap.add_argument("--zero-operands", action="store_true",
                     help="diagnostic: all-zero activations and weights (same instructions, no switching in the multipliers), "
                          "to show what the power limit costs; the line says data = zeros and is not a benchmark result")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: the INT8 linear path has no multi-GPU part (run with --gpus 1)")
+
+    # The counters need child processes: they run first, while this process has not touched the GPU yet.
+    global LIVE_TRAFFIC
+    traffic_source, live_note = "profiles/gemm_hbm_traffic.txt", None
+    if not (a.traffic_probe or a.target_only or a.quant_only or a.no_live_traffic):
+        LIVE_TRAFFIC, calibration, live_note = live_traffic()
+        if LIVE_TRAFFIC is not None:
+            traffic_source = (f"this run: two child runs under rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), calibrated on a device copy "
+                              f"of {TRAFFIC_COPY_BYTES} bytes (fetch x {calibration['fetch_factor']}, write x {calibration['write_factor']})")
 
     import __graft_entry__ as ge
 
@@ -585,6 +672,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if a.traffic_probe:
+        traffic_probe(L, dev)
+        return
     if a.target_only:
         print(json.dumps(target_only(L, dev, a.target_only, a.steps, a.warmup)))
         return
@@ -648,8 +738,8 @@ def main():
         "pct_of_int8_peak": round(100 * value / PEAK_INT8_TOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": traffic,
-                     "traffic_unit": "bytes per launch beyond L2, mean of the two GEMM launches of the step, from "
-                                     "profiles/gemm_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a copy)",
+                     "traffic_unit": "bytes per launch beyond L2, mean of the two GEMM launches of the step",
+                     "traffic_source": traffic_source,
                      "algorithmic_bytes": alg_bytes,
                      "traffic_over_algorithmic": None if traffic is None else round(traffic / alg_bytes, 2),
                      "kernel": "gemm_i8_kernel (int8 MFMA GEMM + dequant epilogue)",
@@ -660,6 +750,8 @@ def main():
     }
     if traffic_note:
         line["roofline"]["traffic_note"] = traffic_note
+    if live_note:
+        line["roofline"]["live_traffic_note"] = "not measured in this run (" + live_note + "): figures of the same procedure from the profile"
     extra = extras(L, dev, quick=a.quick) if not a.no_extras else None   # before the CPU leg: the GPU is still warm
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
@@ -679,7 +771,7 @@ def main():
                                    "cold_operands_frac": tg["cold_operands_frac_of_int8_peak"],
                                    "warm_operands_avg_launch_us": tg["median_us"], "warm_operands_frac": tg["frac_of_int8_peak"],
                                    "vendor_int_mm_warm_us": tg.get("vendor_int_mm_median_us"),
-                                   "traffic": t_traffic, "algorithmic_bytes": t_alg,
+                                   "traffic": t_traffic, "traffic_source": traffic_source, "algorithmic_bytes": t_alg,
                                    "traffic_over_algorithmic": None if t_traffic is None else round(t_traffic / t_alg, 2)}
         if t_note:
             line["roofline_target"]["traffic_note"] = t_note
