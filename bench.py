@@ -119,6 +119,10 @@ def live_traffic():
     import subprocess
     import tempfile
 
+    # Under a profiler this process has the GPU initialised before main() runs (the profiler's preloaded library does
+    # that), and a process in that state must not start other programs: the figures then come from the profile file.
+    if "rocprof" in os.environ.get("LD_PRELOAD", "").lower() or any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ):
+        return None, None, "this run is itself under a profiler"
     exe = shutil.which("rocprofv3")
     if exe is None:
         return None, None, "rocprofv3 not found"
