@@ -551,11 +551,27 @@ def extras(L, dev, quick=False):
     t_sep = time_kernel(block_separate, max(10, iters // 4))
     t_qg = time_kernel(block_quant_grouped, max(10, iters // 4))
     t = time_kernel(block, max(10, iters // 4))
+    # the same block captured in a HIP graph (what torch.compile's reduce-overhead mode replays): no host between launches
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            block(0)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            block(0)
+        graph_ms = round(time_kernel(lambda i: graph.replay(), max(10, iters // 4))["median_us"] / 1e3, 4)
+        del graph
+    except Exception as e:   # the figure is an extra: a capture problem must not cost the benchmark line
+        graph_ms = f"not measured: {type(e).__name__}: {e}"[:200]
     ops = sum(2 * m * n * k for m in (4096, 512) for (n, k) in [c3["linears"][x] for x in ("qkv", "proj", "up", "down")])
     out["dit_block_linears"] = {"ms": round(t["median_us"] / 1e3, 4), "gemm_gop": round(ops / 1e9, 1),
                                 "tops": round(ops / t["median_us"] / 1e6, 1),
                                 "ms_one_launch_per_layer_and_kernel": round(t_sep["median_us"] / 1e3, 4),
                                 "ms_grouped_quantiser_only": round(t_qg["median_us"] / 1e3, 4),
+                                "ms_replayed_from_a_hip_graph": graph_ms,
                                 "note": "8 W8A8 linears and 2 adaLN W8A16 linears at M=1, separate weights for the image (4096 tokens) "
                                         "and the text stream (512 tokens), 340 MB in all; per projection one quantiser launch for both "
                                         "streams and, for the two projections into 3072 columns, one GEMM launch for both (192 + 24 "
