@@ -594,7 +594,8 @@ struct GroupedArgs {
     int n;
 };
 
-template <int DT, bool ROT, int WPR, int RUNS>
+// FULL: every group's rows fill its workgroups and K fills every lane's runs (no bounds tests, no zero fill)
+template <int DT, bool ROT, int WPR, int RUNS, bool FULL>
 __global__ __launch_bounds__(256) void quant16_grouped_kernel(const GroupedArgs g, int64_t K) {
     int grp = 0;
 #pragma unroll
@@ -602,13 +603,19 @@ __global__ __launch_bounds__(256) void quant16_grouped_kernel(const GroupedArgs 
         if (i < g.n && (int)blockIdx.x >= g.first_block[i]) grp = i;
     grp = __builtin_amdgcn_readfirstlane(grp);
     const Prologue none{};
-    quant16_body<DT, ROT, WPR, RUNS, false, I8F_PRO_NONE, 1>(g.x[grp], g.M[grp], K, g.ldx_bytes[grp], g.q[grp], g.scale[grp], none,
+    quant16_body<DT, ROT, WPR, RUNS, FULL, I8F_PRO_NONE, 1>(g.x[grp], g.M[grp], K, g.ldx_bytes[grp], g.q[grp], g.scale[grp], none,
                                                             (int64_t)((int)blockIdx.x - g.first_block[grp]) * (256 / (64 * WPR)));
 }
 
 template <int DT, bool ROT, int WPR, int RUNS>
 int launch16_grouped(const GroupedArgs &g, int64_t K, hipStream_t st) {
-    hipLaunchKernelGGL((quant16_grouped_kernel<DT, ROT, WPR, RUNS>), dim3((unsigned)g.first_block[g.n]), dim3(256), 0, st, g, K);
+    constexpr int ROWS = 256 / (64 * WPR);
+    bool full = K == (int64_t)RUNS * 64 * WPR * 16;
+    for (int i = 0; i < g.n; ++i) full = full && g.M[i] % ROWS == 0;
+    if (full)
+        hipLaunchKernelGGL((quant16_grouped_kernel<DT, ROT, WPR, RUNS, true>), dim3((unsigned)g.first_block[g.n]), dim3(256), 0, st, g, K);
+    else
+        hipLaunchKernelGGL((quant16_grouped_kernel<DT, ROT, WPR, RUNS, false>), dim3((unsigned)g.first_block[g.n]), dim3(256), 0, st, g, K);
     return check_launch();
 }
 

@@ -110,6 +110,13 @@ def test_quant_rowwise_grouped_equals_separate_calls_and_the_oracle(L, dev, rot,
         assert torch.equal(q1, q) and torch.equal(s1, s)
     with pytest.raises(ValueError):
         L.quant_rowwise_grouped([dev_xs[0], dev_xs[0][:, : K // 2]])
+    # groups whose rows fill their workgroups (and, for the model widths, whose K fills every lane): the instantiation
+    # without bounds tests
+    full = [acts(M, K, dt) for M in (128, 64, 4)]
+    for x, (q, s) in zip(full, L.quant_rowwise_grouped([x.to(dev) for x in full], rotate=rot)):
+        xa, code = O.from_torch(x)
+        qo, so = O.quant_rowwise(xa, code, 128 if rot else 0)
+        assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
 
 
 PROLOGUE_CASES = [
