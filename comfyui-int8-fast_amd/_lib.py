@@ -67,13 +67,14 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a8_add.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a8_splitk.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i32, i64, i64, i64, i32, vp, i64, vp]
     L.i8f_linear_w8a8_grouped.argtypes = [vp, i32, i32, i32, i32, i64, i64, i32, vp, i64, vp]
+    L.i8f_linear_w8a8_gated.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, i64, vp, vp, i32, i64, i64, i64, i32, vp, i64, vp]
     L.i8f_linear_w8a8_workspace_bytes.argtypes = []
     L.i8f_linear_w8a8_workspace_bytes.restype = i64
     L.i8f_linear_w8a8_lora.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i64, i32, f32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
+    for name in ("i8f_linear_w8a8_gated", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -83,7 +84,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate",
-    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_gated", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
 
@@ -372,9 +373,11 @@ def clear_splitk_workspaces() -> None:
     _SPLITK_WORKSPACES.clear()
 
 
-def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None, addend=None):
+def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, order=EPI_TORCH, out=None, addend=None, gate=None):
     """Quantised activations (a int8 [M,K], a_scale [M,1]) times int8 weight [N,K] with the fused dequant epilogue.
-    addend ([M,N] of the output dtype) is added to the rounded result in the epilogue and the sum rounded again."""
+    addend ([M,N] of the output dtype) is added to the rounded result in the epilogue and the sum rounded again.
+    gate ([V,N] or [N] of the output dtype, M // V consecutive rows to a vector) multiplies the rounded result first
+    (rounded again): out = addend + gate * y, the gated residual of an adaLN-Zero block."""
     a, w = _i8_matrix(a, "a"), _i8_matrix(w, "w")
     M, K = a.shape
     N, K2 = w.shape
@@ -399,12 +402,22 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
         if addend.numel() != M * N or addend.dtype != out.dtype:
             raise ValueError(f"addend must have {M * N} elements of {out.dtype}")
         addend = addend.reshape(M, N).contiguous()
+    rows_per_gate = 1
+    if gate is not None:
+        _dev(gate, "gate")
+        if gate.dtype != out.dtype or gate.device != a.device or gate.numel() % max(N, 1) or gate.shape[-1] != N:
+            raise ValueError(f"gate must be [V,{N}] of {out.dtype} on {a.device}")
+        gate = gate.reshape(-1, N).contiguous()
+        V = gate.shape[0]
+        if V == 0 or M % V:
+            raise ValueError(f"{M} rows do not split evenly over {V} gate vectors")
+        rows_per_gate = max(1, M // V)
     with _on(a.device):
         work = _splitk_workspace(a, M, N, K)
-        _check(lib().i8f_linear_w8a8_splitk(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode,
-                                            _ptr(addend), _ptr(out), dtype_code(out.dtype), M, N, K, order, _ptr(work),
-                                            0 if work is None else work.numel(), _stream(a)),
-               "i8f_linear_w8a8_splitk")
+        _check(lib().i8f_linear_w8a8_gated(_ptr(a), _ptr(a_scale), _ptr(w), _ptr(ws), ws_host, mode, _ptr(bias), bcode, _ptr(gate),
+                                           rows_per_gate, _ptr(addend), _ptr(out), dtype_code(out.dtype), M, N, K, order, _ptr(work),
+                                           0 if work is None else work.numel(), _stream(a)),
+               "i8f_linear_w8a8_gated")
     return out
 
 

@@ -40,8 +40,18 @@ extern "C" int i8f_linear_w8a8_splitk(const int8_t *a, const float *a_scale, con
                                       float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
                                       const void *addend, void *out, int out_dtype, int64_t M, int64_t N, int64_t K,
                                       int order, void *workspace, int64_t workspace_bytes, void *stream) {
+    return i8f_linear_w8a8_gated(a, a_scale, w, w_scale, w_scale_host, scale_mode, bias, bias_dtype, nullptr, 1, addend, out, out_dtype,
+                                 M, N, K, order, workspace, workspace_bytes, stream);
+}
+
+extern "C" int i8f_linear_w8a8_gated(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                                     float w_scale_host, int scale_mode, const void *bias, int bias_dtype, const void *gate,
+                                     int64_t rows_per_gate, const void *residual, void *out, int out_dtype, int64_t M, int64_t N,
+                                     int64_t K, int order, void *workspace, int64_t workspace_bytes, void *stream) {
     using namespace i8f;
     using namespace i8f::gemm;
+    const void *addend = residual;
+    if (gate && rows_per_gate <= 0) return I8F_ERR_INVALID;
     if (workspace && (workspace_bytes < SPLITK_WORKSPACE_BYTES || (uintptr_t)workspace % 16)) return I8F_ERR_INVALID;
     if (int rc = validate(a, w, M, N, K, out)) return rc;
     if (!valid_dtype(out_dtype) || (bias && !valid_dtype(bias_dtype))) return I8F_ERR_INVALID;
@@ -55,6 +65,7 @@ extern "C" int i8f_linear_w8a8_splitk(const int8_t *a, const float *a_scale, con
     g.x = a, g.w = w, g.M = (int)M, g.N = (int)N, g.K = (int)K, g.out = out;
     g.xs = a_scale, g.ws = w_scale, g.ws_host = w_scale_host, g.row_scale = scale_mode == I8F_SCALE_ROW;
     g.bias = bias, g.bias_dtype = bias_dtype, g.order = order, g.addend = addend;
+    g.gate = gate, g.gate_rows = (int)(rows_per_gate < 0x7fffffff ? rows_per_gate : 0x7fffffff);  // (M itself is below 2^31)
     if (workspace) g.arrivals = (unsigned *)workspace, g.partials = (int *)((char *)workspace + SPLITK_COUNTER_BYTES);
     hipStream_t st = (hipStream_t)stream;
     switch (out_dtype) {

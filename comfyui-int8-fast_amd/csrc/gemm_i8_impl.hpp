@@ -79,6 +79,11 @@ struct GemmArgs {
     int bias_dtype;
     int order;
     const void *addend;  // nullptr or [M,N] of the output dtype, added to the rounded result
+    // nullptr or [ceil(M / gate_rows), N] of the output dtype: the rounded result (side branch included) is multiplied by
+    // gate[m / gate_rows, n] and rounded before the addend is added (the gated residual of an adaLN-Zero block,
+    // x + gate * linear(h), as torch's two tensor operations compute it)
+    const void *gate;
+    int gate_rows;
     // low-rank side branch, side[m,n] = sum_j side_t[m,j] * side_b[n,j] (operands of the output dtype, rank % 16 == 0),
     // rounded to that dtype, times side_alpha if side_has_alpha (rounded again), added to the rounded result
     const void *side_t, *side_b;
@@ -231,6 +236,36 @@ __device__ __forceinline__ uint4 add_rounded(uint4 y, uint4 s) {
             } else {
                 const float lo = f16_bits_to_f32(yv[e] & 0xffffu) + f16_bits_to_f32(sv[e] & 0xffffu);
                 const float hi = f16_bits_to_f32(yv[e] >> 16) + f16_bits_to_f32(sv[e] >> 16);
+                o[e] = f32x2_to_f16x2_bits(lo, hi);
+            }
+        }
+        return make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// Eight (or four) outputs of one 16-byte piece times the gate's, each product rounded to the output dtype: what
+// `gate * y` computes on tensors of that dtype.
+template <int OUT>
+__device__ __forceinline__ uint4 mul_rounded(uint4 y, uint4 s) {
+    if constexpr (OUT == OUT_F32) {
+        return make_uint4(__float_as_uint(__uint_as_float(y.x) * __uint_as_float(s.x)),
+                          __float_as_uint(__uint_as_float(y.y) * __uint_as_float(s.y)),
+                          __float_as_uint(__uint_as_float(y.z) * __uint_as_float(s.z)),
+                          __float_as_uint(__uint_as_float(y.w) * __uint_as_float(s.w)));
+    } else if constexpr (OUT == OUT_I32) {
+        return y;
+    } else {
+        const uint32_t yv[4] = {y.x, y.y, y.z, y.w}, sv[4] = {s.x, s.y, s.z, s.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (OUT == OUT_BF16) {
+                const float lo = bf16_bits_to_f32(yv[e] & 0xffffu) * bf16_bits_to_f32(sv[e] & 0xffffu);
+                const float hi = bf16_bits_to_f32(yv[e] >> 16) * bf16_bits_to_f32(sv[e] >> 16);
+                o[e] = f32x2_to_bf16x2_bits(lo, hi);
+            } else {
+                const float lo = f16_bits_to_f32(yv[e] & 0xffffu) * f16_bits_to_f32(sv[e] & 0xffffu);
+                const float hi = f16_bits_to_f32(yv[e] >> 16) * f16_bits_to_f32(sv[e] >> 16);
                 o[e] = f32x2_to_f16x2_bits(lo, hi);
             }
         }
@@ -893,6 +928,8 @@ __device__ __forceinline__ void gemm_i8_body(const int8_t *gx, const int8_t *gw,
                 {
                     const int64_t off = ((int64_t)mm * gN + nn) * OB;
                     uint4 v = val;
+                    if (g.gate)
+                        v = mul_rounded<OUT>(v, *(const uint4 *)((const char *)g.gate + ((int64_t)((uint32_t)mm / (uint32_t)g.gate_rows) * gN + nn) * OB));
                     if (gaddend) v = add_rounded<OUT>(v, *(const uint4 *)((const char *)gaddend + off));
                     stream_store16((char *)gout + off, v);
                 }
@@ -991,6 +1028,7 @@ __global__ __launch_bounds__(256) void gemm_i8_generic_kernel(const GemmArgs g) 
             t = a * sc;
             if (g.bias) t = t + b;
         }
+        if (g.gate) t = round_to_dtype<DT>(t) * load_as_f32<DT>(g.gate, (int64_t)(m / g.gate_rows) * g.N + n);
         if (g.addend) t = round_to_dtype<DT>(t) + load_as_f32<DT>(g.addend, idx);
         store_from_f32<DT>(g.out, idx, t);
     }
@@ -1184,7 +1222,8 @@ int launch(GemmArgs &g, hipStream_t st) {
     const bool aligned = (g.K % 16 == 0) && (g.N % 8 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
                          ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.N * g.K < (1ll << 31)) &&
                          (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) &&
-                         (!g.bias || (uintptr_t)g.bias % 16 == 0) && (!g.addend || (uintptr_t)g.addend % 16 == 0);
+                         (!g.bias || (uintptr_t)g.bias % 16 == 0) && (!g.addend || (uintptr_t)g.addend % 16 == 0) &&
+                         (!g.gate || (uintptr_t)g.gate % 16 == 0);
     // The buffer descriptors address 2^31 bytes: more activations than that go in row blocks.
     if (aligned && (int64_t)g.M * g.K >= (1ll << 31) && (int64_t)256 * g.K < (1ll << 31)) {
         const int rows_per = (int)((((1ll << 31) - 1) / g.K) / 256 * 256);
@@ -1195,6 +1234,10 @@ int launch(GemmArgs &g, hipStream_t st) {
             if (g.xs) sub.xs = g.xs + m0;
             sub.out = (char *)g.out + m0 * g.N * ob;
             if (g.addend) sub.addend = (const char *)g.addend + m0 * g.N * ob;
+            if (g.gate) {  // the row blocks must start on a gate boundary for the sub-problem to index its vectors from 0
+                if (m0 % g.gate_rows) return I8F_ERR_UNSUPPORTED;
+                sub.gate = (const char *)g.gate + (m0 / g.gate_rows) * g.N * ob;
+            }
             if (g.side_t) sub.side_t = (const char *)g.side_t + m0 * g.side_rank * 2;
             if (int rc = launch<OUT>(sub, st)) return rc;
         }
@@ -1291,7 +1334,7 @@ int launch_group(GemmArgs *gs, int n, hipStream_t st) {
         together = (g.K % 128 == 0) && (g.N % 8 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
                    ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.N * g.K < (1ll << 31)) && ((int64_t)g.M * g.K < (1ll << 31)) &&
                    (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) && (!g.bias || (uintptr_t)g.bias % 16 == 0) &&
-                   (!g.addend || (uintptr_t)g.addend % 16 == 0) && !g.side_t;
+                   (!g.addend || (uintptr_t)g.addend % 16 == 0) && !g.side_t && !g.gate;
     }
     Tile t = TILE_BIG;
     if (together) {

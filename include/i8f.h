@@ -297,6 +297,24 @@ int i8f_linear_w8a8_splitk(const int8_t *a, const float *a_scale, const int8_t *
                            int order, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * i8f_linear_w8a8_splitk with the gated residual of an adaLN-Zero transformer block in the epilogue:
+ *   out[m,n] = round( residual[m,n] + round( gate[m / rows_per_gate, n] * y[m,n] ) ),   y = i8f_linear_w8a8(...)
+ * i.e. `x + gate * linear(h)` as torch's two tensor operations compute it on tensors of out_dtype (each rounded
+ * to out_dtype), bit for bit.  No counterpart in the reference's files: there the multiplication by the gate and
+ * the residual addition are the model's own torch operations behind Linear.forward (int8_quant.py:703-778), two
+ * more passes over [M,N] that torch.compile fuses into one; here neither exists.
+ *   gate       [ceil(M / rows_per_gate), N] of out_dtype, contiguous: one vector per group of rows_per_gate
+ *              consecutive rows (one per image of a batch); NULL: no gate (i8f_linear_w8a8_splitk exactly)
+ *   residual   [M,N] of out_dtype, contiguous, or NULL (then out = round(gate * y)); may equal out
+ * Other arguments and the workspace as for i8f_linear_w8a8_splitk.
+ */
+int i8f_linear_w8a8_gated(const int8_t *a, const float *a_scale, const int8_t *w, const float *w_scale,
+                          float w_scale_host, int scale_mode, const void *bias, int bias_dtype,
+                          const void *gate, int64_t rows_per_gate, const void *residual, void *out,
+                          int out_dtype, int64_t M, int64_t N, int64_t K, int order, void *workspace,
+                          int64_t workspace_bytes, void *stream);
+
+/*
  * i8f_linear_w8a8_splitk for several layers of one shape at once: group i is a problem of its own
  * (activations, weights, scales, bias, addend, output, row count M) and the groups share N, K, the
  * scale mode, the dtypes and the operation order.  No counterpart in the reference, whose operator

@@ -49,6 +49,7 @@ def lib() -> ctypes.CDLL:
         L.orc_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp]
         L.orc_epilogue.argtypes = [vp, vp, vp, i32, vp, i32, vp, i32, i64, i64, i32]
         L.orc_linear_w8a8.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i32, vp, i32, vp, i32, i64, i32]
+        L.orc_gate_residual.argtypes = [vp, i32, i64, i64, vp, i64, vp, vp]
         L.orc_linear_w8a16.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i64]
         L.orc_sr_delta.argtypes = [vp, vp, i32, vp, i64, i64, vp]
         L.orc_merge_i8.argtypes = [vp, vp, i64, vp]
@@ -270,6 +271,22 @@ def linear_w8a8(x, x_dtype, w, ws, bias=None, bias_dtype=BF16, out_dtype=BF16, r
     out = np.empty((M, N), dtype=_NP_OF[out_dtype])
     _chk(lib().orc_linear_w8a8(_p(x), x_dtype, M, K, K, rotate_block, _p(w), _p(ws), mode, _p(bias), bias_dtype,
                                _p(out), out_dtype, N, order), "linear_w8a8")
+    return out
+
+
+def gate_residual(y, dtype_code, gate=None, residual=None, rows_per_gate=1):
+    """residual + gate * y as two tensor operations of one dtype (arrays as from_torch gives them; gate [V,N] with
+    rows_per_gate consecutive rows of y to a vector); returns the storage array of dtype_code."""
+    y = _arr(y, dtype_code)
+    M, N = y.shape
+    if gate is not None:
+        gate = _arr(gate, dtype_code).reshape(-1, N)
+        assert gate.shape[0] * rows_per_gate >= M
+    if residual is not None:
+        residual = _arr(residual, dtype_code).reshape(M, N)
+    out = np.empty((M, N), dtype=y.dtype)
+    _chk(lib().orc_gate_residual(_p(y), dtype_code, M, N, _p(gate) if gate is not None else None, rows_per_gate,
+                                 _p(residual) if residual is not None else None, _p(out)), "gate_residual")
     return out
 
 

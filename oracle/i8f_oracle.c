@@ -476,6 +476,27 @@ int orc_linear_w8a8(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ld
     return rc;
 }
 
+/*
+ * The gated residual behind a linear layer of an adaLN-Zero block, x + gate * y, as torch's two tensor
+ * operations compute it on tensors of one dtype (the model's own operations behind Linear.forward,
+ * int8_quant.py:703-778):  out = round(residual + round(gate[m / rows_per_gate, n] * y[m, n])).
+ * y, gate, residual and out are stored in `dtype`; gate or residual may be NULL (that operation is left out).
+ */
+int orc_gate_residual(const void *y, int dtype, int64_t M, int64_t N, const void *gate, int64_t rows_per_gate,
+                      const void *residual, void *out) {
+    if (M < 0 || N < 0 || (gate && rows_per_gate <= 0)) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        for (int64_t n = 0; n < N; ++n) {
+            float t = load_as_f32(y, dtype, (size_t)(m * N + n));
+            if (gate) t = round_to_dtype(t * load_as_f32(gate, dtype, (size_t)((m / rows_per_gate) * N + n)), dtype);
+            if (residual) t = t + load_as_f32(residual, dtype, (size_t)(m * N + n));
+            store_from_f32(out, dtype, (size_t)(m * N + n), t);
+        }
+    }
+    return 0;
+}
+
 /* ------------------------------------------------------------------------- */
 /* a8: small-M (M <= 16) W8A16 path                                          */
 /* ------------------------------------------------------------------------- */

@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 22
+    assert len(names) == 23
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -102,6 +102,10 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 200, 200, 1e-6, one, one, 4, 128, one, one, null) == INVALID
     assert lib.i8f_quant_rowwise_norm_modulate(null, L.BF16, 0, 256, 256, 1e-6, null, null, 1, 0, null, null, null) == 0
     assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, L.PRO_NORM_MODULATE, one, one, 4, 0, one, one, null) == INVALID  # needs its own entry point: it carries eps
+    # gated residual: a gate needs a positive row count per vector
+    assert lib.i8f_linear_w8a8_gated(one, one, one, one, 1.0, 1, null, 0, one, 0, one, one, L.BF16, 4, 8, 16, 0, null, 0, null) == INVALID
+    assert lib.i8f_linear_w8a8_gated(one, one, one, one, 1.0, 1, null, 0, one, 4, one, null, L.BF16, 4, 8, 16, 0, null, 0, null) == INVALID
+    assert lib.i8f_linear_w8a8_gated(null, null, null, null, 1.0, 1, null, 0, null, 1, null, null, L.BF16, 0, 8, 16, 0, null, 0, null) == 0
     # grouped linear: no groups, a bad mode or dtype, too many groups, a group without output or without scales
     lg = (L._LinearGroup * 5)()
     for g in lg:

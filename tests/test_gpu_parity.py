@@ -429,6 +429,49 @@ def test_linear_w8a8_bit_exact(L, dev, M, N, K, row, bdt, odt, order):
         assert np.array_equal(bits(got2), want)
 
 
+GATED_CASES = [
+    # M, N, K, per-row scales, output dtype, gate vectors, residual: the gated residual x + gate * linear(h) in the epilogue
+    (4608, 3072, 256, True, torch.bfloat16, 1, True), (4096, 3072, 384, True, torch.bfloat16, 2, True),      # 256-wide tiles
+    (4600, 12288, 128, True, torch.float16, 1, True), (1000, 264, 384, False, torch.bfloat16, 4, True),      # 288 x 256; ragged
+    (512, 3072, 12288, True, torch.bfloat16, 2, True),                                                       # few tiles, K split
+    (300, 512, 256, True, torch.float32, 3, True), (130, 96, 128, True, torch.bfloat16, 1, False),           # binary32; gate alone
+    (257, 3076, 640, True, torch.float16, 1, True),                                                          # N % 8 != 0: the one-thread-per-output kernel
+]
+
+
+@pytest.mark.parametrize("M,N,K,row,odt,V,with_res", GATED_CASES)
+def test_linear_w8a8_gated_residual_bit_exact(L, dev, M, N, K, row, odt, V, with_res):
+    """out = residual + gate * linear(h) with both elementwise operations inside the GEMM epilogue (i8f_linear_w8a8_gated):
+    bit-equal to the oracle's linear followed by its restatement of torch's two tensor operations, and to the same two
+    torch operations on the device applied to this library's own linear output; also in place (out = residual)."""
+    M -= M % V
+    x = acts(M, K)
+    wf = torch.randn(N, K, generator=G) * 0.02
+    wq, ws = O.quant_rowwise(wf.numpy(), O.F32) if row else O.quant_tensorwise(wf.numpy(), O.F32)
+    bias = (torch.randn(N, generator=G) * 0.01).to(torch.bfloat16)
+    gate = torch.randn(V, N, generator=G).to(odt)
+    res = (torch.randn(M, N, generator=G) * 0.5).to(odt) if with_res else None
+    ocode = {torch.bfloat16: O.BF16, torch.float16: O.F16, torch.float32: O.F32}[odt]
+    xa, code = O.from_torch(x)
+    y = O.linear_w8a8(xa, code, wq, ws, O.from_torch(bias)[0], O.BF16, ocode, 0, 0)
+    want = O.gate_residual(y, ocode, gate=O.from_torch(gate)[0], residual=None if res is None else O.from_torch(res)[0], rows_per_gate=M // V)
+    q, s = L.quant_rowwise(x.to(dev))
+    ws_arg = torch.from_numpy(ws).to(dev) if row else float(ws[0])
+    wd, bd, gd = torch.from_numpy(wq).to(dev), bias.to(dev), gate.to(dev)
+    rd = None if res is None else res.to(dev)
+    got = L.linear_w8a8(q, s, wd, ws_arg, bd, odt, L.EPI_TORCH, addend=rd, gate=gd)
+    assert np.array_equal(bits(got), want)
+    plain = L.linear_w8a8(q, s, wd, ws_arg, bd, odt, L.EPI_TORCH)
+    torch_way = gd.repeat_interleave(M // V, 0) * plain
+    if rd is not None:
+        torch_way = rd + torch_way
+    assert torch.equal(torch_way, got)
+    if rd is not None:                                  # the residual stream updated in place
+        buf = rd.clone()
+        L.linear_w8a8(q, s, wd, ws_arg, bd, odt, L.EPI_TORCH, out=buf, addend=buf, gate=gd)
+        assert torch.equal(buf, got)
+
+
 GROUPED_CASES = [
     # row counts of the groups, N, K, per-row scales, bias dtype, output dtype, order, residual addend
     ((4096, 512), 3072, 384, True, torch.bfloat16, torch.bfloat16, 0, False),    # 192 + 24 tiles of 256 x 256: one launch

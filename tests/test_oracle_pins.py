@@ -564,3 +564,19 @@ def test_norm_modulate_agrees_with_torch(dt):
     const = torch.full((1, 64), 3.25).to(dt)
     got3 = O.to_torch(O.norm_modulate(O.from_torch(const)[0], code, 1e-5, O.from_torch(sv[:1, :64].contiguous())[0], O.from_torch(tv[:1, :64].contiguous())[0]), code)
     assert torch.equal(got3.view(torch.int16), tv[:1, :64].contiguous().view(torch.int16))
+
+
+@pytest.mark.parametrize("tdt", [torch.bfloat16, torch.float16, torch.float32])
+def test_gate_residual_equals_torch_ops(tdt):
+    """x + gate * y on tensors of one dtype: two elementwise torch operations, each rounded to the dtype; with the gate
+    one vector per group of rows (one per image of a batch), with the gate alone and with the residual alone."""
+    g = torch.Generator().manual_seed(51)
+    y = (torch.randn(3, 8, 96, generator=g) * 3).to(tdt)
+    gate = torch.randn(3, 1, 96, generator=g).to(tdt)
+    res = (torch.randn(3, 8, 96, generator=g) * 2).to(tdt)
+    code = O.from_torch(y)[1]
+    ya, ga, ra = O.from_torch(y.reshape(24, 96))[0], O.from_torch(gate.reshape(3, 96))[0], O.from_torch(res.reshape(24, 96))[0]
+    for want, kw in ((res + gate * y, dict(gate=ga, residual=ra, rows_per_gate=8)), (gate * y, dict(gate=ga, rows_per_gate=8)),
+                     (res + y, dict(residual=ra))):
+        got = O.gate_residual(ya, code, **kw)
+        assert np.array_equal(got, O.from_torch(want.reshape(24, 96))[0])
