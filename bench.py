@@ -475,6 +475,33 @@ def extras(L, dev, quick=False):
                                                "note": "both include the first product x @ A.T in torch (9.5 us of GPU time); the side operands of a tile are staged in LDS and every tile configuration has the side form (here 288x256)"}
     del xu, wqu, yu
 
+    # the residual update of an adaLN-Zero block behind config 1's down-projection, x + gate * linear(h): both elementwise
+    # operations inside the GEMM epilogue against the plain layer followed by torch's two kernels
+    Mg, Ng, Kg = 4608, 3072, 12288
+    hq, hs_ = L.quant_rowwise(_acts(g, Mg, Kg, 0.01, 20.0).to(dev))
+    wqg, wsg = L.quant_rowwise(torch.randn(Ng, Kg, device=dev) * 0.02)
+    bg = (torch.randn(Ng, device=dev) * 0.01).bfloat16()
+    gate_v = torch.randn(1, Ng, device=dev).bfloat16()
+    res = torch.randn(Mg, Ng, device=dev).bfloat16()
+    og = torch.empty(Mg, Ng, dtype=torch.bfloat16, device=dev)
+
+    def gated_fused(_i):
+        L.linear_w8a8(hq, hs_, wqg, wsg, bg, torch.bfloat16, L.EPI_TORCH, og, addend=res, gate=gate_v)
+
+    def gated_unfused(_i):
+        y = L.linear_w8a8(hq, hs_, wqg, wsg, bg, torch.bfloat16, L.EPI_TORCH, og)
+        return res + gate_v * y
+
+    t_gf = time_kernel(gated_fused, max(10, iters // 4))
+    t_gu = time_kernel(gated_unfused, max(10, iters // 4))
+    t_gp = time_kernel(lambda i: L.linear_w8a8(hq, hs_, wqg, wsg, bg, torch.bfloat16, L.EPI_TORCH, og), max(10, iters // 4))
+    out["gated_residual_4608x3072x12288"] = {"gemm_alone_median_us": round(t_gp["median_us"], 2),
+                                             "gate_and_residual_in_epilogue_median_us": round(t_gf["median_us"], 2),
+                                             "gemm_then_torch_mul_and_add_median_us": round(t_gu["median_us"], 2),
+                                             "note": "x + gate * linear(h) with bf16 tensors: the fused form reads the residual (28 MB) inside the "
+                                                     "GEMM; torch's two kernels move 142 MB"}
+    del hq, wqg, res, og
+
     # config 2: QuaRot layer (width 3840, 2 % of the channels x50): time of the rotated path and what the
     # rotation buys in accuracy against the bf16 product
     c2 = make_config(2)

@@ -76,18 +76,19 @@ def _(a, a_scale, weight, weight_scale, weight_scale_value, bias, out_dtype, ord
 @torch.library.custom_op(f"{NAMESPACE}::int8_linear", mutates_args=())
 def int8_linear(x: Tensor, weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
                 bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int,
-                addend: Optional[Tensor] = None) -> Tensor:
+                addend: Optional[Tensor] = None, gate: Optional[Tensor] = None) -> Tensor:
     """Quantise the activations per token (rotated first when `rotate`) and run the W8A8 linear;
-    `addend` (shape and dtype of the result) is added inside the epilogue."""
+    `addend` (as many elements as the result, its dtype) is added inside the epilogue, after `gate` (vectors of the
+    result's width, one per group of consecutive rows) has multiplied the result: addend + gate * y."""
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate)
     y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order,
-                         addend=addend)
+                         addend=addend, gate=gate)
     return y.reshape(*lead, weight.shape[0])
 
 
 @int8_linear.register_fake
-def _(x, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, addend=None):
+def _(x, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, addend=None, gate=None):
     return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
 
 
@@ -109,19 +110,21 @@ def _(x, weight, weight_scale, weight_scale_value, bias, rotate):
 @torch.library.custom_op(f"{NAMESPACE}::int8_linear_prologue", mutates_args=())
 def int8_linear_prologue(x: Tensor, prologue: int, mod_scale: Optional[Tensor], mod_shift: Optional[Tensor],
                          weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
-                         bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int, eps: float = 1e-6) -> Tensor:
+                         bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int, eps: float = 1e-6,
+                         addend: Optional[Tensor] = None, gate: Optional[Tensor] = None) -> Tensor:
     """int8_linear on prologue(x): tanh-GELU, (1 + mod_scale) * x + mod_shift with one pair of vectors per
     group of consecutive rows (PRO_NORM_MODULATE: of layer_norm(x, eps) without affine parameters), or
     silu(x) * mod_scale with a gate operand of x's shape; the transformed activations exist only inside the quantiser."""
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
                               mod_shift=mod_shift, eps=eps)
-    y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order)
+    y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order, addend=addend, gate=gate)
     return y.reshape(*lead, weight.shape[0])
 
 
 @int8_linear_prologue.register_fake
-def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, eps=1e-6):
+def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, eps=1e-6,
+      addend=None, gate=None):
     return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
 
 
@@ -136,9 +139,23 @@ def _is_call(node, *targets):
     return node.op == "call_function" and node.target in targets
 
 
+_OWN_META = "i8f_shape_and_dtype"   # what the rewrites record for the nodes they create (a meta-device tensor)
+
+
+def _meta_val(node):
+    if not isinstance(node, torch.fx.Node):
+        return None
+    return node.meta.get("example_value", node.meta.get("val", node.meta.get(_OWN_META)))
+
+
 def _meta_shape(node):
-    v = node.meta.get("example_value", node.meta.get("val")) if isinstance(node, torch.fx.Node) else None
+    v = _meta_val(node)
     return None if v is None else tuple(v.shape)
+
+
+def _record(node, shape, dtype):
+    node.meta[_OWN_META] = torch.empty(tuple(int(d) for d in shape), dtype=dtype, device="meta")
+    return node
 
 
 def _through_views(node):
@@ -285,9 +302,96 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         with gm.graph.inserting_before(node):
             fused = gm.graph.call_function(torch.ops.i8f.int8_linear_prologue,
                                            (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order, eps))
-            restored = fused if h_shape == x_shape else gm.graph.call_method("reshape", (fused, -1, _out_features(weight)))
+            n_out, old = _out_features(weight), _meta_val(node)
+            if old is not None:   # shapes for the passes that follow (the epilogue rewrite reads them)
+                _record(fused, (*h_shape[:-1], n_out), old.dtype)
+            restored = fused
+            if h_shape != x_shape:
+                restored = gm.graph.call_method("reshape", (fused, -1, n_out))
+                if old is not None:
+                    _record(restored, old.shape, old.dtype)
         node.replace_all_uses_with(restored)
         gm.graph.erase_node(node)
+        n_fused += 1
+    if n_fused:
+        gm.graph.eliminate_dead_code()
+        gm.graph.lint()
+        gm.recompile()
+    return n_fused
+
+
+def _sole_user(node):
+    return next(iter(node.users)) if len(node.users) == 1 else None
+
+
+def fuse_epilogues(gm: torch.fx.GraphModule) -> int:
+    """Rewrite res + gate * int8_linear(...) -- the gated residual behind the projections of an adaLN-Zero block, gate
+    one vector per leading index broadcast over the tokens, res of the result's shape, all of the compute dtype, in any
+    operand order, with shape-only steps between the layer and the multiplication -- into the layer's own epilogue
+    (addend=res, gate=gate); also gate * linear(...) and res + linear(...) alone.  Layers that already carry an addend
+    (a dynamic-LoRA side tensor) are left alone.  Returns the number of layers rewritten."""
+    n_fused = 0
+    lin_targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default,
+                   torch.ops.i8f.int8_linear_prologue, torch.ops.i8f.int8_linear_prologue.default)
+    for node in list(gm.graph.nodes):
+        if not _is_call(node, *lin_targets):
+            continue
+        n_pos = 12 if "prologue" in str(node.target) else 8      # arguments in front of addend, gate
+        given = list(node.args[n_pos:]) + [None, None]
+        if given[0] is not None or given[1] is not None or node.kwargs.get("addend") is not None or node.kwargs.get("gate") is not None:
+            continue
+        y_val = _meta_val(node)
+        if y_val is None:
+            continue
+        cur = node                                 # forward through shape-only steps that keep the feature dimension
+        while True:
+            u = _sole_user(cur)
+            if u is None or not ((u.op == "call_method" and u.target in _VIEW_METHODS) or _is_call(u, torch.reshape, torch.flatten)):
+                break
+            if u.args[0] is not cur or not _meta_shape(u) or _meta_shape(u)[-1] != y_val.shape[-1]:
+                break
+            cur = u
+        u = _sole_user(cur)
+        if u is None:
+            continue
+        cur_val = _meta_val(cur)
+        gate = res = None
+        last = None
+
+        def other(n, operand):
+            return n.args[1] if n.args[0] is operand else n.args[0]
+
+        if _is_call(u, operator.mul, torch.mul) and len(u.args) == 2:
+            g_node = other(u, cur)
+            g_val = _meta_val(g_node)
+            if g_val is None or cur_val is None or not modulation_broadcasts_over_tokens(cur_val, g_val, g_val):
+                continue
+            gate, last = g_node, u
+            a = _sole_user(u)
+            if a is not None and _is_call(a, operator.add, torch.add) and len(a.args) == 2 and not a.kwargs:
+                r_node = other(a, u)
+                r_val = _meta_val(r_node)
+                if r_val is not None and tuple(r_val.shape) == tuple(_meta_shape(u)) and r_val.dtype == cur_val.dtype and r_node is not u:
+                    res, last = r_node, a
+        elif _is_call(u, operator.add, torch.add) and len(u.args) == 2 and not u.kwargs:
+            r_node = other(u, cur)
+            r_val = _meta_val(r_node)
+            if r_val is None or cur_val is None or tuple(r_val.shape) != tuple(cur_val.shape) or r_val.dtype != cur_val.dtype or r_node is cur:
+                continue
+            res, last = r_node, u
+        else:
+            continue
+        final_shape = _meta_shape(last)
+        if final_shape is None or final_shape[-1] != y_val.shape[-1]:
+            continue
+        with gm.graph.inserting_before(last):
+            kwargs = dict(node.kwargs)
+            kwargs.update(addend=res, gate=gate)
+            fused = _record(gm.graph.call_function(node.target, tuple(node.args[:n_pos]), kwargs), y_val.shape, y_val.dtype)
+            restored = fused
+            if tuple(final_shape) != tuple(y_val.shape):
+                restored = _record(gm.graph.call_method("reshape", (fused, *final_shape)), final_shape, y_val.dtype)
+        last.replace_all_uses_with(restored)
         n_fused += 1
     if n_fused:
         gm.graph.eliminate_dead_code()
@@ -304,9 +408,10 @@ def _out_features(weight_node):
 
 
 def backend(inner="inductor"):
-    """A torch.compile backend: fuse_prologues, then `inner` (a registered backend name or a callable)."""
+    """A torch.compile backend: fuse_prologues and fuse_epilogues, then `inner` (a registered backend name or a callable)."""
     def compile_fn(gm, example_inputs):
         fuse_prologues(gm)
+        fuse_epilogues(gm)
         fn = inner
         if isinstance(inner, str):
             from torch._dynamo.backends.registry import lookup_backend

@@ -31,38 +31,42 @@ def hip_quantize_rowwise(x: torch.Tensor, rotate: bool = False):
     return _lib.quant_rowwise(x, rotate=rotate)
 
 
-def _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend=None, prologue=None, side=None):
+def _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend=None, prologue=None, side=None, gate=None):
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
     kind, mod_scale, mod_shift, eps = (tuple(prologue) + (1e-6,))[:4] if prologue else (_lib.PRO_NONE, None, None, 1e-6)
     q, s = _lib.quant_rowwise(x2, rotate=rotate, prologue=kind, mod_scale=mod_scale, mod_shift=mod_shift, eps=eps)
     order = DEFAULT_EPILOGUE if order is None else order
     if side is not None:   # (side_t [M,r], side_b [N,r], alpha or None): the low-rank branch formed inside the epilogue
+        if gate is not None or addend is not None:
+            raise ValueError("the low-rank side branch takes neither a gate nor an addend")
         y = _lib.linear_w8a8_lora(q, s, weight, weight_scale, bias, side[0], side[1], side[2], compute_dtype, order)
     else:
-        y = _lib.linear_w8a8(q, s, weight, weight_scale, bias, compute_dtype, order, addend=addend)
+        y = _lib.linear_w8a8(q, s, weight, weight_scale, bias, compute_dtype, order, addend=addend, gate=gate)
     return y.reshape(*lead, weight.shape[0])
 
 
 def hip_int8_linear(x, weight, weight_scale, bias=None, compute_dtype=torch.float16, rotate=False, order=None,
-                    addend=None, prologue=None, side=None):
+                    addend=None, prologue=None, side=None, gate=None):
     """W8A8 linear with ONE weight scale (Python float or 1-element tensor).  `addend`, a tensor of the
     output's shape and dtype, is added to the result inside the epilogue (and the sum rounded again).
     `prologue` = (kind, mod_scale, mod_shift[, eps]) applies _lib.PRO_GELU_TANH, _lib.PRO_MODULATE, _lib.PRO_SILU_GATE or
     _lib.PRO_NORM_MODULATE to x inside the quantiser.  `side` = (side_t [M,r], side_b [N,r], alpha or None) adds the low-rank product side_t @ side_b.T,
-    formed inside the epilogue (see _lib.linear_w8a8_lora), instead of a ready-made addend."""
+    formed inside the epilogue (see _lib.linear_w8a8_lora), instead of a ready-made addend.  `gate` ([.., 1, N] or [N],
+    one vector per group of consecutive rows) multiplies the rounded result before the addend is added:
+    addend + gate * y, the gated residual of an adaLN-Zero block."""
     if isinstance(weight_scale, torch.Tensor) and weight_scale.numel() != 1:
         # the reference's kernel reads element 0 only (int8_fused_kernel.py:153)
         weight_scale = weight_scale.reshape(-1)[:1]
-    return _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend, prologue, side)
+    return _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend, prologue, side, gate)
 
 
 def hip_int8_linear_per_row(x, weight, weight_scale, bias=None, compute_dtype=torch.float16, rotate=False, order=None,
-                            addend=None, prologue=None, side=None):
+                            addend=None, prologue=None, side=None, gate=None):
     """W8A8 linear with one weight scale per output row ([N,1] or [N] float32 tensor)."""
     if not isinstance(weight_scale, torch.Tensor) or weight_scale.numel() != weight.shape[0]:
         raise ValueError("per-row weight scale must be a tensor with one element per weight row")
-    return _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend, prologue, side)
+    return _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend, prologue, side, gate)
 
 
 def hip_int8_linear_pair(xs, weights, weight_scales, biases=(None, None), compute_dtype=torch.float16, rotate=False, order=None):

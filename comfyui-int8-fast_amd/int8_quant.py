@@ -79,19 +79,26 @@ def stochastic_round_int8_delta(x: Tensor, scale, seed: int = 0, noise: Tensor |
 # --------------------------------------------------------------------------- forward functions
 @torch.no_grad()
 def int8_forward_dynamic(x: Tensor, weight: Tensor, weight_scale, bias, compute_dtype: torch.dtype,
-                         rotate: bool = False, addend: Tensor | None = None, prologue=None, side=None) -> Tensor:
+                         rotate: bool = False, addend: Tensor | None = None, prologue=None, side=None, gate=None) -> Tensor:
     """Dynamic per-token activation quantisation, ONE weight scale (int8_quant.py:68-88)."""
     return hip_int8_linear(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=prologue,
-                           side=side)
+                           side=side, gate=gate)
 
 
 @torch.no_grad()
 def int8_forward_dynamic_per_row(x: Tensor, weight: Tensor, weight_scale: Tensor, bias,
                                  compute_dtype: torch.dtype, rotate: bool = False, addend: Tensor | None = None,
-                                 prologue=None, side=None) -> Tensor:
+                                 prologue=None, side=None, gate=None) -> Tensor:
     """Dynamic per-token activation quantisation, per-row weight scales [N,1] (int8_quant.py:92-119)."""
     return hip_int8_linear_per_row(x, weight, weight_scale, bias, compute_dtype, rotate=rotate, addend=addend,
-                                   prologue=prologue, side=side)
+                                   prologue=prologue, side=side, gate=gate)
+
+
+class _ShapeAndDtype:
+    """What modulation_broadcasts_over_tokens looks at, for a tensor that does not exist yet (a layer's output)."""
+
+    def __init__(self, shape, dtype):
+        self.shape, self.dtype = tuple(shape), dtype
 
 
 def forward_pair(layers, xs):
@@ -436,15 +443,34 @@ class Int8TensorwiseOps(manual_cast):
 
         # -- forward ------------------------------------------------------------------------
         def forward(self, x: Tensor, prologue: int = _lib.PRO_NONE, mod_scale: Tensor | None = None,
-                    mod_shift: Tensor | None = None, eps: float = 1e-6) -> Tensor:
+                    mod_shift: Tensor | None = None, eps: float = 1e-6, gate: Tensor | None = None,
+                    residual: Tensor | None = None) -> Tensor:
             """The reference's forward(x) (int8_quant.py:703-778).  The optional arguments name the elementwise
             operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, _lib.PRO_MODULATE with
             (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension, _lib.PRO_NORM_MODULATE with
             the same modulation of layer_norm(x, eps) (no affine parameters: the whole adaLN producer of a DiT
             block), or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
             path then applies inside its quantiser instead of in passes of their own (under torch.compile the graph
-            rewrite of compile_ops does this without the caller's help)."""
+            rewrite of compile_ops does this without the caller's help).  `gate` / `residual` name what the caller would
+            apply to the result: forward(h, gate=g, residual=x) returns x + g * linear(h), the gated residual of an
+            adaLN-Zero block (g broadcast over the token dimension like the modulation vectors), formed inside the GEMM
+            epilogue with the roundings of torch's two operations; gate or residual alone work the same way."""
             managed = self.comfy_cast_weights or len(self.weight_function) > 0 or len(self.bias_function) > 0
+            fuse_epilogue = False
+            if gate is not None or residual is not None:
+                cdt = x.dtype if x.dtype in (torch.float16, torch.bfloat16) else torch.bfloat16
+                out_shape = (*x.shape[:-1], self.weight.shape[0])
+                fuse_epilogue = (self._is_quantized and x.numel() // max(1, x.shape[-1]) > SMALL_BATCH_ROWS and self.lora_A is None
+                                 and not torch.compiler.is_compiling() and x.dim() >= 2
+                                 and (residual is None or (tuple(residual.shape) == out_shape and residual.dtype == cdt
+                                                           and residual.device == x.device))
+                                 and (gate is None or (gate.device == x.device and compile_ops.modulation_broadcasts_over_tokens(
+                                     _ShapeAndDtype(out_shape, cdt), gate, gate))))
+                if not fuse_epilogue:   # torch applies the two operations, as the caller would have
+                    y = self.forward(x, prologue, mod_scale, mod_shift, eps)
+                    if gate is not None:
+                        y = gate * y
+                    return y if residual is None else residual + y
             if prologue != _lib.PRO_NONE:
                 rows = x.numel() // max(1, x.shape[-1])
                 fusable = (self._is_quantized and rows > SMALL_BATCH_ROWS and self.lora_A is None
@@ -536,8 +562,10 @@ class Int8TensorwiseOps(manual_cast):
                 else:
                     fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
                     pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift, eps)
+                    if fuse_epilogue:   # (no dynamic LoRA here: the addend slot is free for the residual stream)
+                        addend = None if residual is None else residual.reshape(-1, residual.shape[-1])
                     y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=pro,
-                            side=side_factors)
+                            side=side_factors, gate=gate if fuse_epilogue else None)
             else:
                 # W8A16: activations keep their dtype (rotated first when the weight is rotated)
                 if compiling:

@@ -3,6 +3,8 @@ Dynamo tracing of Linear.forward without graph breaks, the graph rewrite that mo
 operation in front of a layer into its quantiser, and (GPU) the compiled forward (aot_eager and
 inductor) against eager and against the CPU oracle."""
 import numpy as np
+import operator
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -239,6 +241,53 @@ def test_graph_rewrite_moves_layer_norm_and_modulation_into_the_quantiser(pkg):
         assert node.args[1] == pkg._lib.PRO_MODULATE and ln_left
 
 
+def test_graph_rewrite_moves_the_gated_residual_into_the_epilogue(pkg):
+    """x + gate * proj(h), the residual update of an adaLN-Zero block: multiplication and addition become the layer's
+    epilogue (in any operand order); the gate alone and the residual alone are taken too; a gate of another dtype, a
+    result that is used elsewhere as well, or a residual that torch would broadcast are left to torch."""
+    g = torch.Generator().manual_seed(14)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Block(torch.nn.Module):
+        def __init__(self, form):
+            super().__init__()
+            self.proj, self.form = lin(256, 128), form
+
+        def forward(self, x, h, gate):
+            y = self.proj(h)
+            if self.form == 0:
+                return x + gate * y
+            if self.form == 1:
+                return y * gate + x
+            if self.form == 2:
+                return gate * y
+            if self.form == 3:
+                return x + y
+            if self.form == 4:
+                return x + gate.float() * y          # promotes: torch's business
+            if self.form == 5:
+                return x + gate * y + y.mean()         # the layer's result has another user
+            return x[:, :1] + gate * y               # a residual that broadcasts
+
+    x, h, gate = torch.randn(2, 24, 256).bfloat16(), torch.randn(2, 24, 128).bfloat16(), torch.randn(2, 1, 256).bfloat16()
+    for form, want in ((0, (True, True)), (1, (True, True)), (2, (True, False)), (3, (False, True)), (4, None), (5, None), (6, (True, False))):
+        gm = torch._dynamo.export(Block(form))(x, h, gate).graph_module
+        n = pkg.compile_ops.fuse_epilogues(gm)
+        lins = [nd for nd in gm.graph.nodes if nd.op == "call_function" and "int8_linear" in str(nd.target)]
+        assert len(lins) == 1
+        if want is None:
+            assert n == 0 and lins[0].kwargs.get("gate") is None and lins[0].kwargs.get("addend") is None
+            continue
+        assert n == 1
+        assert (lins[0].kwargs.get("gate") is not None, lins[0].kwargs.get("addend") is not None) == want
+        left = [str(nd.target) for nd in gm.graph.nodes if nd.op == "call_function" and nd.target in (operator.mul, operator.add, torch.mul, torch.add)]
+        assert len(left) == (1 if form == 6 else 0), left     # (form 6 keeps its broadcasting addition)
+
+
 def test_modulation_broadcast_rule(pkg):
     ok = pkg.compile_ops.modulation_broadcasts_over_tokens
     x = torch.empty(2, 24, 256, dtype=torch.bfloat16)
@@ -352,6 +401,52 @@ def test_compiled_adaln_block_with_the_layer_norm_in_the_quantiser(pkg, dev, O):
     assert (diff != 0).mean() < 0.1
     eager = m(x.to(dev), sc.to(dev), sh.to(dev))       # torch's LayerNorm and modulation, then the layer
     assert (got.float() - eager.float()).abs().max().item() <= 2.0**-7 * eager.float().abs().max().item()
+
+
+@pytest.mark.gpu
+def test_compiled_adaln_zero_block_equals_eager_bit_for_bit(pkg, dev):
+    """x + gate * proj(gelu(up((1 + scale) * norm(x) + shift))) compiled with the rewriting backend over inductor: both
+    layers carry a prologue, the second also the gated residual in its epilogue, and no elementwise kernel of the block
+    is left for inductor; the result equals the same module run with this library's eager fused forward calls."""
+    g = torch.Generator().manual_seed(9)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = torch.nn.LayerNorm(256, elementwise_affine=False, eps=1e-6)
+            self.up, self.down = lin(512, 256), lin(256, 512)
+
+        def forward(self, x, scale, shift, gate):
+            h = self.up((1 + scale) * self.norm(x) + shift)
+            return x + gate * self.down(F.gelu(h, approximate="tanh"))
+
+    m = Block().to(dev)
+    x = (torch.randn(2, 40, 256, generator=g) * 2).bfloat16().to(dev)
+    sc, sh, gate = ((torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev) for _ in range(3))
+    seen = []
+
+    def counting(gm, inputs):
+        calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum("int8_linear_prologue" in str(n.target) for n in calls),
+                     sum(n.kwargs.get("gate") is not None and n.kwargs.get("addend") is not None for n in calls),
+                     sum(n.target in (operator.mul, operator.add, torch.mul, torch.add) or "gelu" in str(n.target) or "layer_norm" in str(n.target)
+                         for n in calls)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x, sc, sh, gate)
+    assert seen == [(2, 1, 0)]
+    L = pkg._lib
+    h = m.up(x, prologue=L.PRO_NORM_MODULATE, mod_scale=sc, mod_shift=sh, eps=1e-6)
+    want = m.down(h, prologue=L.PRO_GELU_TANH, gate=gate, residual=x)
+    assert torch.equal(got, want)
+    loose = m(x, sc, sh, gate)                           # torch's LayerNorm, modulation, gelu, gate and residual around the layers
+    assert (got.float() - loose.float()).abs().max().item() <= 2.0**-6 * loose.float().abs().max().item()
 
 
 @pytest.mark.gpu

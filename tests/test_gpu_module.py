@@ -301,6 +301,39 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
     assert torch.equal(lin(x32, prologue=L.PRO_NORM_MODULATE, mod_scale=sc_, mod_shift=sh_), lin((1 + sc_) * F.layer_norm(x32, (384,), eps=1e-6) + sh_))
 
 
+def test_forward_with_gate_and_residual_equals_the_unfused_sequence(pkg, dev):
+    """forward(h, gate=g, residual=x) == x + g * forward(h) bit for bit (two torch operations of the compute dtype, formed
+    inside the GEMM epilogue), with either one alone, combined with a prologue, on the QuaRot path, and on every path
+    that leaves the operations to torch (small batch, a gate torch would broadcast differently, binary32 residual)."""
+    L = pkg._lib
+    g = torch.Generator().manual_seed(23)
+    lin = pkg.Int8TensorwiseOps.Linear(384, 256, bias=True)
+    lin._load_from_state_dict({"l.weight": torch.randint(-127, 128, (256, 384), dtype=torch.int8, generator=g),
+                               "l.weight_scale": torch.rand(256, 1, generator=g) * 0.002 + 1e-3,
+                               "l.bias": torch.randn(256, generator=g).bfloat16()}, "l.", {}, True, [], [], [])
+    lin = lin.to(dev)
+    h = torch.randn(2, 40, 384, generator=g).bfloat16().to(dev)
+    x = torch.randn(2, 40, 256, generator=g).bfloat16().to(dev)
+    gate = torch.randn(2, 1, 256, generator=g).bfloat16().to(dev)
+    sc, sh = (torch.randn(2, 1, 384, generator=g) * 0.3).bfloat16().to(dev), torch.randn(2, 1, 384, generator=g).bfloat16().to(dev)
+    for quarot in (False, True):
+        lin._use_quarot = quarot
+        y = lin(h)
+        assert torch.equal(lin(h, gate=gate, residual=x), x + gate * y)
+        assert torch.equal(lin(h, gate=gate), gate * y)
+        assert torch.equal(lin(h, residual=x), x + y)
+        assert torch.equal(lin(h, gate=gate.reshape(2, 256)[0], residual=x), x + gate.reshape(2, 256)[0] * y)   # one vector for all rows
+        ym = lin(h, prologue=L.PRO_MODULATE, mod_scale=sc, mod_shift=sh)
+        assert torch.equal(lin(h, prologue=L.PRO_MODULATE, mod_scale=sc, mod_shift=sh, gate=gate, residual=x), x + gate * ym)
+    lin._use_quarot = False
+    y = lin(h)
+    per_token = torch.randn(1, 40, 256, generator=g).bfloat16().to(dev)      # torch broadcasts this over the batch, not over the tokens
+    assert torch.equal(lin(h, gate=per_token, residual=x), x + per_token * y)
+    assert torch.equal(lin(h, gate=gate, residual=x.float()), x.float() + gate * y)
+    small = h[:1, :4]
+    assert torch.equal(lin(small, gate=gate[:1], residual=x[:1, :4]), x[:1, :4] + gate[:1] * lin(small))
+
+
 @pytest.mark.parametrize("quarot", [False, True])
 def test_forward_pair_equals_the_layers_own_forward(pkg, dev, quarot):
     """forward_pair: the same projection of two token streams with their own weights, activations quantised in one
