@@ -502,6 +502,41 @@ def extras(L, dev, quick=False):
                                                      "GEMM; torch's two kernels move 142 MB"}
     del hq, wqg, res, og
 
+    # The MLP half of an adaLN-Zero block on config 1's shapes, x + gate * down(gelu(up((1 + scale) * norm(x) + shift))):
+    # every elementwise operation inside a quantiser or an epilogue (4 launches) against the same two quantised layers
+    # with torch's kernels around them (LayerNorm, modulation, GELU, gate, residual: 8 more launches)
+    Mm, Dm, Hm = 4608, 3072, 12288
+    xm = _acts(g, Mm, Dm, 1.0, 20.0).to(dev)
+    w_up, s_up = L.quant_rowwise(torch.randn(Hm, Dm, device=dev) * 0.02)
+    w_dn, s_dn = L.quant_rowwise(torch.randn(Dm, Hm, device=dev) * 0.02)
+    b_up, b_dn = (torch.randn(Hm, device=dev) * 0.01).bfloat16(), (torch.randn(Dm, device=dev) * 0.01).bfloat16()
+    m_sc, m_sh, m_gate = ((torch.randn(1, Dm, device=dev) * 0.3).bfloat16() for _ in range(3))
+    h_buf = torch.empty(Mm, Hm, dtype=torch.bfloat16, device=dev)
+    o_buf = torch.empty(Mm, Dm, dtype=torch.bfloat16, device=dev)
+
+    def mlp_fused(_i):
+        q1, s1 = L.quant_rowwise(xm, prologue=L.PRO_NORM_MODULATE, mod_scale=m_sc, mod_shift=m_sh, eps=1e-6)
+        L.linear_w8a8(q1, s1, w_up, s_up, b_up, torch.bfloat16, L.EPI_TORCH, h_buf)
+        q2, s2 = L.quant_rowwise(h_buf, prologue=L.PRO_GELU_TANH)
+        L.linear_w8a8(q2, s2, w_dn, s_dn, b_dn, torch.bfloat16, L.EPI_TORCH, o_buf, addend=xm, gate=m_gate)
+
+    def mlp_unfused(_i):
+        z = (1 + m_sc) * F.layer_norm(xm, (Dm,), eps=1e-6) + m_sh
+        q1, s1 = L.quant_rowwise(z)
+        L.linear_w8a8(q1, s1, w_up, s_up, b_up, torch.bfloat16, L.EPI_TORCH, h_buf)
+        q2, s2 = L.quant_rowwise(F.gelu(h_buf, approximate="tanh"))
+        y = L.linear_w8a8(q2, s2, w_dn, s_dn, b_dn, torch.bfloat16, L.EPI_TORCH, o_buf)
+        return xm + m_gate * y
+
+    t_mf = time_kernel(mlp_fused, max(10, iters // 4))
+    t_mu = time_kernel(mlp_unfused, max(10, iters // 4))
+    out["adaln_zero_mlp_4608x3072x12288"] = {"ms_all_elementwise_work_fused": round(t_mf["median_us"] / 1e3, 4),
+                                             "ms_torch_kernels_around_the_layers": round(t_mu["median_us"] / 1e3, 4),
+                                             "note": "x + gate * down(gelu(up((1 + scale) * layer_norm(x) + shift))), bf16, M = 4608: 2 quantiser "
+                                                     "launches (LayerNorm + modulation, tanh-GELU) and 2 GEMMs (the second with gate and residual) "
+                                                     "against the same layers with 8 torch kernels around them"}
+    del xm, w_up, w_dn, h_buf, o_buf
+
     # config 2: QuaRot layer (width 3840, 2 % of the channels x50): time of the rotated path and what the
     # rotation buys in accuracy against the bf16 product
     c2 = make_config(2)
