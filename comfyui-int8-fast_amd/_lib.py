@@ -424,7 +424,7 @@ def linear_w8a8(a, a_scale, w, w_scale, bias=None, out_dtype=torch.bfloat16, ord
 class _LinearGroup(ctypes.Structure):
     _fields_ = [("a", ctypes.c_void_p), ("a_scale", ctypes.c_void_p), ("w", ctypes.c_void_p), ("w_scale", ctypes.c_void_p),
                 ("w_scale_host", ctypes.c_float), ("bias", ctypes.c_void_p), ("addend", ctypes.c_void_p), ("out", ctypes.c_void_p),
-                ("M", ctypes.c_int64)]
+                ("M", ctypes.c_int64), ("gate", ctypes.c_void_p), ("rows_per_gate", ctypes.c_int64)]
 
 
 MAX_LINEAR_GROUPS = 4
@@ -435,20 +435,20 @@ def _addr(t):
 
 
 def linear_w8a8_grouped(problems, out_dtype=torch.bfloat16, order=EPI_TORCH, outs=None):
-    """linear_w8a8 for several problems of one layer shape, each (a, a_scale, w, w_scale, bias) or
-    (a, a_scale, w, w_scale, bias, addend) with its own tensors: the image and the text tokens of a double-stream
+    """linear_w8a8 for several problems of one layer shape, each (a, a_scale, w, w_scale, bias[, addend[, gate]])
+    with its own tensors (addend and gate as for linear_w8a8): the image and the text tokens of a double-stream
     transformer block through the same projection.  One launch where the library finds that the small problems' tiles
     fit into the compute units the largest one's last round leaves idle, else one launch per problem; problems that do
     not share N, K, the scale mode and the bias dtype (or more than MAX_LINEAR_GROUPS of them) are launched one by one
     from here.  outs: optional list of contiguous [M_i, N] tensors of out_dtype to write into.
     -> list of outputs, bit-identical to separate linear_w8a8 calls."""
-    problems = [tuple(p) + (None,) * (6 - len(p)) for p in problems]
+    problems = [tuple(p) + (None,) * (7 - len(p)) for p in problems]
     if not problems:
         return []
     if outs is not None and len(outs) != len(problems):
         raise ValueError("outs must hold one tensor per problem")
     prepared = []
-    for a, a_scale, w, w_scale, bias, addend in problems:
+    for a, a_scale, w, w_scale, bias, addend, gate in problems:
         a, w = _i8_matrix(a, "a"), _i8_matrix(w, "w")
         M, K = a.shape
         N, K2 = w.shape
@@ -465,16 +465,25 @@ def linear_w8a8_grouped(problems, out_dtype=torch.bfloat16, order=EPI_TORCH, out
             if addend.numel() != M * N or addend.dtype != out_dtype:
                 raise ValueError(f"addend must have {M * N} elements of {out_dtype}")
             addend = addend.reshape(M, N).contiguous()
-        for name, t in (("w", w), ("a_scale", a_scale), ("addend", addend)):
+        rows_per_gate = 1
+        if gate is not None:
+            _dev(gate, "gate")
+            if gate.dtype != out_dtype or gate.numel() % max(N, 1) or gate.shape[-1] != N:
+                raise ValueError(f"gate must be [V,{N}] of {out_dtype}")
+            gate = gate.reshape(-1, N).contiguous()
+            if gate.shape[0] == 0 or M % gate.shape[0]:
+                raise ValueError(f"{M} rows do not split evenly over {gate.shape[0]} gate vectors")
+            rows_per_gate = max(1, M // gate.shape[0])
+        for name, t in (("w", w), ("a_scale", a_scale), ("addend", addend), ("gate", gate)):
             if isinstance(t, torch.Tensor) and t.device != a.device:
                 raise ValueError(f"{name} is on {t.device}, a is on {a.device}")
-        prepared.append((a, a_scale, w, ws, ws_host, mode, bias, bcode, addend, M, N, K))
+        prepared.append((a, a_scale, w, ws, ws_host, mode, bias, bcode, addend, M, N, K, gate, rows_per_gate))
     first = prepared[0]
     bcodes = {p[7] for p in prepared if p[6] is not None}
     same = (len(prepared) <= MAX_LINEAR_GROUPS and len(bcodes) <= 1
             and all(p[10] == first[10] and p[11] == first[11] and p[5] == first[5] and p[0].device == first[0].device for p in prepared))
     if not same:
-        return [linear_w8a8(p[0], p[1], p[2], src[3], p[6], out_dtype, order, None if outs is None else outs[i], addend=p[8])
+        return [linear_w8a8(p[0], p[1], p[2], src[3], p[6], out_dtype, order, None if outs is None else outs[i], addend=p[8], gate=p[12])
                 for i, (p, src) in enumerate(zip(prepared, problems))]
     N, K, mode, device = first[10], first[11], first[5], first[0].device
     if outs is None:
@@ -487,6 +496,7 @@ def linear_w8a8_grouped(problems, out_dtype=torch.bfloat16, order=EPI_TORCH, out
     for g, p, o in zip(groups, prepared, outs):
         g.a, g.a_scale, g.w, g.w_scale, g.w_scale_host = _addr(p[0]), _addr(p[1]), _addr(p[2]), _addr(p[3]), p[4]
         g.bias, g.addend, g.out, g.M = _addr(p[6]), _addr(p[8]), _addr(o), p[9]
+        g.gate, g.rows_per_gate = _addr(p[12]), p[13]
     with _on(device):
         work = None
         for p in prepared:   # (used only if the library launches the problems one by one and one of them has a long K)

@@ -129,6 +129,8 @@ extern "C" int i8f_linear_w8a8_grouped(const i8f_linear_group *groups, int n_gro
         g.x = p.a, g.w = p.w, g.M = (int)p.M, g.N = (int)N, g.K = (int)K, g.out = p.out;
         g.xs = p.a_scale, g.ws = p.w_scale, g.ws_host = p.w_scale_host, g.row_scale = scale_mode == I8F_SCALE_ROW;
         g.bias = p.bias, g.bias_dtype = bias_dtype, g.order = order, g.addend = p.addend;
+        if (p.gate && p.rows_per_gate <= 0) return I8F_ERR_INVALID;
+        g.gate = p.gate, g.gate_rows = (int)(p.rows_per_gate < 0x7fffffff ? p.rows_per_gate : 0x7fffffff);
         if (workspace) g.arrivals = (unsigned *)workspace, g.partials = (int *)((char *)workspace + SPLITK_COUNTER_BYTES);
         gs[n++] = g;
     }

@@ -278,11 +278,12 @@ __device__ __forceinline__ uint4 mul_rounded(uint4 y, uint4 s) {
 // first 16 dwords of the kernel arguments are preloaded into SGPRs at wave launch, the rest (epilogue
 // operands) is fetched by scalar loads that have the whole main loop to land.
 // (The body is shared by the kernel of one problem and the kernel of a group of problems: wg_id is the workgroup's
-// number within its problem, gout / gaddend / ws_host that problem's output, addend and host-side weight scale.)
+// number within its problem, gout / gaddend / ggate / ws_host that problem's output, addend, gate and host-side weight scale.)
 template <class C, int OUT, bool KTAIL, bool SIDE = false, bool SPLITK = false>
 __device__ __forceinline__ void gemm_i8_body(const int8_t *gx, const int8_t *gw, int gM, int gN, int gK, int tiles_m, int tiles_n,
                                              const float *gxs, const float *gws, const void *gbias, int flags, const GemmArgs &g,
-                                             const int wg_id, void *gout, const void *gaddend, const float ws_host) {
+                                             const int wg_id, void *gout, const void *gaddend, const float ws_host,
+                                             const void *ggate, const int ggate_rows) {
     constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NW = C::NW, MI = C::MI, NJ = C::NJ, CB = C::CB, CPR = C::CPR;
     constexpr int S = C::STAGES, WS = C::WSTAGES;
     constexpr bool ASYM = WS != S;  // the W tile one stage deeper than the X tile
@@ -928,8 +929,8 @@ __device__ __forceinline__ void gemm_i8_body(const int8_t *gx, const int8_t *gw,
                 {
                     const int64_t off = ((int64_t)mm * gN + nn) * OB;
                     uint4 v = val;
-                    if (g.gate)
-                        v = mul_rounded<OUT>(v, *(const uint4 *)((const char *)g.gate + ((int64_t)((uint32_t)mm / (uint32_t)g.gate_rows) * gN + nn) * OB));
+                    if (ggate)
+                        v = mul_rounded<OUT>(v, *(const uint4 *)((const char *)ggate + ((int64_t)((uint32_t)mm / (uint32_t)ggate_rows) * gN + nn) * OB));
                     if (gaddend) v = add_rounded<OUT>(v, *(const uint4 *)((const char *)gaddend + off));
                     stream_store16((char *)gout + off, v);
                 }
@@ -958,7 +959,7 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_kernel(const int8_t *gx, const 
                                                         const float *gxs, const float *gws, const void *gbias, int flags,
                                                         const GemmArgs g) {
     gemm_i8_body<C, OUT, KTAIL, SIDE, SPLITK>(gx, gw, gM, gN, gK, tiles_m, tiles_n, gxs, gws, gbias, flags, g, (int)blockIdx.x, g.out,
-                                              g.addend, g.ws_host);
+                                              g.addend, g.ws_host, g.gate, g.gate_rows);
 }
 
 // Several problems of one layer shape (N, K, scale mode, dtypes) with their own activations, weights and outputs in
@@ -970,10 +971,10 @@ constexpr int MAX_GEMM_GROUPS = 4;
 struct GemmGroups {
     const int8_t *x[MAX_GEMM_GROUPS], *w[MAX_GEMM_GROUPS];
     const float *xs[MAX_GEMM_GROUPS], *ws[MAX_GEMM_GROUPS];
-    const void *bias[MAX_GEMM_GROUPS], *addend[MAX_GEMM_GROUPS];
+    const void *bias[MAX_GEMM_GROUPS], *addend[MAX_GEMM_GROUPS], *gate[MAX_GEMM_GROUPS];
     void *out[MAX_GEMM_GROUPS];
     float ws_host[MAX_GEMM_GROUPS];
-    int M[MAX_GEMM_GROUPS], tiles_m[MAX_GEMM_GROUPS];
+    int M[MAX_GEMM_GROUPS], tiles_m[MAX_GEMM_GROUPS], gate_rows[MAX_GEMM_GROUPS];
     int first_tile[MAX_GEMM_GROUPS + 1];  // [n] = all tiles
     int n;
 };
@@ -986,7 +987,8 @@ __global__ __launch_bounds__(C::NT) void gemm_i8_grouped_kernel(int gN, int gK, 
         if (i < gg.n && (int)blockIdx.x >= gg.first_tile[i]) grp = i;
     grp = __builtin_amdgcn_readfirstlane(grp);
     gemm_i8_body<C, OUT, false>(gg.x[grp], gg.w[grp], gg.M[grp], gN, gK, gg.tiles_m[grp], tiles_n, gg.xs[grp], gg.ws[grp], gg.bias[grp],
-                                flags, g, (int)blockIdx.x - gg.first_tile[grp], gg.out[grp], gg.addend[grp], gg.ws_host[grp]);
+                                flags, g, (int)blockIdx.x - gg.first_tile[grp], gg.out[grp], gg.addend[grp], gg.ws_host[grp], gg.gate[grp],
+                                gg.gate_rows[grp]);
 }
 
 // ---- slow but shape-agnostic kernel: one thread per output -----------------------------
@@ -1270,6 +1272,7 @@ int launch_cfg_grouped(const GemmArgs *gs, int n, hipStream_t st) {
     for (int i = 0; i < n; ++i) {
         gg.x[i] = gs[i].x, gg.w[i] = gs[i].w, gg.xs[i] = gs[i].xs, gg.ws[i] = gs[i].ws, gg.bias[i] = gs[i].bias;
         gg.addend[i] = gs[i].addend, gg.out[i] = gs[i].out, gg.ws_host[i] = gs[i].ws_host, gg.M[i] = gs[i].M;
+        gg.gate[i] = gs[i].gate, gg.gate_rows[i] = gs[i].gate ? gs[i].gate_rows : 1;
         gg.tiles_m[i] = (gs[i].M + C::BM - 1) / C::BM;
         gg.first_tile[i] = first;
         first += gg.tiles_m[i] * tiles_n;
@@ -1334,7 +1337,7 @@ int launch_group(GemmArgs *gs, int n, hipStream_t st) {
         together = (g.K % 128 == 0) && (g.N % 8 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
                    ((uintptr_t)g.out % 16 == 0) && ((int64_t)g.N * g.K < (1ll << 31)) && ((int64_t)g.M * g.K < (1ll << 31)) &&
                    (!g.ws || !g.row_scale || (uintptr_t)g.ws % 16 == 0) && (!g.bias || (uintptr_t)g.bias % 16 == 0) &&
-                   (!g.addend || (uintptr_t)g.addend % 16 == 0) && !g.side_t && !g.gate;
+                   (!g.addend || (uintptr_t)g.addend % 16 == 0) && (!g.gate || (uintptr_t)g.gate % 16 == 0) && !g.side_t;
     }
     Tile t = TILE_BIG;
     if (together) {

@@ -69,20 +69,25 @@ def hip_int8_linear_per_row(x, weight, weight_scale, bias=None, compute_dtype=to
     return _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend, prologue, side, gate)
 
 
-def hip_int8_linear_pair(xs, weights, weight_scales, biases=(None, None), compute_dtype=torch.float16, rotate=False, order=None):
+def hip_int8_linear_pair(xs, weights, weight_scales, biases=(None, None), compute_dtype=torch.float16, rotate=False, order=None,
+                         gates=None, residuals=None):
     """The same layer type applied to several token streams, each with its own weight (the image and the text stream
     of a double-stream transformer block; the reference calls its operator once per stream, int8_quant.py:703-778):
     the activations of all streams are quantised in ONE launch (they share their width and dtype), and their GEMMs
     go out as one launch where the small stream's tiles fit into the compute units the large one leaves idle (else one
-    launch per stream).  -> list of outputs, bit-identical to separate hip_int8_linear[_per_row] calls."""
+    launch per stream).  gates / residuals: per stream, a gate ([.., 1, N] or [N]) and a residual of the output's shape
+    and dtype, or None: residual + gate * y in the epilogue.
+    -> list of outputs, bit-identical to separate hip_int8_linear[_per_row] calls."""
     leads = [x.shape[:-1] for x in xs]
     quantised = _lib.quant_rowwise_grouped([x.reshape(-1, x.shape[-1]) for x in xs], rotate=rotate)
     order = DEFAULT_EPILOGUE if order is None else order
     problems = []
-    for (q, s), w, ws, b in zip(quantised, weights, weight_scales, biases):
+    gates = gates or [None] * len(xs)
+    residuals = residuals or [None] * len(xs)
+    for (q, s), w, ws, b, gt, rs in zip(quantised, weights, weight_scales, biases, gates, residuals):
         if isinstance(ws, torch.Tensor) and ws.numel() not in (1, w.shape[0]):
             ws = ws.reshape(-1)[:1]
-        problems.append((q, s, w, ws, b))
+        problems.append((q, s, w, ws, b, None if rs is None else rs.reshape(-1, rs.shape[-1]), gt))
     outs = _lib.linear_w8a8_grouped(problems, compute_dtype, order)
     return [o.reshape(*lead, o.shape[-1]) for o, lead in zip(outs, leads)]
 

@@ -101,15 +101,18 @@ class _ShapeAndDtype:
         self.shape, self.dtype = tuple(shape), dtype
 
 
-def forward_pair(layers, xs):
+def forward_pair(layers, xs, gates=None, residuals=None):
     """Linear.forward for several quantised layers of one shape at once, e.g. the same projection of the image and of
     the text stream of a double-stream block: [layer(x) for layer, x in zip(layers, xs)], with the activations of all
     streams quantised by ONE kernel launch where the layers allow it (W8A8 path on every stream: more than 16 rows,
     quantised weights on the inputs' device, no dynamic LoRA, no managed casting, the same rotation flag, inputs of one
-    width and one 16-bit dtype, eager mode).  Anything else falls back to the layers' own forward; results are
-    bit-identical either way."""
+    width and one 16-bit dtype, eager mode).  gates / residuals: per layer, what forward(x, gate=, residual=) takes
+    (the gated residual of the block in the epilogue), or None.  Anything else falls back to the layers' own forward;
+    results are bit-identical either way."""
     layers, xs = list(layers), list(xs)
-    ok = len(layers) >= 2 and len(layers) == len(xs) and not torch.compiler.is_compiling()
+    gates = list(gates) if gates is not None else [None] * len(xs)
+    residuals = list(residuals) if residuals is not None else [None] * len(xs)
+    ok = len(layers) >= 2 and len(layers) == len(xs) == len(gates) == len(residuals) and not torch.compiler.is_compiling()
     if ok:
         x0 = xs[0]
         rot = bool(getattr(layers[0], "_use_quarot", False))
@@ -120,8 +123,14 @@ def forward_pair(layers, xs):
                          and x.dtype == x0.dtype and x.dtype in (torch.float16, torch.bfloat16) and x.shape[-1] == x0.shape[-1]
                          and x.device == x0.device and x.numel() // max(1, x.shape[-1]) > SMALL_BATCH_ROWS
                          and bool(getattr(lin, "_use_quarot", False)) == rot)
+    if ok:   # gates and residuals in the form the epilogue takes, else every layer goes alone
+        for lin, x, gt, rs in zip(layers, xs, gates, residuals):
+            shape = (*x.shape[:-1], lin.weight.shape[0])
+            ok = ok and (rs is None or (tuple(rs.shape) == shape and rs.dtype == x.dtype and rs.device == x.device))
+            ok = ok and (gt is None or (gt.device == x.device and x.dim() >= 2
+                                        and compile_ops.modulation_broadcasts_over_tokens(_ShapeAndDtype(shape, x.dtype), gt, gt)))
     if not ok:
-        return [lin(x) for lin, x in zip(layers, xs)]
+        return [lin(x, gate=gt, residual=rs) for lin, x, gt, rs in zip(layers, xs, gates, residuals)]
     scales = []
     for lin in layers:
         ws = lin._get_weight_scale()
@@ -129,7 +138,7 @@ def forward_pair(layers, xs):
             ws = ws.to(xs[0].device, non_blocking=True)
         scales.append(ws)
     return int8_fused_kernel.hip_int8_linear_pair(xs, [lin.weight for lin in layers], scales, [lin.bias for lin in layers],
-                                                  xs[0].dtype, rotate=rot)
+                                                  xs[0].dtype, rotate=rot, gates=gates, residuals=residuals)
 
 
 # --------------------------------------------------------------------------- LoRA delta reconstruction

@@ -316,7 +316,7 @@ int i8f_linear_w8a8_gated(const int8_t *a, const float *a_scale, const int8_t *w
 
 /*
  * i8f_linear_w8a8_splitk for several layers of one shape at once: group i is a problem of its own
- * (activations, weights, scales, bias, addend, output, row count M) and the groups share N, K, the
+ * (activations, weights, scales, bias, gate, addend, output, row count M) and the groups share N, K, the
  * scale mode, the dtypes and the operation order.  No counterpart in the reference, whose operator
  * (int8_forward_dynamic*, int8_quant.py:65-118; Int8TensorwiseOps.Linear.forward, :703-778) takes one
  * layer: a double-stream transformer block runs every projection twice, for its image and for its
@@ -339,6 +339,8 @@ typedef struct i8f_linear_group {
     const void *addend;     /* [M,N] of out_dtype or NULL */
     void *out;              /* [M,N] of out_dtype */
     int64_t M;
+    const void *gate;       /* [ceil(M / rows_per_gate), N] of out_dtype or NULL: as for i8f_linear_w8a8_gated */
+    int64_t rows_per_gate;
 } i8f_linear_group;
 int i8f_linear_w8a8_grouped(const i8f_linear_group *groups, int n_groups, int scale_mode,
                             int bias_dtype, int out_dtype, int64_t N, int64_t K, int order,

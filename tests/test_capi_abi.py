@@ -118,6 +118,9 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 7, null, 0, null) == INVALID
     assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 0, one, 64, null) == INVALID      # workspace too small
     assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 5, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == UNSUPPORTED
+    lg[1].gate, lg[1].rows_per_gate = one.value, 0       # a gate without a row count
+    assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == INVALID
+    lg[1].gate = None
     lg[1].out = None
     assert lib.i8f_linear_w8a8_grouped(ctypes.byref(lg), 2, 1, L.BF16, L.BF16, 8, 16, 0, null, 0, null) == INVALID
     lg[1].out, lg[1].w_scale = one.value, None

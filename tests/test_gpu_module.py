@@ -356,3 +356,13 @@ def test_forward_pair_equals_the_layers_own_forward(pkg, dev, quarot):
     small = x_txt[:1, :3]                                  # three rows: that stream takes the W8A16 path, so no shared launch
     y_img2, y_small = pkg.forward_pair([img, txt], [x_img, small])
     assert torch.equal(y_img2, y_img) and torch.equal(y_small, txt(small))
+    # the residual update of both streams in the same launch: x + gate * layer(h) per stream, gate for one stream only,
+    # and a pair that falls back (the small batch) with its gates applied by torch
+    r_img, r_txt = torch.randn(2, 100, 192, generator=g).bfloat16().to(dev), torch.randn(2, 20, 192, generator=g).bfloat16().to(dev)
+    g_img, g_txt = torch.randn(2, 1, 192, generator=g).bfloat16().to(dev), torch.randn(2, 1, 192, generator=g).bfloat16().to(dev)
+    o_img, o_txt = pkg.forward_pair([img, txt], [x_img, x_txt], gates=[g_img, g_txt], residuals=[r_img, r_txt])
+    assert torch.equal(o_img, r_img + g_img * y_img) and torch.equal(o_txt, r_txt + g_txt * y_txt)
+    o_img, o_txt = pkg.forward_pair([img, txt], [x_img, x_txt], gates=[g_img, None], residuals=[None, r_txt])
+    assert torch.equal(o_img, g_img * y_img) and torch.equal(o_txt, r_txt + y_txt)
+    o_img, o_small = pkg.forward_pair([img, txt], [x_img, small], gates=[g_img, g_txt[:1]], residuals=[r_img, r_txt[:1, :3]])
+    assert torch.equal(o_img, r_img + g_img * y_img) and torch.equal(o_small, r_txt[:1, :3] + g_txt[:1] * txt(small))

@@ -498,15 +498,17 @@ def test_linear_w8a8_grouped_equals_separate_calls_and_the_oracle(L, dev, Ms, N,
         wq, ws = O.quant_rowwise(wf.numpy(), O.F32) if row else O.quant_tensorwise(wf.numpy(), O.F32)
         bias = None if bdt is None else (torch.randn(N, generator=G) * 0.01).to(bdt)
         addend = (torch.randn(M, N, generator=G) * 0.3).to(odt) if add else None
+        gate = torch.randn(2 if M % 2 == 0 and M else 1, N, generator=G).to(odt) if add and M else None   # (with the addends: gated residuals)
         q, s = L.quant_rowwise(x.to(dev)) if M else (torch.empty(0, K, dtype=torch.int8, device=dev), torch.empty(0, 1, device=dev))
         ws_arg = torch.from_numpy(ws).to(dev) if row else float(ws[0])
-        problems.append((q, s, torch.from_numpy(wq).to(dev), ws_arg, None if bias is None else bias.to(dev), None if addend is None else addend.to(dev)))
+        problems.append((q, s, torch.from_numpy(wq).to(dev), ws_arg, None if bias is None else bias.to(dev), None if addend is None else addend.to(dev),
+                         None if gate is None else gate.to(dev)))
         if M:
             xa, code = O.from_torch(x)
             ba, bcode = (None, O.BF16) if bias is None else O.from_torch(bias)
             y = O.linear_w8a8(xa, code, wq, ws, ba, bcode, ocode, 0, order)
             if add:
-                y = O.from_torch((O.to_torch(y, ocode).float() + addend.float()).to(odt))[0]
+                y = O.gate_residual(y, ocode, gate=O.from_torch(gate)[0], residual=O.from_torch(addend)[0], rows_per_gate=M // gate.shape[0])
             wants.append(y)
         else:
             wants.append(None)
@@ -517,7 +519,7 @@ def test_linear_w8a8_grouped_equals_separate_calls_and_the_oracle(L, dev, Ms, N,
         if M == 0:
             continue
         assert np.array_equal(bits(g), want)
-        alone = L.linear_w8a8(p[0], p[1], p[2], p[3], p[4], odt, order, addend=p[5])
+        alone = L.linear_w8a8(p[0], p[1], p[2], p[3], p[4], odt, order, addend=p[5], gate=p[6])
         assert torch.equal(alone, g)
 
 
