@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libi8f_gfx950.so")
 BF16, F16, F32 = 0, 1, 2
 SCALE_TENSOR, SCALE_ROW = 0, 1
 EPI_TORCH, EPI_FUSED = 0, 1
-PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE = 0, 1, 2, 3, 4
+PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE, PRO_CONCAT_GELU = 0, 1, 2, 3, 4, 5
 
 _DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
 
@@ -56,6 +56,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_quant_rowwise_grouped.argtypes = [vp, i32, i32, i64, i32, vp]
     L.i8f_quant_rowwise_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, i32, vp, vp, vp]
     L.i8f_quant_rowwise_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, i32, vp, vp, vp]
+    L.i8f_quant_rowwise_concat_gelu.argtypes = [vp, i32, i64, i64, i64, vp, i64, i64, i32, vp, vp, vp]
     L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
     L.i8f_quant_tensorwise_workspace_bytes.restype = i64
     L.i8f_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp, vp, i64, vp]
@@ -74,7 +75,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_linear_w8a8_gated", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
+    for name in ("i8f_quant_rowwise_concat_gelu", "i8f_linear_w8a8_gated", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -83,7 +84,7 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_rotate128",
-    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate",
+    "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_rowwise_concat_gelu",
     "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_gated", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
@@ -173,6 +174,38 @@ def _scale(ws, N: int, device):
 
 
 # --------------------------------------------------------------------------- entry points
+def concat_gelu_fusable(a: torch.Tensor, b: torch.Tensor) -> bool:
+    """Whether the quantiser takes cat(a, gelu(b)) itself (PRO_CONCAT_GELU): 2-D tensors of one 16-bit dtype and one row
+    count on one GPU, widths in multiples of 16 that add up to at most 16384, contiguous 16-byte aligned rows."""
+    def rows_ok(t):
+        return t.stride(1) == 1 and (t.shape[0] <= 1 or (t.stride(0) % 8 == 0 and t.stride(0) >= t.shape[1])) and t.data_ptr() % 16 == 0
+
+    return (a.is_cuda and a.dim() == 2 and b.dim() == 2 and a.dtype == b.dtype and a.dtype in (torch.bfloat16, torch.float16)
+            and a.device == b.device and a.shape[0] == b.shape[0] and a.shape[0] > 0 and a.shape[1] % 16 == 0 and b.shape[1] % 16 == 0
+            and a.shape[1] > 0 and b.shape[1] > 0 and a.shape[1] + b.shape[1] <= 16384 and rows_ok(a) and rows_ok(b))
+
+
+def quant_rowwise_concat_gelu(a: torch.Tensor, b: torch.Tensor, rotate: bool = False):
+    """quant_rowwise(cat((a, gelu(b, approximate="tanh")), -1)) without the activated tensor or the concatenation ever
+    existing: the input of the second projection of a single-stream transformer block.  a [M,Ka], b [M,Kb]
+    -> (int8 [M, Ka+Kb], float32 [M,1])."""
+    _dev(a, "a")
+    _dev(b, "b")
+    if not concat_gelu_fusable(a, b):
+        raise ValueError("these tensors have no fused concatenation (see concat_gelu_fusable)")
+    M, Ka = a.shape
+    Kb = b.shape[1]
+    if rotate and (Ka % 128 or Kb % 128):
+        raise ValueError(f"rotation needs both widths in multiples of 128, got {Ka} and {Kb}")
+    q = torch.empty((M, Ka + Kb), dtype=torch.int8, device=a.device)
+    s = torch.empty((M, 1), dtype=torch.float32, device=a.device)
+    with _on(a.device):
+        _check(lib().i8f_quant_rowwise_concat_gelu(_ptr(a), dtype_code(a.dtype), M, Ka, a.stride(0) if M > 1 else Ka, _ptr(b), Kb,
+                                                   b.stride(0) if M > 1 else Kb, 128 if rotate else 0, _ptr(q), _ptr(s), _stream(a)),
+               "i8f_quant_rowwise_concat_gelu")
+    return q, s
+
+
 def norm_modulate_fusable(x: torch.Tensor) -> bool:
     """Whether the quantiser takes PRO_NORM_MODULATE for these rows (one wavefront holds a row): 16-bit elements,
     a width of at most 4096 in multiples of 16, 16-byte aligned rows."""
@@ -186,8 +219,11 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
     mod_scale / mod_shift of x's dtype, [V,K] (or [K]): (1 + mod_scale) * x + mod_shift, M // V consecutive rows
     to a vector, or PRO_SILU_GATE with the gate operand as mod_scale (x's dtype, [M,K], or [V,K] like the vectors
     above): silu(x) * mod_scale, or PRO_NORM_MODULATE: the modulation applied to layer_norm(x, eps) without affine
-    parameters (see norm_modulate_fusable for the rows it takes)."""
+    parameters (see norm_modulate_fusable for the rows it takes), or PRO_CONCAT_GELU with a second tensor [M,Kb] as
+    mod_scale: cat((x, gelu(mod_scale)), -1) (see quant_rowwise_concat_gelu)."""
     _dev(x, "x")
+    if prologue == PRO_CONCAT_GELU:   # x followed by gelu(mod_scale) along the row
+        return quant_rowwise_concat_gelu(x, mod_scale, rotate=rotate)
     x = _rows(x, "x")
     M, K = x.shape
     if rotate and K % 128:

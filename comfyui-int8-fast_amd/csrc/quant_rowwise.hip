@@ -51,6 +51,10 @@ struct Prologue {
     const void *s, *t;       // modulation vectors (MODULATE, NORM_MODULATE), gate operand (SILU_GATE)
     int64_t rows_per_vec;    // rows that share one pair of vectors
     float eps;               // NORM_MODULATE: added to the row's variance
+    // CONCAT_GELU: the row is x's row (runs_a runs of 16 elements) followed by gelu(b's row); b [M, .] with its own stride
+    const void *b;
+    int64_t ldb_bytes;
+    int runs_a;
 };
 
 // the sum over the wave in a fixed order (the same in every lane)
@@ -455,12 +459,18 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
     {
         const bool ok = FULL || m < M;
         const char *xrow = x + (ok ? m : 0) * ldx_bytes;
+        [[maybe_unused]] const char *brow = nullptr;
+        if constexpr (PRO == I8F_PRO_CONCAT_GELU) brow = (const char *)pro.b + (ok ? m : 0) * pro.ldb_bytes;
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
             const int R = r * TPR + p;
             if (FULL || (ok && R < nruns)) {
-                raw[r][0] = *(const uint4 *)(xrow + (seg_run + R) * 32);
-                raw[r][1] = *(const uint4 *)(xrow + (seg_run + R) * 32 + 16);
+                const char *src = xrow + (seg_run + R) * 32;
+                if constexpr (PRO == I8F_PRO_CONCAT_GELU) {   // the runs behind x's row come from b's
+                    if (R >= pro.runs_a) src = brow + (int64_t)(R - pro.runs_a) * 32;
+                }
+                raw[r][0] = *(const uint4 *)src;
+                raw[r][1] = *(const uint4 *)(src + 16);
             } else {
                 raw[r][0] = make_uint4(0, 0, 0, 0);
                 raw[r][1] = make_uint4(0, 0, 0, 0);
@@ -524,6 +534,13 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
             } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) v[r][j] = apply_prologue<DT, PRO>(v[r][j], 0.0f, 0.0f);
+            } else if constexpr (PRO == I8F_PRO_CONCAT_GELU) {
+                const bool from_b = r * TPR + p >= pro.runs_a;   // (per lane: a wave's runs straddle the seam)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const float act = apply_prologue<DT, I8F_PRO_GELU_TANH>(v[r][j], 0.0f, 0.0f);
+                    v[r][j] = from_b ? act : v[r][j];
+                }
             }
             if constexpr (ROT) rotate_run16<DT>(v[r], s0, s1, s2);
 #pragma unroll
@@ -834,6 +851,7 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
     bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) && ((uintptr_t)q % 8 == 0);
     if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_NORM_MODULATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0 && (uintptr_t)pro.t % 16 == 0;
     if constexpr (PRO == I8F_PRO_SILU_GATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0;
+    if constexpr (PRO == I8F_PRO_CONCAT_GELU) aligned = aligned && (uintptr_t)pro.b % 16 == 0 && pro.ldb_bytes % 16 == 0;
     const int64_t nchunks = K / EPC;
     if constexpr (DT != I8F_F32) {
         const int64_t nruns = K / 16;
@@ -842,8 +860,9 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
             if constexpr (PRO != I8F_PRO_NORM_MODULATE) return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
         }
     }
-    // the normalising prologue exists where one wave holds the row: 16-bit rows of up to 4096 aligned elements
-    if constexpr (PRO == I8F_PRO_NORM_MODULATE) return I8F_ERR_UNSUPPORTED;
+    // the normalising prologue exists where one wave holds the row: 16-bit rows of up to 4096 aligned elements;
+    // the concatenating one where the row stays in registers: 16-bit rows of up to 16384 aligned elements
+    if constexpr (PRO == I8F_PRO_NORM_MODULATE || PRO == I8F_PRO_CONCAT_GELU) return I8F_ERR_UNSUPPORTED;
     else {
     if constexpr (PRO == I8F_PRO_NONE) {  // the chunked kernels have no prologue form: such shapes take the generic kernel
         if (aligned && nchunks <= 1024 * 8) {
@@ -871,6 +890,10 @@ int dispatch_rot(bool rot, const void *x, int64_t M, int64_t K, int64_t ldx, int
     case I8F_PRO_SILU_GATE:
         return rot ? dispatch<DT, true, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro)
                    : dispatch<DT, false, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro);
+    case I8F_PRO_CONCAT_GELU:
+        if constexpr (DT == I8F_F32) return I8F_ERR_UNSUPPORTED;
+        else return rot ? dispatch<DT, true, I8F_PRO_CONCAT_GELU>(x, M, K, ldx, q, scale, st, pro)
+                        : dispatch<DT, false, I8F_PRO_CONCAT_GELU>(x, M, K, ldx, q, scale, st, pro);
     case I8F_PRO_NORM_MODULATE:
         if constexpr (DT == I8F_F32) return I8F_ERR_UNSUPPORTED;
         else return rot ? dispatch<DT, true, I8F_PRO_NORM_MODULATE>(x, M, K, ldx, q, scale, st, pro)
@@ -995,6 +1018,28 @@ extern "C" int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64
     case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st, pro);
     default: return I8F_ERR_UNSUPPORTED;
     }
+}
+
+extern "C" int i8f_quant_rowwise_concat_gelu(const void *a, int dtype, int64_t M, int64_t Ka, int64_t lda, const void *b, int64_t Kb,
+                                             int64_t ldb, int rotate_block, int8_t *q, float *scale, void *stream) {
+    using namespace i8f;
+    if (M < 0 || Ka < 0 || Kb < 0 || !valid_dtype(dtype)) return I8F_ERR_INVALID;
+    if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
+    const int64_t K = Ka + Kb;
+    if (rotate_block && (Ka % rotate_block || Kb % rotate_block)) return I8F_ERR_INVALID;
+    if (M == 0) return I8F_OK;
+    if (!scale || lda < Ka || ldb < Kb || K == 0 || !q || (Ka > 0 && !a) || (Kb > 0 && !b)) return I8F_ERR_INVALID;
+    if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
+    // both parts in whole runs of 16 elements with 16-byte aligned rows
+    if (dtype == I8F_F32 || Ka % 16 || Kb % 16 || lda % 8 || ldb % 8 || K > 16 * 64 * 4 * 4) return I8F_ERR_UNSUPPORTED;
+    if (int rc = check_device()) return rc;
+    Prologue pro{I8F_PRO_CONCAT_GELU, nullptr, nullptr, 1, 0.0f, b, ldb * 2, (int)(Ka / 16)};
+    // (a part without elements: its pointer is never read, the other one stands in so that alignment checks pass)
+    const void *x = Ka > 0 ? a : b;
+    if (Kb == 0) pro.b = a;
+    hipStream_t st = (hipStream_t)stream;
+    const bool rot = rotate_block != 0;
+    return dtype == I8F_BF16 ? dispatch_rot<I8F_BF16>(rot, x, M, K, lda, q, scale, st, pro) : dispatch_rot<I8F_F16>(rot, x, M, K, lda, q, scale, st, pro);
 }
 
 extern "C" int i8f_rotate128(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, void *out, void *stream) {

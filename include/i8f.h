@@ -81,9 +81,12 @@ typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
  *                      dtype, then the product rounded to x's dtype, as torch's two eager kernels do
  *   I8F_PRO_NORM_MODULATE  (1 + s[k]) * layer_norm(x) + t[k] (no affine parameters); taken by
  *                      i8f_quant_rowwise_norm_modulate only, which carries the epsilon
+ *   I8F_PRO_CONCAT_GELU  cat(a, gelu(b, approximate="tanh")) along the row; taken by
+ *                      i8f_quant_rowwise_concat_gelu only, which carries the second tensor
  */
 typedef enum i8f_prologue {
-    I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2, I8F_PRO_SILU_GATE = 3, I8F_PRO_NORM_MODULATE = 4
+    I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2, I8F_PRO_SILU_GATE = 3, I8F_PRO_NORM_MODULATE = 4,
+    I8F_PRO_CONCAT_GELU = 5
 } i8f_prologue;
 
 /* Library version (I8F_VERSION of the build). */
@@ -174,6 +177,22 @@ int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64
                                     float eps, const void *mod_scale, const void *mod_shift,
                                     int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale,
                                     void *stream);
+
+/*
+ * The quantiser on the concatenation of two tensors along the row, the second through tanh-GELU:
+ *   z[m] = ( a[m, 0..Ka) , gelu(b[m, 0..Kb), approximate="tanh") )        then rotation, absmax and int8 over Ka + Kb
+ * the input of the second projection of a single-stream transformer block, linear2(cat(attn, gelu(mlp))): neither
+ * the activated tensor nor the concatenation is ever written to memory.  No counterpart in the reference's files:
+ * there both are the model's own torch operations in front of Linear.forward (int8_quant.py:703), fused by
+ * torch.compile into the quantiser's producer (README.md:4,56).  GELU as I8F_PRO_GELU_TANH (same tolerance); the
+ * a part is taken as it is, so with Kb == 0 the result is i8f_quant_rowwise's bit for bit.
+ *   a [M,Ka] (row stride lda), b [M,Kb] (row stride ldb) of dtype; q [M, Ka+Kb] contiguous; scale [M]
+ * I8F_ERR_UNSUPPORTED unless dtype is I8F_BF16 or I8F_F16, Ka % 16 == 0, Kb % 16 == 0, Ka + Kb <= 16384 and rows
+ * are 16-byte aligned: other callers concatenate themselves and use i8f_quant_rowwise.
+ */
+int i8f_quant_rowwise_concat_gelu(const void *a, int dtype, int64_t M, int64_t Ka, int64_t lda, const void *b,
+                                  int64_t Kb, int64_t ldb, int rotate_block, int8_t *q, float *scale,
+                                  void *stream);
 
 /*
  * One absmax scale for a whole tensor, then int8 quantisation with it.

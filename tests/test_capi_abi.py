@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 23
+    assert len(names) == 24
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -102,6 +102,15 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 200, 200, 1e-6, one, one, 4, 128, one, one, null) == INVALID
     assert lib.i8f_quant_rowwise_norm_modulate(null, L.BF16, 0, 256, 256, 1e-6, null, null, 1, 0, null, null, null) == 0
     assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, L.PRO_NORM_MODULATE, one, one, 4, 0, one, one, null) == INVALID  # needs its own entry point: it carries eps
+    # concatenating quantiser: negative widths, operands missing, a rotation block that would straddle the seam, binary32,
+    # widths that are not whole runs of 16, more than 16384 columns
+    assert lib.i8f_quant_rowwise_concat_gelu(one, L.BF16, 4, -16, 16, one, 16, 16, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_concat_gelu(one, L.BF16, 4, 16, 16, null, 16, 16, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_concat_gelu(one, L.BF16, 4, 64, 64, one, 128, 128, 128, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_concat_gelu(one, L.F32, 4, 16, 16, one, 16, 16, 0, one, one, null) == UNSUPPORTED
+    assert lib.i8f_quant_rowwise_concat_gelu(one, L.BF16, 4, 24, 24, one, 16, 16, 0, one, one, null) == UNSUPPORTED
+    assert lib.i8f_quant_rowwise_concat_gelu(one, L.BF16, 4, 8192, 8192, one, 8208, 8208, 0, one, one, null) == UNSUPPORTED
+    assert lib.i8f_quant_rowwise_concat_gelu(null, L.BF16, 0, 16, 16, null, 16, 16, 0, null, null, null) == 0
     # gated residual: a gate needs a positive row count per vector
     assert lib.i8f_linear_w8a8_gated(one, one, one, one, 1.0, 1, null, 0, one, 0, one, one, L.BF16, 4, 8, 16, 0, null, 0, null) == INVALID
     assert lib.i8f_linear_w8a8_gated(one, one, one, one, 1.0, 1, null, 0, one, 4, one, null, L.BF16, 4, 8, 16, 0, null, 0, null) == INVALID

@@ -224,6 +224,42 @@ def test_quant_rowwise_norm_modulate_refuses_rows_it_does_not_take(L, dev):
         L.quant_rowwise(torch.zeros(4, 256, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s[:, :256].float(), mod_shift=s[:, :256].float())
 
 
+@pytest.mark.parametrize("M,Ka,Kb,dt,rot", [
+    (64, 3072, 12288, torch.bfloat16, False), (33, 3072, 12288, torch.bfloat16, True), (10, 1024, 2048, torch.float16, False),
+    (7, 16, 48, torch.bfloat16, False), (12, 384, 128, torch.float16, True), (4608, 3072, 12288, torch.bfloat16, False),
+    (9, 3200, 800, torch.bfloat16, False),
+])
+def test_quant_rowwise_concat_gelu_prologue(L, dev, M, Ka, Kb, dt, rot):
+    """cat(a, gelu(b)) along the row inside the quantiser (i8f_quant_rowwise_concat_gelu; the input of linear2 of a
+    single-stream block) against the oracle's GELU on b, numpy's concatenation and the oracle's quantiser, and against
+    torch's gelu and cat on the device followed by the plain quantiser: the bar of the GELU prologue (scales within 2 ulp
+    of the dtype, int8 at most 1 apart, at least 99.9 % equal, 99 % with rotation).  The columns that come from a are
+    exact whenever the row's scale is; with an empty-handed GELU (b = 0) the whole result is the plain quantiser's."""
+    a = acts(M, Ka, dt)
+    b = (acts(M, Kb, dt).float() * 0.5).to(dt)
+    aa, code = O.from_torch(a)
+    z = np.concatenate([aa, O.prologue(O.from_torch(b)[0], code, O.PRO_GELU_TANH)], axis=1)
+    qo, so = O.quant_rowwise(z, code, 128 if rot else 0)
+    wide_a, wide_b = acts(M, Ka + 32, dt), None
+    q, s = L.quant_rowwise(a.to(dev), rotate=rot, prologue=L.PRO_CONCAT_GELU, mod_scale=b.to(dev))
+    assert q.shape == (M, Ka + Kb)
+    zt = torch.cat((a.to(dev), torch.nn.functional.gelu(b.to(dev), approximate="tanh")), -1)
+    q2, s2 = L.quant_rowwise(zt, rotate=rot)
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[dt]
+    for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+        d = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() <= (1e-2 if rot else 1e-3)
+        assert (np.abs(s.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
+    zero_b = torch.zeros(M, Kb, dtype=dt, device=dev)                       # gelu(0) = 0: nothing toleranced is left
+    q0, s0 = L.quant_rowwise(a.to(dev), rotate=rot, prologue=L.PRO_CONCAT_GELU, mod_scale=zero_b)
+    q1, s1 = L.quant_rowwise(torch.cat((a.to(dev), zero_b), -1), rotate=rot)
+    assert torch.equal(q0, q1) and torch.equal(s0, s1)
+    a_str = wide_a.to(dev)[:, :Ka]                                          # a row stride larger than the width
+    q3, s3 = L.quant_rowwise(a_str, rotate=rot, prologue=L.PRO_CONCAT_GELU, mod_scale=b.to(dev))
+    q4, s4 = L.quant_rowwise(a_str.contiguous(), rotate=rot, prologue=L.PRO_CONCAT_GELU, mod_scale=b.to(dev))
+    assert torch.equal(q3, q4) and torch.equal(s3, s4)
+
+
 TENSORWISE_CASES = [
     # shape, dtype
     ((3072, 3072), torch.bfloat16), ((3072, 3072), torch.float32), ((1, 1), torch.float32), ((7,), torch.float16),
