@@ -367,7 +367,25 @@ def extras(L, dev, quick=False):
                                     "plain_quant_median_us": round(t_p["median_us"], 2), "fused_gbs": round(hbytes / t_f["median_us"] / 1e3, 1),
                                     "plain_gbs": round(hbytes / t_p["median_us"] / 1e3, 1),
                                     "note": "config 1's down-projection input: the fused form never writes the 113 MB activated tensor"}
-    del hq
+    # the input of linear2 of a single-stream block, cat((attn [M,3072], gelu(mlp [M,12288])), -1): one launch that reads
+    # both operands and writes int8, against torch's gelu and cat kernels followed by the plain quantiser
+    Kc = K + 12288
+    cq = [torch.empty(M, Kc, dtype=torch.int8, device=dev) for _ in range(3)]
+
+    def concat_fused(i):
+        rc = lib.i8f_quant_rowwise_concat_gelu(ptr(xs[i]), L.BF16, M, K, K, ptr(hs[i]), 12288, 12288, 0, ptr(cq[i]), ptr(ss[i]), stream)
+        assert rc == 0, rc
+
+    def concat_unfused(i):
+        plain_call(torch.cat((xs[i], F.gelu(hs[i], approximate="tanh")), -1), cq[i], ss[i], Kc)
+
+    t_f = time_kernel(concat_fused, reps, sets=3, burst=3)
+    t_u = time_kernel(concat_unfused, reps, sets=3, burst=3)
+    cbytes = M * Kc * 3 + 4 * M
+    out["concat_gelu_quant_4608x3072+12288"] = {"fused_median_us": round(t_f["median_us"], 2), "torch_ops_then_quant_median_us": round(t_u["median_us"], 2),
+                                                "fused_gbs": round(cbytes / t_f["median_us"] / 1e3, 1),
+                                                "note": "neither the activated tensor nor the 141 MB concatenation is written"}
+    del hq, cq
     del xs, qs, ss, srcs, dsts, hs
 
     # config 4: stochastic LoRA merge (rank 32 rebuilt in the kernel, float noise) and the skinny GEMM

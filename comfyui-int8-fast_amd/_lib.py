@@ -191,7 +191,13 @@ def quant_rowwise_concat_gelu(a: torch.Tensor, b: torch.Tensor, rotate: bool = F
     -> (int8 [M, Ka+Kb], float32 [M,1])."""
     _dev(a, "a")
     _dev(b, "b")
-    if not concat_gelu_fusable(a, b):
+    if a.dim() > 2:   # leading dimensions are rows
+        a = a.reshape(-1, a.shape[-1])
+    if b.dim() > 2:
+        b = b.reshape(-1, b.shape[-1])
+    if a.dim() == 2 and b.dim() == 2 and not concat_gelu_fusable(a, b):   # rows that are not contiguous or aligned: copies
+        a, b = a.contiguous(), b.contiguous()
+    if a.dim() != 2 or b.dim() != 2 or not concat_gelu_fusable(a, b):
         raise ValueError("these tensors have no fused concatenation (see concat_gelu_fusable)")
     M, Ka = a.shape
     Kb = b.shape[1]

@@ -180,6 +180,26 @@ def _match_gelu(node):
     return node.args[0] if approx == "tanh" else None
 
 
+def _match_concat_gelu(node):
+    """cat((a, gelu(b, approximate="tanh")), dim=-1) with a, b of one 16-bit dtype and equal leading dimensions, widths
+    in multiples of 16 that add up to at most 16384, the activated tensor used nowhere else -> (a, b) nodes."""
+    if not (_is_call(node, torch.cat, torch.concat, torch.concatenate) and len(node.users) == 1):
+        return None
+    parts = node.args[0] if node.args else node.kwargs.get("tensors")
+    dim = node.args[1] if len(node.args) > 1 else node.kwargs.get("dim", 0)
+    if not isinstance(parts, (list, tuple)) or len(parts) != 2 or not all(isinstance(p, torch.fx.Node) for p in parts):
+        return None
+    a, act = parts
+    b = _match_gelu(act)
+    va, vb = _meta_val(a), _meta_val(b) if b is not None else None
+    if va is None or vb is None or dim not in (-1, len(va.shape) - 1):
+        return None
+    if va.dtype != vb.dtype or va.dtype not in (torch.bfloat16, torch.float16) or tuple(va.shape[:-1]) != tuple(vb.shape[:-1]) or len(va.shape) < 2:
+        return None
+    ka, kb = int(va.shape[-1]), int(vb.shape[-1])
+    return (a, b) if ka % 16 == 0 and kb % 16 == 0 and ka > 0 and kb > 0 and ka + kb <= 16384 else None
+
+
 def _match_silu_gate(node):
     """silu(a) * b in either operand order (a, b of one shape and dtype by the traced metadata) -> (a, b) nodes."""
     if not (_is_call(node, operator.mul, torch.mul) and len(node.users) == 1 and len(node.args) == 2):
@@ -257,8 +277,9 @@ def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
 
 
 def fuse_prologues(gm: torch.fx.GraphModule) -> int:
-    """Rewrite int8_linear(gelu_tanh(h)), int8_linear((1 + s) * h + t), int8_linear((1 + s) * layer_norm(h) + t) and
-    int8_linear(silu(h) * g) (no dynamic-LoRA addend, producers used nowhere else) into int8_linear_prologue(h, ...).
+    """Rewrite int8_linear(gelu_tanh(h)), int8_linear((1 + s) * h + t), int8_linear((1 + s) * layer_norm(h) + t),
+    int8_linear(silu(h) * g) and int8_linear(cat((a, gelu_tanh(b)), -1)) (no dynamic-LoRA addend, producers used nowhere
+    else) into int8_linear_prologue(h, ...).
     Returns the number of layers rewritten."""
     n_fused = 0
     targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
@@ -282,6 +303,7 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         else:
             m = _match_modulate(src)
             g = _match_silu_gate(src) if m is None else None
+            c = _match_concat_gelu(src) if m is None and g is None else None
             if m is not None and _vectors_broadcast_over_tokens(*m):
                 new_args = (m[0], _lib.PRO_MODULATE, m[1], m[2])
                 ln = _match_plain_layer_norm(m[0])   # the modulated tensor is a LayerNorm without affine: that goes in too
@@ -289,13 +311,21 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
                     new_args, eps = (ln[0], _lib.PRO_NORM_MODULATE, m[1], m[2]), ln[1]
             elif g is not None:
                 new_args = (g[0], _lib.PRO_SILU_GATE, g[1], None)
+            elif c is not None and not (rotate and (_meta_shape(c[0])[-1] % 128 or _meta_shape(c[1])[-1] % 128)):
+                new_args = (c[0], _lib.PRO_CONCAT_GELU, c[1], None)
         if new_args is None:
             continue
         # The fused operator returns the leading shape of h, the original one that of x_in: the same when nothing
         # sat between them; a layer that flattened h to 2-D gets its 2-D result back by a reshape; anything else
         # (a direct caller with another regrouping of the rows) is left alone.
         h_shape = _meta_shape(new_args[0])
-        if h_shape is None or h_shape[-1] != x_shape[-1]:
+        if h_shape is None:
+            continue
+        if new_args[1] == _lib.PRO_CONCAT_GELU:   # the layer's input is wider than h by the second tensor: compare the rows
+            if h_shape[-1] + _meta_shape(new_args[2])[-1] != x_shape[-1]:
+                continue
+            h_shape = (*h_shape[:-1], x_shape[-1])
+        if h_shape[-1] != x_shape[-1]:
             continue
         if h_shape != x_shape and len(x_shape) != 2:
             continue

@@ -458,7 +458,8 @@ class Int8TensorwiseOps(manual_cast):
             operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, _lib.PRO_MODULATE with
             (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension, _lib.PRO_NORM_MODULATE with
             the same modulation of layer_norm(x, eps) (no affine parameters: the whole adaLN producer of a DiT
-            block), or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
+            block), _lib.PRO_CONCAT_GELU with cat((x, gelu(mod_scale)), -1), the input of the second projection of a
+            single-stream block, or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
             path then applies inside its quantiser instead of in passes of their own (under torch.compile the graph
             rewrite of compile_ops does this without the caller's help).  `gate` / `residual` name what the caller would
             apply to the result: forward(h, gate=g, residual=x) returns x + g * linear(h), the gated residual of an
@@ -484,6 +485,13 @@ class Int8TensorwiseOps(manual_cast):
                 rows = x.numel() // max(1, x.shape[-1])
                 fusable = (self._is_quantized and rows > SMALL_BATCH_ROWS and self.lora_A is None
                            and not torch.compiler.is_compiling())
+                if fusable and prologue == _lib.PRO_CONCAT_GELU:   # x followed by gelu(mod_scale) along the feature dimension
+                    fusable = (isinstance(mod_scale, Tensor) and mod_scale.shape[:-1] == x.shape[:-1]
+                               and x.shape[-1] + mod_scale.shape[-1] == self.weight.shape[1]
+                               and _lib.concat_gelu_fusable(x.reshape(-1, x.shape[-1]), mod_scale.reshape(-1, mod_scale.shape[-1]))
+                               and not (getattr(self, "_use_quarot", False) and (x.shape[-1] % 128 or mod_scale.shape[-1] % 128)))
+                    if fusable:
+                        mod_scale = mod_scale.reshape(-1, mod_scale.shape[-1])
                 if fusable and prologue == _lib.PRO_SILU_GATE:   # the gate operand has x's shape and dtype, or torch does it
                     fusable = isinstance(mod_scale, Tensor) and mod_scale.shape == x.shape and mod_scale.dtype == x.dtype
                 if fusable and prologue in (_lib.PRO_MODULATE, _lib.PRO_NORM_MODULATE):
@@ -497,6 +505,8 @@ class Int8TensorwiseOps(manual_cast):
                 if not fusable:   # every other path takes the operation as torch would have applied it
                     if prologue == _lib.PRO_GELU_TANH:
                         x = F.gelu(x, approximate="tanh")
+                    elif prologue == _lib.PRO_CONCAT_GELU:
+                        x = torch.cat((x, F.gelu(mod_scale, approximate="tanh")), -1)
                     elif prologue == _lib.PRO_SILU_GATE:
                         x = F.silu(x) * mod_scale
                     else:

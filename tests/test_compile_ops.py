@@ -241,6 +241,41 @@ def test_graph_rewrite_moves_layer_norm_and_modulation_into_the_quantiser(pkg):
         assert node.args[1] == pkg._lib.PRO_MODULATE and ln_left
 
 
+def test_graph_rewrite_moves_concatenation_and_gelu_into_the_quantiser(pkg):
+    """linear2(cat((attn, gelu(mlp)), -1)), the second projection of a single-stream block: both producers become the
+    layer's prologue; a concatenation along another dimension, of three tensors, or with an exact GELU stays torch's."""
+    g = torch.Generator().manual_seed(15)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Single(torch.nn.Module):
+        def __init__(self, form):
+            super().__init__()
+            self.linear2, self.form = lin(128, 128 + 512 if form != 2 else 128 + 512 + 128), form
+
+        def forward(self, attn, mlp):
+            if self.form == 0:
+                z = torch.cat((attn, F.gelu(mlp, approximate="tanh")), 2)
+            elif self.form == 1:
+                z = torch.cat((attn, F.gelu(mlp)), -1)                       # exact GELU
+            else:
+                z = torch.cat((attn, F.gelu(mlp, approximate="tanh"), attn), -1)
+            return self.linear2(z)
+
+    attn, mlp = torch.randn(2, 24, 128).bfloat16(), torch.randn(2, 24, 512).bfloat16()
+    for form, fused in ((0, 1), (1, 0), (2, 0)):
+        gm = torch._dynamo.export(Single(form))(attn, mlp).graph_module
+        assert pkg.compile_ops.fuse_prologues(gm) == fused
+        nodes = [n for n in gm.graph.nodes if n.op == "call_function" and "int8_linear_prologue" in str(n.target)]
+        assert len(nodes) == fused
+        if fused:
+            assert nodes[0].args[1] == pkg._lib.PRO_CONCAT_GELU
+            assert not any(n.target in (torch.cat, F.gelu) for n in gm.graph.nodes if n.op == "call_function")
+
+
 def test_graph_rewrite_moves_the_gated_residual_into_the_epilogue(pkg):
     """x + gate * proj(h), the residual update of an adaLN-Zero block: multiplication and addition become the layer's
     epilogue (in any operand order); the gate alone and the residual alone are taken too; a gate of another dtype, a
@@ -447,6 +482,53 @@ def test_compiled_adaln_zero_block_equals_eager_bit_for_bit(pkg, dev):
     assert torch.equal(got, want)
     loose = m(x, sc, sh, gate)                           # torch's LayerNorm, modulation, gelu, gate and residual around the layers
     assert (got.float() - loose.float()).abs().max().item() <= 2.0**-6 * loose.float().abs().max().item()
+
+
+@pytest.mark.gpu
+def test_compiled_single_stream_block_equals_eager_bit_for_bit(pkg, dev):
+    """x + gate * linear2(cat((a, gelu(mlp)), -1)) with a and mlp split from linear1's output, the shape of a
+    single-stream block: the split halves reach the quantiser as strided views, neither the activated tensor nor the
+    concatenation exists, the gated residual sits in linear2's epilogue; equal to the eager fused forward calls and
+    within rounding of torch's operations around the layers."""
+    g = torch.Generator().manual_seed(16)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+
+    class Single(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear1, self.linear2 = lin(256 + 512, 256), lin(256, 256 + 512)
+
+        def forward(self, x, gate):
+            a, mlp = torch.split(self.linear1(x), [256, 512], dim=-1)
+            return x + gate * self.linear2(torch.cat((a, F.gelu(mlp, approximate="tanh")), 2))
+
+    m = Single().to(dev)
+    x = torch.randn(2, 40, 256, generator=g).bfloat16().to(dev)
+    gate = (torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev)
+    seen = []
+
+    def counting(gm, inputs):
+        calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum("int8_linear_prologue" in str(n.target) for n in calls),
+                     sum(n.kwargs.get("gate") is not None and n.kwargs.get("addend") is not None for n in calls),
+                     sum(n.target in (operator.mul, operator.add, torch.mul, torch.add, torch.cat) or "gelu" in str(n.target) for n in calls)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x, gate)
+    assert seen == [(1, 1, 0)]
+    a, mlp = torch.split(m.linear1(x), [256, 512], dim=-1)
+    want = m.linear2(a, prologue=pkg._lib.PRO_CONCAT_GELU, mod_scale=mlp, gate=gate, residual=x)
+    assert torch.equal(got, want)
+    loose = m(x, gate)
+    assert (got.float() - loose.float()).abs().max().item() <= 2.0**-6 * loose.float().abs().max().item()
+    few = m.linear2(a[:, :4], prologue=pkg._lib.PRO_CONCAT_GELU, mod_scale=mlp[:, :4])     # 8 rows: torch concatenates, the small-batch path runs
+    ref = m.linear2(torch.cat((a[:, :4], F.gelu(mlp[:, :4], approximate="tanh")), -1))
+    assert torch.equal(few, ref)
 
 
 @pytest.mark.gpu

@@ -280,6 +280,11 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
         a = lin(x, prologue=L.PRO_SILU_GATE, mod_scale=gate)
         b = lin(F.silu(x) * gate)
         assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
+        wide = x[..., :256].contiguous()                                       # cat((a, gelu(b)), -1): 256 + 128 features
+        tail = torch.randn(2, 20, 128, generator=g).bfloat16().to(dev)
+        a = lin(wide, prologue=L.PRO_CONCAT_GELU, mod_scale=tail)
+        b = lin(torch.cat((wide, F.gelu(tail, approximate="tanh")), -1))
+        assert a.shape == (2, 20, 96) and (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
         a = lin(x, prologue=L.PRO_NORM_MODULATE, mod_scale=sc, mod_shift=sh, eps=1e-6)   # the whole adaLN producer
         b = lin((1 + sc) * F.layer_norm(x, (384,), eps=1e-6) + sh)
         assert a.shape == (2, 20, 96) and (a.float() - b.float()).abs().max() <= 2.0**-6 * b.float().abs().max()
