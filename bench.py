@@ -367,6 +367,32 @@ def extras(L, dev, quick=False):
                                     "plain_quant_median_us": round(t_p["median_us"], 2), "fused_gbs": round(hbytes / t_f["median_us"] / 1e3, 1),
                                     "plain_gbs": round(hbytes / t_p["median_us"] / 1e3, 1),
                                     "note": "config 1's down-projection input: the fused form never writes the 113 MB activated tensor"}
+    t_f = time_kernel(lambda i: fused_call(i, L.PRO_GELU_ERF, hs, hq, ss, 12288), reps, sets=3, burst=3)
+    t_u = time_kernel(lambda i: plain_call(F.gelu(hs[i]), hq[i], ss[i], 12288), reps, sets=3, burst=3)
+    out["gelu_erf_quant_4608x12288"] = {"fused_median_us": round(t_f["median_us"], 2), "torch_gelu_then_quant_median_us": round(t_u["median_us"], 2),
+                                        "fused_gbs": round(hbytes / t_f["median_us"] / 1e3, 1),
+                                        "note": "GELU in its exact form (erf), 13 vector + 2 transcendental instructions per element"}
+
+    # RMSNorm with its weight and the scale-only modulation behind it (z-image's modulate(norm(x), scale), width 3840)
+    Kz = 3840
+    zs = [torch.randn(M, Kz, device=dev).bfloat16() for _ in range(sets)]
+    zq = [torch.empty(M, Kz, dtype=torch.int8, device=dev) for _ in range(sets)]
+    nw, zsc = (torch.randn(Kz, device=dev) * 0.2 + 1).bfloat16(), (torch.randn(1, Kz, device=dev) * 0.3).bfloat16()
+
+    def rms_fused(i):
+        rc = lib.i8f_quant_rowwise_rms_norm(ptr(zs[i]), L.BF16, M, Kz, Kz, 1e-5, ptr(nw), ptr(zsc), None, M, 0, ptr(zq[i]), ptr(ss[i]), stream)
+        assert rc == 0, rc
+
+    def rms_unfused(i):
+        plain_call(F.rms_norm(zs[i], (Kz,), nw, 1e-5) * (1 + zsc), zq[i], ss[i], Kz)
+
+    t_f = time_kernel(rms_fused, reps, sets=sets, burst=sets)
+    t_u = time_kernel(rms_unfused, reps, sets=sets, burst=sets)
+    out["rms_norm_modulate_quant_4608x3840"] = {"fused_median_us": round(t_f["median_us"], 2), "torch_ops_then_quant_median_us": round(t_u["median_us"], 2),
+                                                "fused_gbs": round((M * Kz * 3 + 4 * M) / t_f["median_us"] / 1e3, 1),
+                                                "note": "rms_norm(x, w) * (1 + scale) + quantise: one launch against torch's three kernels and the quantiser"}
+    del zs, zq
+
     # the input of linear2 of a single-stream block, cat((attn [M,3072], gelu(mlp [M,12288])), -1): one launch that reads
     # both operands and writes int8, against torch's gelu and cat kernels followed by the plain quantiser
     Kc = K + 12288

@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libi8f_gfx950.so")
 BF16, F16, F32 = 0, 1, 2
 SCALE_TENSOR, SCALE_ROW = 0, 1
 EPI_TORCH, EPI_FUSED = 0, 1
-PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE, PRO_CONCAT_GELU = 0, 1, 2, 3, 4, 5
+PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE, PRO_CONCAT_GELU, PRO_GELU_ERF, PRO_RMS_NORM = 0, 1, 2, 3, 4, 5, 6, 7
 
 _DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
 
@@ -56,6 +56,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_quant_rowwise_grouped.argtypes = [vp, i32, i32, i64, i32, vp]
     L.i8f_quant_rowwise_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, i32, vp, vp, vp]
     L.i8f_quant_rowwise_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, i32, vp, vp, vp]
+    L.i8f_quant_rowwise_rms_norm.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, vp, i64, i32, vp, vp, vp]
     L.i8f_quant_rowwise_concat_gelu.argtypes = [vp, i32, i64, i64, i64, vp, i64, i64, i32, vp, vp, vp]
     L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
     L.i8f_quant_tensorwise_workspace_bytes.restype = i64
@@ -75,7 +76,7 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
-    for name in ("i8f_quant_rowwise_concat_gelu", "i8f_linear_w8a8_gated", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
+    for name in ("i8f_quant_rowwise_concat_gelu", "i8f_quant_rowwise_rms_norm", "i8f_linear_w8a8_gated", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
                  "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
@@ -85,6 +86,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_rowwise_concat_gelu",
+    "i8f_quant_rowwise_rms_norm",
     "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_gated", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
@@ -219,15 +221,57 @@ def norm_modulate_fusable(x: torch.Tensor) -> bool:
             and x.stride(1) == 1 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0)
 
 
-def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NONE, mod_scale=None, mod_shift=None, eps: float = 1e-6):
+def quant_rowwise_rms_norm(x: torch.Tensor, eps: float = 1e-6, weight=None, mod_scale=None, mod_shift=None, rotate: bool = False):
+    """quant_rowwise of rms_norm(x, weight, eps) [* (1 + mod_scale)] [+ mod_shift] with no intermediate tensor in memory:
+    the producer of the projections of blocks that normalise with an RMSNorm.  x [M,K] as norm_modulate_fusable
+    describes; weight [K]; mod_scale / mod_shift [V,K] (or [K]), M // V consecutive rows to a vector; each optional."""
+    _dev(x, "x")
+    if not norm_modulate_fusable(x):
+        raise ValueError("the normalising quantiser takes contiguous 16-bit rows of at most 4096 elements in multiples of 16 "
+                         "(see norm_modulate_fusable); normalise with torch")
+    M, K = x.shape
+    if rotate and K % 128:
+        raise ValueError(f"rotation needs K % 128 == 0, got K={K}")
+    if weight is not None:
+        _dev(weight, "weight")
+        if weight.dtype != x.dtype or weight.device != x.device or weight.numel() != K:
+            raise ValueError(f"weight must be [{K}] of {x.dtype} on {x.device}")
+        weight = weight.reshape(K).contiguous()
+    rows_per_vec, vecs = 1, []
+    for name, v in (("mod_scale", mod_scale), ("mod_shift", mod_shift)):
+        if v is not None:
+            _dev(v, name)
+            if v.dtype != x.dtype or v.device != x.device or v.numel() % K or v.shape[-1] != K:
+                raise ValueError(f"{name} must be [V,{K}] of {x.dtype} on {x.device}")
+            v = v.reshape(-1, K).contiguous()
+            if v.shape[0] == 0 or M % v.shape[0] or (vecs and vecs[0] is not None and vecs[0].shape[0] != v.shape[0]):
+                raise ValueError(f"{M} rows do not split evenly over the modulation vectors")
+            rows_per_vec = max(1, M // v.shape[0])
+        vecs.append(v)
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    s = torch.empty((M, 1), dtype=torch.float32, device=x.device)
+    with _on(x.device):
+        _check(lib().i8f_quant_rowwise_rms_norm(_ptr(x), dtype_code(x.dtype), M, K, x.stride(0) if M > 1 else K, float(eps),
+                                                _ptr(weight) if weight is not None else None, *(None if v is None else _ptr(v) for v in vecs),
+                                                rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s), _stream(x)),
+               "i8f_quant_rowwise_rms_norm")
+    return q, s
+
+
+def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NONE, mod_scale=None, mod_shift=None, eps: float = 1e-6,
+                  norm_weight=None):
     """x [M,K] (bf16/fp16/fp32, cuda) -> (int8 [M,K], float32 [M,1]); rotate=True applies the 128-block Hadamard first.
     prologue applies an elementwise operation while the rows are read: PRO_GELU_TANH, or PRO_MODULATE with
     mod_scale / mod_shift of x's dtype, [V,K] (or [K]): (1 + mod_scale) * x + mod_shift, M // V consecutive rows
     to a vector, or PRO_SILU_GATE with the gate operand as mod_scale (x's dtype, [M,K], or [V,K] like the vectors
     above): silu(x) * mod_scale, or PRO_NORM_MODULATE: the modulation applied to layer_norm(x, eps) without affine
     parameters (see norm_modulate_fusable for the rows it takes), or PRO_CONCAT_GELU with a second tensor [M,Kb] as
-    mod_scale: cat((x, gelu(mod_scale)), -1) (see quant_rowwise_concat_gelu)."""
+    mod_scale: cat((x, gelu(mod_scale)), -1) (see quant_rowwise_concat_gelu), or PRO_GELU_ERF, GELU in its exact form, or
+    PRO_RMS_NORM: rms_norm(x, norm_weight, eps), then the modulation's operations where mod_scale / mod_shift are given
+    (see quant_rowwise_rms_norm)."""
     _dev(x, "x")
+    if prologue == PRO_RMS_NORM:
+        return quant_rowwise_rms_norm(x, eps, norm_weight, mod_scale, mod_shift, rotate=rotate)
     if prologue == PRO_CONCAT_GELU:   # x followed by gelu(mod_scale) along the row
         return quant_rowwise_concat_gelu(x, mod_scale, rotate=rotate)
     x = _rows(x, "x")
@@ -255,7 +299,7 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
         if mod_shift.shape[0] != V or V == 0 or M % V:
             raise ValueError(f"{M} rows do not split evenly over {V} modulation vectors")
         rows_per_vec = max(1, M // V)
-    elif prologue not in (PRO_NONE, PRO_GELU_TANH):
+    elif prologue not in (PRO_NONE, PRO_GELU_TANH, PRO_GELU_ERF):
         raise ValueError(f"unknown prologue {prologue}")
     else:
         mod_scale = mod_shift = None

@@ -111,21 +111,24 @@ def _(x, weight, weight_scale, weight_scale_value, bias, rotate):
 def int8_linear_prologue(x: Tensor, prologue: int, mod_scale: Optional[Tensor], mod_shift: Optional[Tensor],
                          weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
                          bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int, eps: float = 1e-6,
-                         addend: Optional[Tensor] = None, gate: Optional[Tensor] = None) -> Tensor:
-    """int8_linear on prologue(x): tanh-GELU, (1 + mod_scale) * x + mod_shift with one pair of vectors per
-    group of consecutive rows (PRO_NORM_MODULATE: of layer_norm(x, eps) without affine parameters), or
-    silu(x) * mod_scale with a gate operand of x's shape; the transformed activations exist only inside the quantiser."""
+                         addend: Optional[Tensor] = None, gate: Optional[Tensor] = None,
+                         norm_weight: Optional[Tensor] = None) -> Tensor:
+    """int8_linear on prologue(x): GELU (tanh or exact form), (1 + mod_scale) * x + mod_shift with one pair of vectors per
+    group of consecutive rows (PRO_NORM_MODULATE: of layer_norm(x, eps) without affine parameters; PRO_RMS_NORM: of
+    rms_norm(x, norm_weight, eps), scale and shift each optional), silu(x) * mod_scale with a gate operand of x's shape,
+    or cat((x, gelu(mod_scale)), -1); the transformed activations exist only inside the quantiser."""
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
-                              mod_shift=mod_shift, eps=eps)
+                              mod_shift=mod_shift, eps=eps, norm_weight=norm_weight)
     y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order, addend=addend, gate=gate)
     return y.reshape(*lead, weight.shape[0])
 
 
 @int8_linear_prologue.register_fake
 def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, eps=1e-6,
-      addend=None, gate=None):
-    return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
+      addend=None, gate=None, norm_weight=None):
+    width = weight.shape[0]
+    return x.new_empty((*x.shape[:-1], width), dtype=compute_dtype)
 
 
 OPS = ("quantize_rowwise", "rotate128", "linear_w8a8", "int8_linear", "linear_w8a16_small_m", "int8_linear_prologue")
@@ -180,6 +183,14 @@ def _match_gelu(node):
     return node.args[0] if approx == "tanh" else None
 
 
+def _match_gelu_erf(node):
+    """gelu(h) in its exact form (approximate="none", the default), used nowhere else -> h."""
+    if not (_is_call(node, torch.nn.functional.gelu, torch._C._nn.gelu) and len(node.users) == 1):
+        return None
+    approx = node.kwargs.get("approximate", node.args[1] if len(node.args) > 1 else "none")
+    return node.args[0] if approx == "none" else None
+
+
 def _match_concat_gelu(node):
     """cat((a, gelu(b, approximate="tanh")), dim=-1) with a, b of one 16-bit dtype and equal leading dimensions, widths
     in multiples of 16 that add up to at most 16384, the activated tensor used nowhere else -> (a, b) nodes."""
@@ -231,6 +242,42 @@ def _match_modulate(node):
     return None
 
 
+def _match_scale_only(node):
+    """(1 + scale) * x in either operand order -> (x, scale) nodes."""
+    if not (_is_call(node, operator.mul, torch.mul) and len(node.users) == 1 and len(node.args) == 2):
+        return None
+    for gain, x in (node.args, node.args[::-1]):
+        if isinstance(gain, torch.fx.Node) and _is_call(gain, operator.add, torch.add) and len(gain.users) == 1 and len(gain.args) == 2:
+            for one, scale in (gain.args, gain.args[::-1]):
+                if isinstance(one, (int, float)) and one == 1 and isinstance(scale, torch.fx.Node) and isinstance(x, torch.fx.Node):
+                    return x, scale
+    return None
+
+
+def _match_rms_norm(node):
+    """rms_norm(h, (K,), weight, eps) over the last dimension, used nowhere else, on 16-bit rows of a width the
+    normalising quantiser takes, the weight absent or [K] of h's dtype -> (h, weight or None, eps)."""
+    if not (_is_call(node, torch.nn.functional.rms_norm, torch.rms_norm) and len(node.users) == 1):
+        return None
+    a = dict(zip(("input", "normalized_shape", "weight", "eps"), node.args))
+    a.update(node.kwargs)
+    h, shape, w = a.get("input"), a.get("normalized_shape"), a.get("weight")
+    v = _meta_val(h)
+    if v is None or v.dtype not in (torch.bfloat16, torch.float16) or len(v.shape) < 2:
+        return None
+    K = int(v.shape[-1])
+    if tuple(int(d) for d in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,))) != (K,) or K % 16 or K > 4096:
+        return None
+    if w is not None:
+        vw = _meta_val(w)
+        if vw is None or vw.dtype != v.dtype or tuple(vw.shape) != (K,):
+            return None
+    eps = a.get("eps")
+    if eps is None:
+        eps = torch.finfo(v.dtype).eps      # what torch takes when none is given
+    return (h, w, float(eps)) if isinstance(eps, (int, float)) else None
+
+
 def _match_plain_layer_norm(node):
     """layer_norm(h, (K,), eps=...) over the last dimension without weight and bias, used nowhere else, on 16-bit rows
     of a width the normalising quantiser takes -> (h, eps)."""
@@ -277,9 +324,9 @@ def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
 
 
 def fuse_prologues(gm: torch.fx.GraphModule) -> int:
-    """Rewrite int8_linear(gelu_tanh(h)), int8_linear((1 + s) * h + t), int8_linear((1 + s) * layer_norm(h) + t),
-    int8_linear(silu(h) * g) and int8_linear(cat((a, gelu_tanh(b)), -1)) (no dynamic-LoRA addend, producers used nowhere
-    else) into int8_linear_prologue(h, ...).
+    """Rewrite int8_linear(gelu(h)) (either form), int8_linear((1 + s) * h + t), int8_linear((1 + s) * layer_norm(h) + t),
+    int8_linear(rms_norm(h, w) [* (1 + s)] [+ t]), int8_linear(silu(h) * g) and int8_linear(cat((a, gelu_tanh(b)), -1))
+    (no dynamic-LoRA addend, producers used nowhere else) into int8_linear_prologue(h, ...).
     Returns the number of layers rewritten."""
     n_fused = 0
     targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
@@ -297,9 +344,19 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         if x_shape is None:
             continue
         h = _match_gelu(src)
-        new_args, eps = None, 1e-6
+        new_args, eps, norm_w = None, 1e-6, None
         if h is not None:
             new_args = (h, _lib.PRO_GELU_TANH, None, None)
+        elif _match_gelu_erf(src) is not None:
+            new_args = (_match_gelu_erf(src), _lib.PRO_GELU_ERF, None, None)
+        elif _match_rms_norm(src) is not None:                       # the norm alone
+            r = _match_rms_norm(src)
+            new_args, eps, norm_w = (r[0], _lib.PRO_RMS_NORM, None, None), r[2], r[1]
+        elif _match_scale_only(src) is not None and _match_rms_norm(_match_scale_only(src)[0]) is not None:
+            y, sc = _match_scale_only(src)                           # modulate(norm(x), scale) = norm(x) * (1 + scale)
+            r = _match_rms_norm(y)
+            if _vectors_broadcast_over_tokens(r[0], sc, sc):
+                new_args, eps, norm_w = (r[0], _lib.PRO_RMS_NORM, sc, None), r[2], r[1]
         else:
             m = _match_modulate(src)
             g = _match_silu_gate(src) if m is None else None
@@ -307,8 +364,11 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
             if m is not None and _vectors_broadcast_over_tokens(*m):
                 new_args = (m[0], _lib.PRO_MODULATE, m[1], m[2])
                 ln = _match_plain_layer_norm(m[0])   # the modulated tensor is a LayerNorm without affine: that goes in too
+                rn = _match_rms_norm(m[0]) if ln is None else None
                 if ln is not None:
                     new_args, eps = (ln[0], _lib.PRO_NORM_MODULATE, m[1], m[2]), ln[1]
+                elif rn is not None and _vectors_broadcast_over_tokens(rn[0], m[1], m[2]):   # or an RMSNorm
+                    new_args, eps, norm_w = (rn[0], _lib.PRO_RMS_NORM, m[1], m[2]), rn[2], rn[1]
             elif g is not None:
                 new_args = (g[0], _lib.PRO_SILU_GATE, g[1], None)
             elif c is not None and not (rotate and (_meta_shape(c[0])[-1] % 128 or _meta_shape(c[1])[-1] % 128)):
@@ -331,7 +391,8 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
             continue
         with gm.graph.inserting_before(node):
             fused = gm.graph.call_function(torch.ops.i8f.int8_linear_prologue,
-                                           (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order, eps))
+                                           (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order, eps),
+                                           {} if norm_w is None else {"norm_weight": norm_w})
             n_out, old = _out_features(weight), _meta_val(node)
             if old is not None:   # shapes for the passes that follow (the epilogue rewrite reads them)
                 _record(fused, (*h_shape[:-1], n_out), old.dtype)

@@ -46,6 +46,9 @@ struct Elem {
 //                                                     evaluated in binary32 and rounded once to x's dtype,
 //                                                     tanh(u) = 1 - 2 / (exp(2u) + 1) on the hardware's
 //                                                     exp2 and reciprocal (a few binary32 ulp).
+//   I8F_PRO_GELU_ERF   v = gelu(x), exact form        0.5 x (1 + erf(x / sqrt(2))) = x Phi(x), in binary32, rounded once;
+//                                                     erfc by a rational-exponential form good to 1.5e-7 of Phi.
+//   I8F_PRO_RMS_NORM   v = x / rms(x) * w[k], then optionally (1 + s[k]) * v and + t[k]; w, s, t may each be absent.
 struct Prologue {
     int kind;
     const void *s, *t;       // modulation vectors (MODULATE, NORM_MODULATE), gate operand (SILU_GATE)
@@ -55,6 +58,7 @@ struct Prologue {
     const void *b;
     int64_t ldb_bytes;
     int runs_a;
+    const void *w;           // RMS_NORM: the norm's weight vector [K] (or nullptr)
 };
 
 // the sum over the wave in a fixed order (the same in every lane)
@@ -78,6 +82,21 @@ __device__ __forceinline__ float silu_f32(float x) {
     return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
+// x Phi(x) with Phi(x) = 1 - erfc(|x| / sqrt 2) / 2 for x >= 0 and erfc(|x| / sqrt 2) / 2 below, so that the negative tail
+// is formed without cancellation; erfc(z) = t (a1 + t (a2 + t (a3 + t (a4 + t a5)))) exp(-z^2), t = 1 / (1 + p z)
+// (Abramowitz & Stegun 7.1.26, |error| <= 1.5e-7), on the hardware's reciprocal and exp2; the halves are folded into
+// the coefficients.  Thirteen vector instructions and the two transcendental ones.
+__device__ __forceinline__ float gelu_erf_f32(float x) {
+    const float z = fabsf(x) * 0.7071067811865476f;
+    const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(z, 0.3275911f, 1.0f));
+    float pl = __builtin_fmaf(t, 0.5307027145f, -0.7265760135f);
+    pl = __builtin_fmaf(t, pl, 0.7107068705f);
+    pl = __builtin_fmaf(t, pl, -0.142248368f);
+    pl = __builtin_fmaf(t, pl, 0.127414796f);
+    const float h = pl * t * __builtin_amdgcn_exp2f(z * z * -1.4426950408889634f);   // erfc(z) / 2
+    return x * (x >= 0.0f ? 1.0f - h : h);
+}
+
 template <int DT, int PRO>
 __device__ __forceinline__ float apply_prologue(float x, float s, float t) {
     if constexpr (PRO == I8F_PRO_SILU_GATE) {
@@ -88,6 +107,8 @@ __device__ __forceinline__ float apply_prologue(float x, float s, float t) {
         return round_to_dtype<DT>(b + t);
     } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
         return round_to_dtype<DT>(gelu_tanh_f32(x));
+    } else if constexpr (PRO == I8F_PRO_GELU_ERF) {
+        return round_to_dtype<DT>(gelu_erf_f32(x));
     } else {
         return x;
     }
@@ -481,7 +502,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
         float v[RUNS][16];
         float amax = 0.0f;
         [[maybe_unused]] int64_t vrow = 0;  // the row's pair of modulation vectors (M < 2^31: a 32-bit division)
-        if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_SILU_GATE || PRO == I8F_PRO_NORM_MODULATE)
+        if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_SILU_GATE || PRO == I8F_PRO_NORM_MODULATE || PRO == I8F_PRO_RMS_NORM)
             vrow = (uint32_t)(FULL || m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
         if constexpr (PRO == I8F_PRO_NORM_MODULATE) {
             // LayerNorm without affine over the row, which this wave holds whole: mean, then the variance of the
@@ -512,9 +533,52 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
 #pragma unroll
                 for (int j = 0; j < 16; ++j) v[r][j] = round_to_dtype<DT>(v[r][j] * rstd);
         }
+        if constexpr (PRO == I8F_PRO_RMS_NORM) {
+            // RMSNorm over the row, which this wave holds whole: y = x / sqrt(sum x^2 / K + eps) * w in binary32, rounded
+            // once to the dtype (torch's rms_norm); then the modulation's operations, each rounded, where s / t exist.
+            static_assert(WPR == 1 && SEG == 1, "the row's statistics are taken by the one wave that holds it");
+            float ss = 0.0f;
+#pragma unroll
+            for (int r = 0; r < RUNS; ++r) {
+                expand16<DT>(raw[r][0], raw[r][1], v[r]);   // (runs beyond the row are zeros)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) ss = __builtin_fmaf(v[r][j], v[r][j], ss);
+            }
+            const float rstd = 1.0f / sqrtf(wave_sum_all(ss) / (float)K + pro.eps);
+#pragma unroll
+            for (int r = 0; r < RUNS; ++r) {
+                const int R = r * TPR + p;
+                const bool in = FULL || R < nruns;
+                const int64_t col = (in ? R : 0) * 32;   // byte offset of the run's columns in a vector
+                float wv[16];
+                if (pro.w) {
+                    expand16<DT>(*(const uint4 *)((const char *)pro.w + col), *(const uint4 *)((const char *)pro.w + col + 16), wv);
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) v[r][j] = round_to_dtype<DT>(v[r][j] * rstd * wv[j]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) v[r][j] = round_to_dtype<DT>(v[r][j] * rstd);
+                }
+                const int64_t off = vrow * K * 2 + col;
+                if (pro.s) {
+                    expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), wv);
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) v[r][j] = round_to_dtype<DT>(round_to_dtype<DT>(1.0f + wv[j]) * v[r][j]);
+                }
+                if (pro.t) {
+                    expand16<DT>(*(const uint4 *)((const char *)pro.t + off), *(const uint4 *)((const char *)pro.t + off + 16), wv);
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) v[r][j] = round_to_dtype<DT>(v[r][j] + wv[j]);
+                }
+                if (!in) {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) v[r][j] = 0.0f;
+                }
+            }
+        }
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
-            if constexpr (PRO != I8F_PRO_NORM_MODULATE) expand16<DT>(raw[r][0], raw[r][1], v[r]);
+            if constexpr (PRO != I8F_PRO_NORM_MODULATE && PRO != I8F_PRO_RMS_NORM) expand16<DT>(raw[r][0], raw[r][1], v[r]);
             if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_NORM_MODULATE) {
                 // the vectors of this row's group, same 16 columns (they come from cache: every row of the group reads them)
                 const int R = r * TPR + p;
@@ -531,7 +595,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
                 expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), gv);
 #pragma unroll
                 for (int j = 0; j < 16; ++j) v[r][j] = FULL || R < nruns ? apply_prologue<DT, PRO>(v[r][j], gv[j], 0.0f) : 0.0f;
-            } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
+            } else if constexpr (PRO == I8F_PRO_GELU_TANH || PRO == I8F_PRO_GELU_ERF) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) v[r][j] = apply_prologue<DT, PRO>(v[r][j], 0.0f, 0.0f);
             } else if constexpr (PRO == I8F_PRO_CONCAT_GELU) {
@@ -850,6 +914,8 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
     const size_t es = dtype_size(DT);
     bool aligned = ((uintptr_t)x % 16 == 0) && ((ldx * es) % 16 == 0) && (K % EPC == 0) && ((uintptr_t)q % 8 == 0);
     if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_NORM_MODULATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0 && (uintptr_t)pro.t % 16 == 0;
+    if constexpr (PRO == I8F_PRO_RMS_NORM)   // (absent vectors are null pointers, which pass)
+        aligned = aligned && (uintptr_t)pro.s % 16 == 0 && (uintptr_t)pro.t % 16 == 0 && (uintptr_t)pro.w % 16 == 0;
     if constexpr (PRO == I8F_PRO_SILU_GATE) aligned = aligned && (uintptr_t)pro.s % 16 == 0;
     if constexpr (PRO == I8F_PRO_CONCAT_GELU) aligned = aligned && (uintptr_t)pro.b % 16 == 0 && pro.ldb_bytes % 16 == 0;
     const int64_t nchunks = K / EPC;
@@ -857,12 +923,12 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
         const int64_t nruns = K / 16;
         if (aligned && K % 16 == 0 && (uintptr_t)q % 16 == 0 && nruns >= 1 && nruns <= 64 * 4 * 4) {
             if (nruns <= 64 * 4) return pick_runs16<DT, ROT, 1, PRO>((int)((nruns + 63) / 64), x, M, K, ldx, q, scale, st, pro);
-            if constexpr (PRO != I8F_PRO_NORM_MODULATE) return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
+            if constexpr (PRO != I8F_PRO_NORM_MODULATE && PRO != I8F_PRO_RMS_NORM) return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
         }
     }
     // the normalising prologue exists where one wave holds the row: 16-bit rows of up to 4096 aligned elements;
     // the concatenating one where the row stays in registers: 16-bit rows of up to 16384 aligned elements
-    if constexpr (PRO == I8F_PRO_NORM_MODULATE || PRO == I8F_PRO_CONCAT_GELU) return I8F_ERR_UNSUPPORTED;
+    if constexpr (PRO == I8F_PRO_NORM_MODULATE || PRO == I8F_PRO_RMS_NORM || PRO == I8F_PRO_CONCAT_GELU) return I8F_ERR_UNSUPPORTED;
     else {
     if constexpr (PRO == I8F_PRO_NONE) {  // the chunked kernels have no prologue form: such shapes take the generic kernel
         if (aligned && nchunks <= 1024 * 8) {
@@ -887,6 +953,13 @@ int dispatch_rot(bool rot, const void *x, int64_t M, int64_t K, int64_t ldx, int
     case I8F_PRO_GELU_TANH:
         return rot ? dispatch<DT, true, I8F_PRO_GELU_TANH>(x, M, K, ldx, q, scale, st, pro)
                    : dispatch<DT, false, I8F_PRO_GELU_TANH>(x, M, K, ldx, q, scale, st, pro);
+    case I8F_PRO_GELU_ERF:
+        return rot ? dispatch<DT, true, I8F_PRO_GELU_ERF>(x, M, K, ldx, q, scale, st, pro)
+                   : dispatch<DT, false, I8F_PRO_GELU_ERF>(x, M, K, ldx, q, scale, st, pro);
+    case I8F_PRO_RMS_NORM:
+        if constexpr (DT == I8F_F32) return I8F_ERR_UNSUPPORTED;
+        else return rot ? dispatch<DT, true, I8F_PRO_RMS_NORM>(x, M, K, ldx, q, scale, st, pro)
+                        : dispatch<DT, false, I8F_PRO_RMS_NORM>(x, M, K, ldx, q, scale, st, pro);
     case I8F_PRO_SILU_GATE:
         return rot ? dispatch<DT, true, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro)
                    : dispatch<DT, false, I8F_PRO_SILU_GATE>(x, M, K, ldx, q, scale, st, pro);
@@ -976,7 +1049,8 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
                                           int rotate_block, int8_t *q, float *scale, void *stream) {
     using namespace i8f;
     if (prologue == I8F_PRO_NONE) return i8f_quant_rowwise(x, x_dtype, M, K, ldx, rotate_block, q, scale, stream);
-    if (prologue != I8F_PRO_MODULATE && prologue != I8F_PRO_GELU_TANH && prologue != I8F_PRO_SILU_GATE) return I8F_ERR_INVALID;
+    if (prologue != I8F_PRO_MODULATE && prologue != I8F_PRO_GELU_TANH && prologue != I8F_PRO_SILU_GATE && prologue != I8F_PRO_GELU_ERF)
+        return I8F_ERR_INVALID;
     if (M < 0 || K < 0 || !valid_dtype(x_dtype)) return I8F_ERR_INVALID;
     if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
     if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
@@ -1011,6 +1085,29 @@ extern "C" int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64
     if (int rc = check_device()) return rc;
     if (rows_per_vec > 0x7fffffff) rows_per_vec = 0x7fffffff;
     Prologue pro{I8F_PRO_NORM_MODULATE, mod_scale, mod_shift, rows_per_vec, eps};
+    hipStream_t st = (hipStream_t)stream;
+    const bool rot = rotate_block != 0;
+    switch (x_dtype) {
+    case I8F_BF16: return dispatch_rot<I8F_BF16>(rot, x, M, K, ldx, q, scale, st, pro);
+    case I8F_F16: return dispatch_rot<I8F_F16>(rot, x, M, K, ldx, q, scale, st, pro);
+    default: return I8F_ERR_UNSUPPORTED;
+    }
+}
+
+extern "C" int i8f_quant_rowwise_rms_norm(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, float eps, const void *weight,
+                                          const void *mod_scale, const void *mod_shift, int64_t rows_per_vec, int rotate_block,
+                                          int8_t *q, float *scale, void *stream) {
+    using namespace i8f;
+    if (M < 0 || K < 0 || !valid_dtype(x_dtype) || !(eps >= 0.0f)) return I8F_ERR_INVALID;
+    if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
+    if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
+    if (M == 0) return I8F_OK;
+    if (!scale || ldx < K || K == 0 || !x || !q) return I8F_ERR_INVALID;
+    if ((mod_scale || mod_shift) && rows_per_vec <= 0) return I8F_ERR_INVALID;
+    if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
+    if (int rc = check_device()) return rc;
+    if (rows_per_vec > 0x7fffffff || rows_per_vec <= 0) rows_per_vec = 0x7fffffff;
+    Prologue pro{I8F_PRO_RMS_NORM, mod_scale, mod_shift, rows_per_vec, eps, nullptr, 0, 0, weight};
     hipStream_t st = (hipStream_t)stream;
     const bool rot = rotate_block != 0;
     switch (x_dtype) {

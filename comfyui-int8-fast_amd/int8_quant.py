@@ -453,13 +453,15 @@ class Int8TensorwiseOps(manual_cast):
         # -- forward ------------------------------------------------------------------------
         def forward(self, x: Tensor, prologue: int = _lib.PRO_NONE, mod_scale: Tensor | None = None,
                     mod_shift: Tensor | None = None, eps: float = 1e-6, gate: Tensor | None = None,
-                    residual: Tensor | None = None) -> Tensor:
+                    residual: Tensor | None = None, norm_weight: Tensor | None = None) -> Tensor:
             """The reference's forward(x) (int8_quant.py:703-778).  The optional arguments name the elementwise
             operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, _lib.PRO_MODULATE with
             (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension, _lib.PRO_NORM_MODULATE with
             the same modulation of layer_norm(x, eps) (no affine parameters: the whole adaLN producer of a DiT
             block), _lib.PRO_CONCAT_GELU with cat((x, gelu(mod_scale)), -1), the input of the second projection of a
-            single-stream block, or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
+            single-stream block, _lib.PRO_GELU_ERF (GELU in its exact form), _lib.PRO_RMS_NORM with
+            rms_norm(x, norm_weight, eps) followed by * (1 + mod_scale) and + mod_shift where those are given (the
+            producer in blocks that normalise with an RMSNorm), or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
             path then applies inside its quantiser instead of in passes of their own (under torch.compile the graph
             rewrite of compile_ops does this without the caller's help).  `gate` / `residual` name what the caller would
             apply to the result: forward(h, gate=g, residual=x) returns x + g * linear(h), the gated residual of an
@@ -477,7 +479,7 @@ class Int8TensorwiseOps(manual_cast):
                                  and (gate is None or (gate.device == x.device and compile_ops.modulation_broadcasts_over_tokens(
                                      _ShapeAndDtype(out_shape, cdt), gate, gate))))
                 if not fuse_epilogue:   # torch applies the two operations, as the caller would have
-                    y = self.forward(x, prologue, mod_scale, mod_shift, eps)
+                    y = self.forward(x, prologue, mod_scale, mod_shift, eps, norm_weight=norm_weight)
                     if gate is not None:
                         y = gate * y
                     return y if residual is None else residual + y
@@ -498,6 +500,13 @@ class Int8TensorwiseOps(manual_cast):
                     # vectors of another dtype or another broadcast pattern are torch's business (as under compile)
                     fusable = (isinstance(mod_scale, Tensor) and isinstance(mod_shift, Tensor) and x.dim() >= 2
                                and compile_ops.modulation_broadcasts_over_tokens(x, mod_scale, mod_shift))
+                if fusable and prologue == _lib.PRO_RMS_NORM:
+                    vecs = [v for v in (mod_scale, mod_shift) if v is not None]
+                    fusable = (x.dim() >= 2 and _lib.norm_modulate_fusable(x.reshape(-1, x.shape[-1]))
+                               and (norm_weight is None or (norm_weight.dtype == x.dtype and tuple(norm_weight.shape) == (x.shape[-1],)
+                                                            and norm_weight.device == x.device))
+                               and all(isinstance(v, Tensor) and v.device == x.device
+                                       and compile_ops.modulation_broadcasts_over_tokens(x, v, v) for v in vecs))
                 if prologue == _lib.PRO_NORM_MODULATE and not (fusable and _lib.norm_modulate_fusable(x.reshape(-1, x.shape[-1]))):
                     # rows the normalising quantiser does not take: torch normalises, the modulation may still be fused
                     x = F.layer_norm(x, (x.shape[-1],), eps=eps)
@@ -505,6 +514,14 @@ class Int8TensorwiseOps(manual_cast):
                 if not fusable:   # every other path takes the operation as torch would have applied it
                     if prologue == _lib.PRO_GELU_TANH:
                         x = F.gelu(x, approximate="tanh")
+                    elif prologue == _lib.PRO_GELU_ERF:
+                        x = F.gelu(x)
+                    elif prologue == _lib.PRO_RMS_NORM:
+                        x = F.rms_norm(x, (x.shape[-1],), norm_weight, eps)
+                        if mod_scale is not None:
+                            x = x * (1 + mod_scale)
+                        if mod_shift is not None:
+                            x = x + mod_shift
                     elif prologue == _lib.PRO_CONCAT_GELU:
                         x = torch.cat((x, F.gelu(mod_scale, approximate="tanh")), -1)
                     elif prologue == _lib.PRO_SILU_GATE:
@@ -580,7 +597,7 @@ class Int8TensorwiseOps(manual_cast):
                                                   int8_fused_kernel.DEFAULT_EPILOGUE, addend)
                 else:
                     fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
-                    pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift, eps)
+                    pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift, eps, norm_weight)
                     if fuse_epilogue:   # (no dynamic LoRA here: the addend slot is free for the residual stream)
                         addend = None if residual is None else residual.reshape(-1, residual.shape[-1])
                     y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=pro,

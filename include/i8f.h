@@ -83,10 +83,13 @@ typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
  *                      i8f_quant_rowwise_norm_modulate only, which carries the epsilon
  *   I8F_PRO_CONCAT_GELU  cat(a, gelu(b, approximate="tanh")) along the row; taken by
  *                      i8f_quant_rowwise_concat_gelu only, which carries the second tensor
+ *   I8F_PRO_GELU_ERF   gelu(x) in its exact form, 0.5 x (1 + erf(x / sqrt 2)), in binary32, rounded once to x's dtype
+ *   I8F_PRO_RMS_NORM   rms_norm(x, weight, eps), optionally followed by (1 + s[k]) * y and + t[k]; taken by
+ *                      i8f_quant_rowwise_rms_norm only, which carries the epsilon and the weight
  */
 typedef enum i8f_prologue {
     I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2, I8F_PRO_SILU_GATE = 3, I8F_PRO_NORM_MODULATE = 4,
-    I8F_PRO_CONCAT_GELU = 5
+    I8F_PRO_CONCAT_GELU = 5, I8F_PRO_GELU_ERF = 6, I8F_PRO_RMS_NORM = 7
 } i8f_prologue;
 
 /* Library version (I8F_VERSION of the build). */
@@ -148,7 +151,7 @@ int i8f_quant_rowwise_grouped(const i8f_quant_group *groups, int n_groups, int x
  *                 same layout (rows_per_vec = 1 for a gate tensor of x's shape), mod_shift
  *                 is ignored.  Both ignored otherwise.
  * I8F_PRO_MODULATE is bit-identical to torch's three eager operations followed by
- * i8f_quant_rowwise; I8F_PRO_GELU_TANH and I8F_PRO_SILU_GATE agree with torch's gelu / silu
+ * i8f_quant_rowwise; I8F_PRO_GELU_TANH, I8F_PRO_GELU_ERF and I8F_PRO_SILU_GATE agree with torch's gelu / silu
  * to the last bits of binary32 before the rounding to x_dtype (tests state the tolerance).
  */
 int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
@@ -177,6 +180,29 @@ int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64
                                     float eps, const void *mod_scale, const void *mod_shift,
                                     int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale,
                                     void *stream);
+
+/*
+ * The quantiser with an RMSNorm, and optionally the modulation behind it, in front of it:
+ *   y = x * (1 / sqrt(sum x^2 / K + eps)) * weight[k]      in binary32, rounded once to x's dtype (torch's rms_norm;
+ *                                                          weight NULL: no weight)
+ *   z = (1 + s[k]) * y    if mod_scale is given: 1 + s rounded, the product rounded
+ *   z = z + t[k]          if mod_shift is given: rounded
+ *   then rotation, absmax and int8 as i8f_quant_rowwise.
+ * The producer of the attention and feed-forward projections of blocks that normalise with an RMSNorm
+ * (modulate(norm(x), scale) = norm(x) * (1 + scale) in the z-image family, rms_norm(x) * (1 + scale) + shift in the
+ * ltx family; the loader names both, int8_unet_loader.py:60-93).  No counterpart in the reference's files: there
+ * these are the model's own torch operations in front of Linear.forward (int8_quant.py:703), fused by torch.compile
+ * into the quantiser's producer (README.md:4,56); here none of the intermediate tensors is written to memory.
+ * The row's sum is taken in this kernel's order, torch's in its own: y agrees with torch's to the last place of the
+ * dtype (tests state the tolerance).
+ *   weight [K] of x_dtype or NULL; mod_scale, mod_shift [ceil(M / rows_per_vec), K] of x_dtype or NULL each;
+ *   rows_per_vec as for I8F_PRO_MODULATE (ignored when both are NULL).
+ * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 4096 and x, q and the vectors are
+ * 16-byte aligned (one wavefront holds a row): other callers normalise with their own kernel.
+ */
+int i8f_quant_rowwise_rms_norm(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, float eps,
+                               const void *weight, const void *mod_scale, const void *mod_shift,
+                               int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale, void *stream);
 
 /*
  * The quantiser on the concatenation of two tensors along the row, the second through tanh-GELU:

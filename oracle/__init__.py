@@ -46,6 +46,7 @@ def lib() -> ctypes.CDLL:
         L.orc_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp]
         L.orc_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, vp]
         L.orc_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, vp]
+        L.orc_rms_norm.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, vp, i64, vp]
         L.orc_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp]
         L.orc_epilogue.argtypes = [vp, vp, vp, i32, vp, i32, vp, i32, i64, i64, i32]
         L.orc_linear_w8a8.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i32, vp, i32, vp, i32, i64, i32]
@@ -168,7 +169,7 @@ def quant_tensorwise(x, dtype_code):
     return q, s
 
 
-PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE = 1, 2, 3, 4
+PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE, PRO_GELU_ERF = 1, 2, 3, 4, 6
 
 
 def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
@@ -197,6 +198,22 @@ def norm_modulate(x, dtype_code, eps, s, t, rows_per_vec=1):
     assert s.shape == t.shape and s.shape[0] * rows_per_vec >= M
     out = np.empty((M, K), dtype=x.dtype)
     _chk(lib().orc_norm_modulate(_p(x), dtype_code, M, K, K, float(eps), _p(s), _p(t), rows_per_vec, _p(out)), "norm_modulate")
+    return out
+
+
+def rms_norm(x, dtype_code, eps, w=None, s=None, t=None, rows_per_vec=1):
+    """rms_norm(x, w, eps) rounded once to the dtype as torch's kernel does, then (1 + s) * y and + t where given, each
+    rounded; returns the storage array of dtype_code, shape of x."""
+    x = _arr(x, dtype_code)
+    M, K = x.shape
+    w = None if w is None else _arr(w, dtype_code).reshape(K)
+    s = None if s is None else _arr(s, dtype_code).reshape(-1, K)
+    t = None if t is None else _arr(t, dtype_code).reshape(-1, K)
+    for v in (s, t):
+        assert v is None or v.shape[0] * rows_per_vec >= M
+    out = np.empty((M, K), dtype=x.dtype)
+    _chk(lib().orc_rms_norm(_p(x), dtype_code, M, K, K, float(eps), *(None if v is None else _p(v) for v in (w, s, t)),
+                            rows_per_vec, _p(out)), "rms_norm")
     return out
 
 

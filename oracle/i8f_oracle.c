@@ -260,12 +260,14 @@ int orc_quant_rowwise(const void *x, int dtype, int64_t M, int64_t K, int64_t ld
  *           SwiGLU feed-forward, e.g. the z-image family the loader names,
  *           int8_unet_loader.py:60-93); g is s, laid out like s of kind 1; expf is the C
  *           library's: a tolerance reference like kind 2
+ *   kind 6  gelu(x) in its exact form, x * 0.5 * (1 + erf(x / sqrt 2)) in binary32 as torch's kernel writes it,
+ *           rounded once to dtype (erff is the C library's: a tolerance reference)
  * out is [M,K] of dtype, contiguous.  Followed by orc_quant_rowwise it is the
  * oracle of the fused quantiser.
  */
 int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, int kind,
                  const void *s, const void *t, int64_t rows_per_vec, void *out) {
-    if (M < 0 || K < 0 || ldx < K || (kind != 1 && kind != 2 && kind != 3)) return -1;
+    if (M < 0 || K < 0 || ldx < K || (kind != 1 && kind != 2 && kind != 3 && kind != 6)) return -1;
     if (kind == 1 && (rows_per_vec <= 0 || !s || !t)) return -1;
     if (kind == 3 && (rows_per_vec <= 0 || !s)) return -1;
 #pragma omp parallel for schedule(static)
@@ -284,6 +286,8 @@ int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, in
                 const size_t vi = (size_t)((m / rows_per_vec) * K + k);
                 const float a = round_to_dtype(xv / (1.0f + expf(-xv)), dtype);
                 v = a * load_as_f32(s, dtype, vi);
+            } else if (kind == 6) {
+                v = xv * 0.5f * (1.0f + erff(xv * 0.70710678118654752440f));
             } else {
                 const float kBeta = 0.7978845608028654f, kKappa = 0.044715f;
                 const float x3 = xv * xv * xv;
@@ -291,6 +295,38 @@ int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, in
                 v = 0.5f * xv * (1.0f + tanhf(inner));
             }
             store_from_f32(out, dtype, (size_t)(m * K + k), v);
+        }
+    }
+    return 0;
+}
+
+/*
+ * RMSNorm, optionally followed by the modulation (the model's own torch operations in front of
+ * Linear.forward, int8_quant.py:703, in the families the loader names that normalise with an RMSNorm,
+ * int8_unet_loader.py:60-93):
+ *   y = round(x * rstd * w),  rstd = 1 / sqrt(sum x^2 / K + eps)     (torch's rms_norm: binary32, one rounding; w optional)
+ *   z = round(round(1 + s) * y)   if s,   z = round(z + t)   if t
+ * The row's sum is taken in double (torch takes it in binary32 in its own order).
+ */
+int orc_rms_norm(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, float eps, const void *w,
+                 const void *s, const void *t, int64_t rows_per_vec, void *out) {
+    if (M < 0 || K <= 0 || ldx < K || ((s || t) && rows_per_vec <= 0)) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        double ss = 0.0;
+        for (int64_t k = 0; k < K; ++k) {
+            const double d = (double)load_as_f32(x, dtype, (size_t)(m * ldx + k));
+            ss += d * d;
+        }
+        const float rstd = 1.0f / sqrtf((float)(ss / (double)K) + eps);
+        for (int64_t k = 0; k < K; ++k) {
+            const size_t vi = (s || t) ? (size_t)((m / rows_per_vec) * K + k) : 0;
+            float y = load_as_f32(x, dtype, (size_t)(m * ldx + k)) * rstd;
+            if (w) y = y * load_as_f32(w, dtype, (size_t)k);
+            y = round_to_dtype(y, dtype);
+            if (s) y = round_to_dtype(round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype) * y, dtype);
+            if (t) y = y + load_as_f32(t, dtype, vi);
+            store_from_f32(out, dtype, (size_t)(m * K + k), y);
         }
     }
     return 0;

@@ -241,6 +241,67 @@ def test_graph_rewrite_moves_layer_norm_and_modulation_into_the_quantiser(pkg):
         assert node.args[1] == pkg._lib.PRO_MODULATE and ln_left
 
 
+def test_graph_rewrite_moves_rms_norm_and_exact_gelu_into_the_quantiser(pkg):
+    """rms_norm(h, w) * (1 + scale) -> linear (z-image's modulate(norm(x), scale)), (1 + scale) * rms_norm(h) + shift ->
+    linear (ltx), a bare rms_norm -> linear, and gelu(h) in its exact form -> linear: all become the layer's prologue,
+    the weight of the norm travelling as the operator's norm_weight; an RMSNorm whose weight has another dtype, one used
+    elsewhere too, or rows wider than a wavefront holds stay torch's."""
+    g = torch.Generator().manual_seed(14)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Block(torch.nn.Module):
+        def __init__(self, k, form, wdt=torch.bfloat16):
+            super().__init__()
+            self.norm = torch.nn.RMSNorm(k, eps=1e-5, elementwise_affine=form != "ltx").to(wdt)
+            self.qkv, self.form = lin(64, k), form
+
+        def forward(self, x, scale, shift):
+            h = self.norm(x)
+            if self.form == "zimage":
+                return self.qkv(h * (1 + scale))
+            if self.form == "ltx":
+                return self.qkv(h * (1 + scale) + shift)
+            if self.form == "reuse":
+                return self.qkv(h * (1 + scale)) + h.sum()
+            return self.qkv(h)
+
+    def rewrite(mod, k):
+        x, v = torch.randn(2, 24, k).bfloat16(), torch.randn(2, 1, k).bfloat16()
+        gm = torch._dynamo.export(mod)(x, v, v).graph_module
+        n = pkg.compile_ops.fuse_prologues(gm)
+        nodes = [n_ for n_ in gm.graph.nodes if n_.op == "call_function" and "int8_linear_prologue" in str(n_.target)]
+        return n, nodes, any("rms_norm" in str(n_.target) for n_ in gm.graph.nodes if n_.op == "call_function")
+
+    for form, has_w, has_s, has_t in (("zimage", True, True, False), ("ltx", False, True, True), ("bare", True, False, False)):
+        n, nodes, norm_left = rewrite(Block(256, form), 256)
+        assert n == 1 and len(nodes) == 1 and not norm_left
+        node = nodes[0]
+        assert node.args[1] == pkg._lib.PRO_RMS_NORM and abs(node.args[11] - 1e-5) < 1e-12
+        assert (node.kwargs.get("norm_weight") is not None) == has_w
+        assert (node.args[2] is not None) == has_s and (node.args[3] is not None) == has_t
+    for mod, k in ((Block(256, "zimage", torch.float32), 256), (Block(256, "reuse"), 256), (Block(8192, "zimage"), 8192)):
+        n, nodes, norm_left = rewrite(mod, k)
+        assert n == 0 and norm_left
+
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up, self.down = lin(128, 64), lin(64, 128)
+
+        def forward(self, x):
+            return self.down(F.gelu(self.up(x)))
+
+    gm = torch._dynamo.export(Mlp())(torch.randn(2, 24, 64).bfloat16()).graph_module
+    assert pkg.compile_ops.fuse_prologues(gm) == 1
+    node = [n_ for n_ in gm.graph.nodes if n_.op == "call_function" and "int8_linear_prologue" in str(n_.target)][0]
+    assert node.args[1] == pkg._lib.PRO_GELU_ERF
+    assert not any(n_.target is F.gelu for n_ in gm.graph.nodes if n_.op == "call_function")
+
+
 def test_graph_rewrite_moves_concatenation_and_gelu_into_the_quantiser(pkg):
     """linear2(cat((attn, gelu(mlp)), -1)), the second projection of a single-stream block: both producers become the
     layer's prologue; a concatenation along another dimension, of three tensors, or with an exact GELU stays torch's."""
@@ -481,6 +542,52 @@ def test_compiled_adaln_zero_block_equals_eager_bit_for_bit(pkg, dev):
     want = m.down(h, prologue=L.PRO_GELU_TANH, gate=gate, residual=x)
     assert torch.equal(got, want)
     loose = m(x, sc, sh, gate)                           # torch's LayerNorm, modulation, gelu, gate and residual around the layers
+    assert (got.float() - loose.float()).abs().max().item() <= 2.0**-6 * loose.float().abs().max().item()
+
+
+@pytest.mark.gpu
+def test_compiled_rms_norm_producer_and_exact_gelu_equal_eager_bit_for_bit(pkg, dev):
+    """down(gelu(up(norm(x) * (1 + scale)))) with an RMSNorm that has a weight and GELU in its exact form, compiled with the
+    rewriting backend over inductor: two fused operators, neither an rms_norm nor a gelu kernel left; equal to the
+    eager fused forward calls bit for bit and within rounding of torch's operations around the layers."""
+    g = torch.Generator().manual_seed(17)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = torch.nn.RMSNorm(256, eps=1e-5).bfloat16()
+            self.up, self.down = lin(512, 256), lin(256, 512)
+
+        def forward(self, x, scale):
+            return self.down(F.gelu(self.up(self.norm(x) * (1 + scale))))
+
+    m = Block().to(dev)
+    with torch.no_grad():
+        m.norm.weight.copy_((torch.randn(256, generator=g) * 0.2 + 1).bfloat16())
+    x = (torch.randn(2, 40, 256, generator=g) * 2).bfloat16().to(dev)
+    scale = (torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev)
+    seen = []
+
+    def counting(gm, inputs):
+        calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum("int8_linear_prologue" in str(n.target) for n in calls),
+                     sum("rms_norm" in str(n.target) or "gelu" in str(n.target) or n.target in (operator.mul, operator.add) for n in calls)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    with torch.no_grad():
+        got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x, scale)
+        assert seen == [(2, 0)]
+        L = pkg._lib
+        h = m.up(x, prologue=L.PRO_RMS_NORM, norm_weight=m.norm.weight, mod_scale=scale, eps=1e-5)
+        want = m.down(h, prologue=L.PRO_GELU_ERF)
+        assert torch.equal(got, want)
+        loose = m(x, scale)
     assert (got.float() - loose.float()).abs().max().item() <= 2.0**-6 * loose.float().abs().max().item()
 
 

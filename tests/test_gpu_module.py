@@ -289,6 +289,17 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
         b = lin((1 + sc) * F.layer_norm(x, (384,), eps=1e-6) + sh)
         assert a.shape == (2, 20, 96) and (a.float() - b.float()).abs().max() <= 2.0**-6 * b.float().abs().max()
         assert (a != b).float().mean().item() <= 0.2
+        a = lin(x, prologue=L.PRO_GELU_ERF)
+        b = lin(F.gelu(x))
+        assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
+        nw = (torch.randn(384, generator=g) * 0.2 + 1).bfloat16().to(dev)
+        for w_, s_, t_ in ((nw, sc, None), (None, sc, sh), (nw, None, None)):   # z-image's and ltx's producers, a bare RMSNorm
+            a = lin(x, prologue=L.PRO_RMS_NORM, norm_weight=w_, mod_scale=s_, mod_shift=t_, eps=1e-5)
+            h = F.rms_norm(x, (384,), w_, 1e-5)
+            h = h if s_ is None else h * (1 + s_)
+            b = lin(h if t_ is None else h + t_)
+            assert a.shape == (2, 20, 96) and (a.float() - b.float()).abs().max() <= 2.0**-6 * b.float().abs().max()
+            assert (a != b).float().mean().item() <= 0.2
     # vectors that torch would broadcast differently, or of another dtype, are left to torch: same result as the
     # unfused expression (a [1, T, K] vector against a batch of 2 must not be dealt over the rows as if it were [2, 1, K])
     lin._use_quarot = False
@@ -300,6 +311,10 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
     assert torch.equal(lin(small, prologue=L.PRO_GELU_TANH), lin(F.gelu(small, approximate="tanh")))
     assert torch.equal(lin(small, prologue=L.PRO_NORM_MODULATE, mod_scale=sc[:1], mod_shift=sh[:1], eps=1e-5),
                        lin((1 + sc[:1]) * F.layer_norm(small, (384,), eps=1e-5) + sh[:1]))
+    assert torch.equal(lin(small, prologue=L.PRO_RMS_NORM, norm_weight=nw, mod_scale=sc[:1], eps=1e-5),
+                       lin(F.rms_norm(small, (384,), nw, 1e-5) * (1 + sc[:1])))
+    assert torch.equal(lin(x, prologue=L.PRO_RMS_NORM, norm_weight=nw.float(), eps=1e-5), lin(F.rms_norm(x, (384,), nw.float(), 1e-5)))
+    assert torch.equal(lin(small, prologue=L.PRO_GELU_ERF), lin(F.gelu(small)))
     # rows that the normalising quantiser does not take (binary32 here): torch normalises, and the result is that of
     # the unfused expression
     x32, sc_, sh_ = x.float(), sc.float(), sh.float()

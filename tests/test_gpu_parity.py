@@ -216,12 +216,75 @@ def test_quant_rowwise_norm_modulate_prologue_within_tolerance(L, dev, M, K, dt,
     assert torch.equal(again[0], q) and torch.equal(again[1], sc)     # fixed order of the sums: launches agree bit for bit
 
 
+@pytest.mark.parametrize("M,K,dt,rot,V", PROLOGUE_CASES)
+def test_quant_rowwise_gelu_erf_prologue_within_tolerance(L, dev, M, K, dt, rot, V):
+    """GELU in its exact form inside the quantiser (x Phi(x), the complementary error function by a rational-exponential
+    form good to 1.5e-7 of Phi) against the oracle (C erff) and against torch's gelu on the device followed by the plain
+    quantiser: the bar of the tanh form -- scales within 2 ulp of the dtype, int8 at most 1 apart, at least 99.9 % equal
+    (99 % with rotation); in binary32, where nothing hides the approximation, int8 still at most 1 apart."""
+    x = (acts(M, K, dt).float() * 0.5).to(dt)
+    xa, code = O.from_torch(x)
+    qo, so = O.quant_rowwise(O.prologue(xa, code, O.PRO_GELU_ERF), code, 128 if rot else 0)
+    q, s = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_GELU_ERF)
+    q2, s2 = L.quant_rowwise(torch.nn.functional.gelu(x.to(dev)), rotate=rot)
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11, torch.float32: 2.0**-20}[dt]
+    for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+        d = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() <= (1e-2 if rot else 1e-3)
+        assert (np.abs(s.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
+    qt, _ = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_GELU_TANH)
+    if M * K > 10000 and not rot:
+        assert not torch.equal(q, qt)     # the two forms differ by up to 5e-4: visible in int8 on enough elements
+
+
+@pytest.mark.parametrize("M,K,dt,rot,V,eps,parts", [
+    (64, 3072, torch.bfloat16, False, 1, 1e-6, "wst"), (48, 3072, torch.bfloat16, True, 2, 1e-6, "ws"), (33, 4096, torch.float16, False, 3, 1e-5, "w"),
+    (10, 1008, torch.bfloat16, False, 2, 1e-6, "st"), (6, 384, torch.float16, True, 1, 1e-5, ""), (5, 16, torch.bfloat16, False, 1, 1e-6, "wt"),
+    (4608, 3840, torch.bfloat16, False, 1, 1e-5, "ws"),
+])
+def test_quant_rowwise_rms_norm_prologue_within_tolerance(L, dev, M, K, dt, rot, V, eps, parts):
+    """RMSNorm with its weight and the modulation behind it inside the quantiser (i8f_quant_rowwise_rms_norm; each of
+    weight, scale and shift present or not) against the oracle (row sum in double) and against torch's rms_norm and
+    eager operations on the device followed by the plain quantiser.  The bar of the LayerNorm form: scales within 2 ulp
+    of the dtype, int8 at most 1 apart, at least 99.5 % equal (98 % with rotation)."""
+    rows = M - M % V
+    x = (acts(rows, K, dt).float() * 3 + 0.25).to(dt)
+    w = (torch.randn(K, generator=G) * 0.2 + 1).to(dt) if "w" in parts else None
+    s = (torch.randn(V, K, generator=G) * 0.3).to(dt) if "s" in parts else None
+    t = (torch.randn(V, K, generator=G) * 0.2).to(dt) if "t" in parts else None
+    xa, code = O.from_torch(x)
+    z = O.rms_norm(xa, code, eps, *(None if v is None else O.from_torch(v)[0] for v in (w, s, t)), rows_per_vec=rows // V)
+    qo, so = O.quant_rowwise(z, code, 128 if rot else 0)
+    d = lambda v: None if v is None else v.to(dev)
+    q, sc = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_RMS_NORM, norm_weight=d(w), mod_scale=d(s), mod_shift=d(t), eps=eps)
+    zt = torch.nn.functional.rms_norm(x.to(dev), (K,), d(w), eps).reshape(V, rows // V, K)
+    if s is not None:
+        zt = zt * (1 + d(s)[:, None])
+    if t is not None:
+        zt = zt + d(t)[:, None]
+    q2, s2 = L.quant_rowwise(zt.reshape(rows, K), rotate=rot)
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[dt]
+    for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+        df = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+        assert df.max() <= 1 and (df != 0).mean() <= (2e-2 if rot else 5e-3)
+        assert (np.abs(sc.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
+    again = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_RMS_NORM, norm_weight=d(w), mod_scale=d(s), mod_shift=d(t), eps=eps)
+    assert torch.equal(again[0], q) and torch.equal(again[1], sc)
+    if parts == "":      # nothing but the normalisation: invariant under a positive power-of-two factor (eps scaled with it)
+        q4, s4 = L.quant_rowwise((x.float() * 4).to(dt).to(dev), rotate=rot, prologue=L.PRO_RMS_NORM, eps=eps * 16)
+        assert torch.equal(q4, q) and torch.equal(s4, sc)
+
+
 def test_quant_rowwise_norm_modulate_refuses_rows_it_does_not_take(L, dev):
     s = torch.zeros(1, 8192, dtype=torch.bfloat16, device=dev)
     with pytest.raises(ValueError):
         L.quant_rowwise(torch.zeros(4, 8192, dtype=torch.bfloat16, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s, mod_shift=s)
     with pytest.raises(ValueError):
         L.quant_rowwise(torch.zeros(4, 256, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s[:, :256].float(), mod_shift=s[:, :256].float())
+    with pytest.raises(ValueError):
+        L.quant_rowwise(torch.zeros(4, 8192, dtype=torch.bfloat16, device=dev), prologue=L.PRO_RMS_NORM)
+    with pytest.raises(ValueError):
+        L.quant_rowwise(torch.zeros(4, 256, dtype=torch.bfloat16, device=dev), prologue=L.PRO_RMS_NORM, norm_weight=s[0, :128])
 
 
 @pytest.mark.parametrize("M,Ka,Kb,dt,rot", [

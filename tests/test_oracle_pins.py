@@ -566,6 +566,87 @@ def test_norm_modulate_agrees_with_torch(dt):
     assert torch.equal(got3.view(torch.int16), tv[:1, :64].contiguous().view(torch.int16))
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+def test_prologue_gelu_erf_agrees_with_torch_and_with_the_normal_distribution(dt):
+    """GELU in its exact form, x Phi(x): against torch's gelu (same binary32 expression, its own vectorised erf: at most
+    one unit in the last place of the storage dtype apart, and rarely) and against scipy's normal distribution function
+    in double (what the mathematics fixes; the binary32 expression 1 + erf cancels in the negative tail, so the bound
+    carries a few units of 2^-24 |x| on top of the dtype's rounding)."""
+    from scipy.special import ndtr
+    g = torch.Generator().manual_seed(34)
+    x = (torch.randn(64, 512, generator=g) * 3).to(dt)
+    x[0, :8] = torch.tensor([0.0, -0.0, 1e-6, -1e-6, 20.0, -20.0, 100.0, -100.0]).to(dt)
+    want = torch.nn.functional.gelu(x)
+    xa, code = O.from_torch(x)
+    got = O.to_f32(O.prologue(xa, code, O.PRO_GELU_ERF), code)
+    w = want.float().numpy()
+    ulp = {torch.bfloat16: 2.0**-7, torch.float16: 2.0**-10, torch.float32: 2.0**-22}[dt]
+    xf = x.float().numpy()
+    tiny = 2.0**-24 if dt == torch.float16 else 0.0      # the spacing of fp16's subnormals, where the far tail ends up
+    # (torch's vectorised binary32 erf is itself a rational-exponential form good to about 1e-6: in binary32 the comparison
+    # with torch is that loose, the one with the normal distribution below is the tight one)
+    slack = 2.0**-19 if dt == torch.float32 else 2.0**-22
+    assert (np.abs(got - w) <= ulp * np.abs(w) + slack * np.abs(xf) + tiny).all()
+    # left of -2 the sum 1 + erf keeps few bits of the erf (torch's and the C library's differ in the last one), and
+    # the result is below 0.05 in magnitude: there a fifth of the 16-bit values may sit one unit apart; elsewhere none
+    if dt != torch.float32:
+        assert (got != w)[xf > -2].mean() < 1e-3 and (got != w).mean() < 0.1
+    exact = xf.astype(np.float64) * ndtr(xf.astype(np.float64))
+    assert (np.abs(got - exact) <= ulp * np.abs(exact) + 2.0**-21 * np.abs(xf) + tiny + 1e-30).all()
+    assert got[0, 4] == 20.0 and got[0, 5] == 0.0 and got[0, 0] == 0.0
+    # and it is not the tanh form: the two differ by up to 5e-4 around |x| = 2, which binary32 resolves
+    if dt == torch.float32:
+        tanh_form = O.to_f32(O.prologue(xa, code, O.PRO_GELU_TANH), code)
+        assert np.abs(got - tanh_form).max() > 1e-4
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_rms_norm_agrees_with_torch(dt):
+    """rms_norm(x, w, eps) as torch computes it on 16-bit tensors (binary32, one rounding), then the modulation's
+    operations.  The oracle takes the row's sum of squares in double, torch in binary32 in its own order: the
+    normalised value may land on the other side of a rounding boundary, rarely.  Also pinned: the closed form on rows
+    of +-c (rms = c, so y = +-w to the rounding of 1 / sqrt(1 + eps / c^2) = 1), the modulation half against the
+    modulation prologue applied to the oracle's own normalised tensor, and each optional operand left out."""
+    g = torch.Generator().manual_seed(42)
+    M, K, eps = 48, 768, 1e-6
+    x = (torch.randn(M, K, generator=g) * 2 + 0.3).to(dt)
+    x[:, 5] *= 30
+    w = (torch.randn(K, generator=g) * 0.2 + 1).to(dt)
+    s = (torch.randn(2, K, generator=g) * 0.3).to(dt)
+    t = (torch.randn(2, K, generator=g) * 0.2).to(dt)
+    xa, code = O.from_torch(x)
+    ulp = {torch.bfloat16: 2.0**-7, torch.float16: 2.0**-10}[dt]
+    for weight in (w, None):
+        want = torch.nn.functional.rms_norm(x, (K,), weight, eps)
+        got = O.to_f32(O.rms_norm(xa, code, eps, None if weight is None else O.from_torch(weight)[0]), code)
+        wn = want.float().numpy()
+        assert (np.abs(got - wn) <= ulp * np.abs(wn) + 1e-30).all()
+        assert (got != wn).mean() < 5e-3
+    # the modulation half: the same three roundings as the modulation prologue on the normalised tensor
+    y = O.rms_norm(xa, code, eps, O.from_torch(w)[0])
+    both = O.rms_norm(xa, code, eps, O.from_torch(w)[0], O.from_torch(s)[0], O.from_torch(t)[0], rows_per_vec=M // 2)
+    assert np.array_equal(both, O.prologue(y, code, O.PRO_MODULATE, O.from_torch(s)[0], O.from_torch(t)[0], rows_per_vec=M // 2))
+    zero = torch.zeros(2, K).to(dt)
+    only_s = O.rms_norm(xa, code, eps, O.from_torch(w)[0], O.from_torch(s)[0], None, rows_per_vec=M // 2)
+    assert np.array_equal(only_s, O.prologue(y, code, O.PRO_MODULATE, O.from_torch(s)[0], O.from_torch(zero)[0], rows_per_vec=M // 2))
+    only_t = O.rms_norm(xa, code, eps, O.from_torch(w)[0], None, O.from_torch(t)[0], rows_per_vec=M // 2)
+    assert np.array_equal(only_t, O.prologue(y, code, O.PRO_MODULATE, O.from_torch(zero)[0], O.from_torch(t)[0], rows_per_vec=M // 2))
+    # against torch end to end (z-image's modulate(norm(x), scale) and ltx's rms_norm(x) * (1 + scale) + shift)
+    want = torch.nn.functional.rms_norm(x, (K,), w, eps).view(2, M // 2, K) * (1 + s[:, None])
+    wn = want.reshape(M, K).float().numpy()
+    got = O.to_f32(only_s, code)
+    assert (np.abs(got - wn) <= 2 * ulp * np.abs(wn) + 1e-30).all() and (got != wn).mean() < 1e-2
+    # closed form: rows of +-4 have rms 4 exactly, y = +-1 * w
+    pm = torch.full((4, 256), 4.0)
+    pm[:, ::2] = -4.0
+    wv = (torch.randn(256, generator=g) * 0.5 + 1).to(dt)
+    got2 = O.to_torch(O.rms_norm(O.from_torch(pm.to(dt))[0], code, 1e-6, O.from_torch(wv)[0]), code)
+    assert torch.equal(got2.view(torch.int16), (torch.sign(pm).to(dt) * wv).view(torch.int16))
+    # a row of zeros stays zero (rstd = 1 / sqrt(eps) is finite)
+    got3 = O.to_f32(O.rms_norm(O.from_torch(torch.zeros(1, 64).to(dt))[0], code, 1e-6, O.from_torch(wv[:64].contiguous())[0]), code)
+    assert (got3 == 0).all()
+
+
 @pytest.mark.parametrize("tdt", [torch.bfloat16, torch.float16, torch.float32])
 def test_gate_residual_equals_torch_ops(tdt):
     """x + gate * y on tensors of one dtype: two elementwise torch operations, each rounded to the dtype; with the gate
