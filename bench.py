@@ -579,7 +579,29 @@ def extras(L, dev, quick=False):
                                              "note": "x + gate * down(gelu(up((1 + scale) * layer_norm(x) + shift))), bf16, M = 4608: 2 quantiser "
                                                      "launches (LayerNorm + modulation, tanh-GELU) and 2 GEMMs (the second with gate and residual) "
                                                      "against the same layers with 8 torch kernels around them"}
-    del xm, w_up, w_dn, h_buf, o_buf
+    del w_up, w_dn, h_buf
+
+    # separate q, k and v projections of one tensor (4608 x 3072 -> 3 x 3072): one quantiser for the three GEMMs against
+    # the reference's one per Linear.forward
+    wf = [L.quant_rowwise(torch.randn(Dm, Dm, device=dev) * 0.02) for _ in range(3)]
+    of = [torch.empty(Mm, Dm, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+
+    def fan_shared(_i):
+        q1, s1 = L.quant_rowwise(xm)
+        for (wq_, ws_), o_ in zip(wf, of):
+            L.linear_w8a8(q1, s1, wq_, ws_, None, torch.bfloat16, L.EPI_TORCH, o_)
+
+    def fan_separate(_i):
+        for (wq_, ws_), o_ in zip(wf, of):
+            q1, s1 = L.quant_rowwise(xm)
+            L.linear_w8a8(q1, s1, wq_, ws_, None, torch.bfloat16, L.EPI_TORCH, o_)
+
+    t_fs = time_kernel(fan_shared, max(10, iters // 4))
+    t_fp = time_kernel(fan_separate, max(10, iters // 4))
+    out["qkv_fanout_4608x3072_to_3x3072"] = {"one_quantiser_median_us": round(t_fs["median_us"], 2),
+                                             "a_quantiser_per_layer_median_us": round(t_fp["median_us"], 2),
+                                             "note": "forward_fanout / compile_ops.share_quantisation: layers that read one tensor share its int8 rows"}
+    del xm, wf, of, o_buf
 
     # config 2: QuaRot layer (width 3840, 2 % of the channels x50): time of the rotated path and what the
     # rotation buys in accuracy against the bf16 product

@@ -36,6 +36,7 @@ from .int8_quant import (  # noqa: F401
     INT8MergedLoRAPatchAdapter,
     Int8TensorwiseOps,
     dequantize,
+    forward_fanout,
     forward_pair,
     int8_forward_dynamic,
     int8_forward_dynamic_per_row,

@@ -19,9 +19,11 @@ the namespace `i8f` with a shape-only ("fake") implementation:
 dispatcher overhead per layer.  A weight scale is passed either as a tensor or, for the
 single-scale layout, as a float beside a `None` tensor.
 
-`fuse_prologues(graph_module)` rewrites a traced graph so that `gelu(x, approximate="tanh")`,
-`(1 + scale) * x + shift` and `silu(a) * b` feeding an `int8_linear` become its prologue, and `backend(inner)` is a
-torch.compile backend that applies the rewrite and hands the graph to `inner` ("inductor" by default):
+`fuse_prologues(graph_module)` rewrites a traced graph so that the elementwise producer of a layer's activations
+(GELU, adaLN modulation with its LayerNorm or RMSNorm, `silu(a) * b`, `cat((a, gelu(b)), -1)`) becomes the prologue of
+its quantiser, `fuse_epilogues` moves `res + gate * layer(h)` into the GEMM epilogue, `share_quantisation` gives layers
+that read one tensor a single quantiser, and `backend(inner)` is a torch.compile backend that applies the three and
+hands the graph to `inner` ("inductor" by default):
 
     model = torch.compile(model, backend=compile_ops.backend())
 """
@@ -52,6 +54,23 @@ def _(x, rotate):
     return (x.new_empty(x.shape, dtype=torch.int8), x.new_empty((x.shape[0], 1), dtype=torch.float32))
 
 
+@torch.library.custom_op(f"{NAMESPACE}::quantize_rowwise_prologue", mutates_args=())
+def quantize_rowwise_prologue(x: Tensor, rotate: bool, prologue: int, mod_scale: Optional[Tensor], mod_shift: Optional[Tensor],
+                              eps: float = 1e-6, norm_weight: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """quantize_rowwise on prologue(x) (the kinds of int8_linear_prologue), x with any leading dimensions:
+    -> int8 [rows, K'] and float32 [rows, 1], K' the width behind the prologue.  What the layers that read one
+    activation tensor share when the graph rewrite gives them a single quantiser."""
+    return _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
+                              mod_shift=mod_shift, eps=eps, norm_weight=norm_weight)
+
+
+@quantize_rowwise_prologue.register_fake
+def _(x, rotate, prologue, mod_scale, mod_shift, eps=1e-6, norm_weight=None):
+    rows = x.numel() // max(1, x.shape[-1])
+    width = x.shape[-1] + (mod_scale.shape[-1] if prologue == _lib.PRO_CONCAT_GELU else 0)
+    return (x.new_empty((rows, width), dtype=torch.int8), x.new_empty((rows, 1), dtype=torch.float32))
+
+
 @torch.library.custom_op(f"{NAMESPACE}::rotate128", mutates_args=())
 def rotate128(x: Tensor) -> Tensor:
     return _lib.rotate128(x)
@@ -64,12 +83,15 @@ def _(x):
 
 @torch.library.custom_op(f"{NAMESPACE}::linear_w8a8", mutates_args=())
 def linear_w8a8(a: Tensor, a_scale: Tensor, weight: Tensor, weight_scale: Optional[Tensor],
-                weight_scale_value: float, bias: Optional[Tensor], out_dtype: torch.dtype, order: int) -> Tensor:
-    return _lib.linear_w8a8(a, a_scale, weight, _scale_arg(weight_scale, weight_scale_value), bias, out_dtype, order)
+                weight_scale_value: float, bias: Optional[Tensor], out_dtype: torch.dtype, order: int,
+                addend: Optional[Tensor] = None, gate: Optional[Tensor] = None) -> Tensor:
+    """The GEMM on quantised activations [M,K]; addend / gate as for int8_linear.  -> [M,N]"""
+    return _lib.linear_w8a8(a, a_scale, weight, _scale_arg(weight_scale, weight_scale_value), bias, out_dtype, order,
+                            addend=addend, gate=gate)
 
 
 @linear_w8a8.register_fake
-def _(a, a_scale, weight, weight_scale, weight_scale_value, bias, out_dtype, order):
+def _(a, a_scale, weight, weight_scale, weight_scale_value, bias, out_dtype, order, addend=None, gate=None):
     return a.new_empty((a.shape[0], weight.shape[0]), dtype=out_dtype)
 
 
@@ -131,7 +153,8 @@ def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_valu
     return x.new_empty((*x.shape[:-1], width), dtype=compute_dtype)
 
 
-OPS = ("quantize_rowwise", "rotate128", "linear_w8a8", "int8_linear", "linear_w8a16_small_m", "int8_linear_prologue")
+OPS = ("quantize_rowwise", "quantize_rowwise_prologue", "rotate128", "linear_w8a8", "int8_linear", "linear_w8a16_small_m",
+       "int8_linear_prologue")
 
 
 # --------------------------------------------------------------------------- graph rewrite
@@ -220,7 +243,7 @@ def _match_silu_gate(node):
                 and _is_call(act, torch.nn.functional.silu)):
             continue
         a = act.args[0]
-        va, vb = (n.meta.get("example_value", n.meta.get("val")) if isinstance(n, torch.fx.Node) else None for n in (a, gate))
+        va, vb = _meta_val(a), _meta_val(gate)
         if va is not None and vb is not None and tuple(va.shape) == tuple(vb.shape) and va.dtype == vb.dtype:
             return a, gate
     return None
@@ -289,7 +312,7 @@ def _match_plain_layer_norm(node):
     h, shape = a.get("input"), a.get("normalized_shape")
     if a.get("weight") is not None or a.get("bias") is not None or not isinstance(h, torch.fx.Node):
         return None
-    v = h.meta.get("example_value", h.meta.get("val"))
+    v = _meta_val(h)
     if v is None or v.dtype not in (torch.bfloat16, torch.float16):
         return None
     K = int(v.shape[-1])
@@ -302,12 +325,9 @@ def _match_plain_layer_norm(node):
 def _vectors_broadcast_over_tokens(x, scale, shift) -> bool:
     """True if the traced shapes say scale/shift are [.., 1, K] (or [K]) against x [.., T, K]: one vector per
     leading index, shared by the T rows that become consecutive rows of the flattened activations."""
-    def meta(n):
-        return n.meta.get("example_value", n.meta.get("val"))
-
-    if any(not isinstance(n, torch.fx.Node) or meta(n) is None for n in (x, scale, shift)):
+    if any(_meta_val(n) is None for n in (x, scale, shift)):
         return False
-    return modulation_broadcasts_over_tokens(meta(x), meta(scale), meta(shift))
+    return modulation_broadcasts_over_tokens(_meta_val(x), _meta_val(scale), _meta_val(shift))
 
 
 def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
@@ -323,75 +343,98 @@ def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
     return len(ss) == len(xs) and ss[-1] == xs[-1] and ss[-2] == 1 and ss[:-2] == xs[:-2]
 
 
+def _match_producer(src, rotate):
+    """The producer of a layer's activations as a prologue kind -> (h, kind, mod_scale, mod_shift, eps, norm_weight)
+    nodes / values, or None.  Every node matched is used nowhere else."""
+    h = _match_gelu(src)
+    if h is not None:
+        return h, _lib.PRO_GELU_TANH, None, None, 1e-6, None
+    h = _match_gelu_erf(src)
+    if h is not None:
+        return h, _lib.PRO_GELU_ERF, None, None, 1e-6, None
+    r = _match_rms_norm(src)
+    if r is not None:                                               # the norm alone
+        return r[0], _lib.PRO_RMS_NORM, None, None, r[2], r[1]
+    so = _match_scale_only(src)
+    if so is not None:                                              # modulate(norm(x), scale) = norm(x) * (1 + scale)
+        r = _match_rms_norm(so[0])
+        if r is not None and _vectors_broadcast_over_tokens(r[0], so[1], so[1]):
+            return r[0], _lib.PRO_RMS_NORM, so[1], None, r[2], r[1]
+    m = _match_modulate(src)
+    if m is not None:
+        if not _vectors_broadcast_over_tokens(*m):
+            return None
+        ln = _match_plain_layer_norm(m[0])   # the modulated tensor is a LayerNorm without affine: that goes in too
+        if ln is not None:
+            return ln[0], _lib.PRO_NORM_MODULATE, m[1], m[2], ln[1], None
+        rn = _match_rms_norm(m[0])           # or an RMSNorm
+        if rn is not None and _vectors_broadcast_over_tokens(rn[0], m[1], m[2]):
+            return rn[0], _lib.PRO_RMS_NORM, m[1], m[2], rn[2], rn[1]
+        return m[0], _lib.PRO_MODULATE, m[1], m[2], 1e-6, None
+    g = _match_silu_gate(src)
+    if g is not None:
+        return g[0], _lib.PRO_SILU_GATE, g[1], None, 1e-6, None
+    c = _match_concat_gelu(src)
+    if c is not None and not (rotate and (_meta_shape(c[0])[-1] % 128 or _meta_shape(c[1])[-1] % 128)):
+        return c[0], _lib.PRO_CONCAT_GELU, c[1], None, 1e-6, None
+    return None
+
+
 def fuse_prologues(gm: torch.fx.GraphModule) -> int:
     """Rewrite int8_linear(gelu(h)) (either form), int8_linear((1 + s) * h + t), int8_linear((1 + s) * layer_norm(h) + t),
     int8_linear(rms_norm(h, w) [* (1 + s)] [+ t]), int8_linear(silu(h) * g) and int8_linear(cat((a, gelu_tanh(b)), -1))
-    (no dynamic-LoRA addend, producers used nowhere else) into int8_linear_prologue(h, ...).
-    Returns the number of layers rewritten."""
+    (no dynamic-LoRA addend, producers used nowhere else) into int8_linear_prologue(h, ...); the same producers in front
+    of a quantize_rowwise that several layers share (share_quantisation) into quantize_rowwise_prologue(h, ...).
+    Returns the number of consumers rewritten."""
     n_fused = 0
-    targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
+    lin_targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
+    quant_targets = (torch.ops.i8f.quantize_rowwise, torch.ops.i8f.quantize_rowwise.default)
     for node in list(gm.graph.nodes):
-        if not _is_call(node, *targets):
+        is_lin = _is_call(node, *lin_targets)
+        if not is_lin and not _is_call(node, *quant_targets):
             continue
-        args = list(node.args) + [node.kwargs.get("addend")] * (9 - len(node.args))
-        x_in, weight, ws_t, ws_v, bias, cdt, rotate, order, addend = args[:9]
-        if addend is not None or not isinstance(x_in, torch.fx.Node):
+        if is_lin:
+            args = list(node.args) + [node.kwargs.get("addend")] * (9 - len(node.args))
+            x_in, weight, ws_t, ws_v, bias, cdt, rotate, order, addend = args[:9]
+            if addend is not None:
+                continue
+        else:
+            x_in, rotate = node.args[0], node.args[1]
+        if not isinstance(x_in, torch.fx.Node):
             continue
         src = _through_views(x_in)
-        if not isinstance(src, torch.fx.Node):
-            continue
         x_shape = _meta_shape(x_in)
-        if x_shape is None:
+        if not isinstance(src, torch.fx.Node) or x_shape is None:
             continue
-        h = _match_gelu(src)
-        new_args, eps, norm_w = None, 1e-6, None
-        if h is not None:
-            new_args = (h, _lib.PRO_GELU_TANH, None, None)
-        elif _match_gelu_erf(src) is not None:
-            new_args = (_match_gelu_erf(src), _lib.PRO_GELU_ERF, None, None)
-        elif _match_rms_norm(src) is not None:                       # the norm alone
-            r = _match_rms_norm(src)
-            new_args, eps, norm_w = (r[0], _lib.PRO_RMS_NORM, None, None), r[2], r[1]
-        elif _match_scale_only(src) is not None and _match_rms_norm(_match_scale_only(src)[0]) is not None:
-            y, sc = _match_scale_only(src)                           # modulate(norm(x), scale) = norm(x) * (1 + scale)
-            r = _match_rms_norm(y)
-            if _vectors_broadcast_over_tokens(r[0], sc, sc):
-                new_args, eps, norm_w = (r[0], _lib.PRO_RMS_NORM, sc, None), r[2], r[1]
-        else:
-            m = _match_modulate(src)
-            g = _match_silu_gate(src) if m is None else None
-            c = _match_concat_gelu(src) if m is None and g is None else None
-            if m is not None and _vectors_broadcast_over_tokens(*m):
-                new_args = (m[0], _lib.PRO_MODULATE, m[1], m[2])
-                ln = _match_plain_layer_norm(m[0])   # the modulated tensor is a LayerNorm without affine: that goes in too
-                rn = _match_rms_norm(m[0]) if ln is None else None
-                if ln is not None:
-                    new_args, eps = (ln[0], _lib.PRO_NORM_MODULATE, m[1], m[2]), ln[1]
-                elif rn is not None and _vectors_broadcast_over_tokens(rn[0], m[1], m[2]):   # or an RMSNorm
-                    new_args, eps, norm_w = (rn[0], _lib.PRO_RMS_NORM, m[1], m[2]), rn[2], rn[1]
-            elif g is not None:
-                new_args = (g[0], _lib.PRO_SILU_GATE, g[1], None)
-            elif c is not None and not (rotate and (_meta_shape(c[0])[-1] % 128 or _meta_shape(c[1])[-1] % 128)):
-                new_args = (c[0], _lib.PRO_CONCAT_GELU, c[1], None)
-        if new_args is None:
+        found = _match_producer(src, rotate)
+        if found is None:
             continue
+        h, kind, mod_scale, mod_shift, eps, norm_w = found
         # The fused operator returns the leading shape of h, the original one that of x_in: the same when nothing
         # sat between them; a layer that flattened h to 2-D gets its 2-D result back by a reshape; anything else
         # (a direct caller with another regrouping of the rows) is left alone.
-        h_shape = _meta_shape(new_args[0])
+        h_shape = _meta_shape(h)
         if h_shape is None:
             continue
-        if new_args[1] == _lib.PRO_CONCAT_GELU:   # the layer's input is wider than h by the second tensor: compare the rows
-            if h_shape[-1] + _meta_shape(new_args[2])[-1] != x_shape[-1]:
+        if kind == _lib.PRO_CONCAT_GELU:   # the layer's input is wider than h by the second tensor: compare the rows
+            if h_shape[-1] + _meta_shape(mod_scale)[-1] != x_shape[-1]:
                 continue
             h_shape = (*h_shape[:-1], x_shape[-1])
         if h_shape[-1] != x_shape[-1]:
             continue
         if h_shape != x_shape and len(x_shape) != 2:
             continue
+        if not is_lin:   # the shared quantiser: its outputs are 2-D whatever h's leading dimensions are
+            with gm.graph.inserting_before(node):
+                fused = gm.graph.call_function(torch.ops.i8f.quantize_rowwise_prologue,
+                                               (h, rotate, kind, mod_scale, mod_shift, eps, norm_w))
+            node.replace_all_uses_with(fused)
+            gm.graph.erase_node(node)
+            n_fused += 1
+            continue
         with gm.graph.inserting_before(node):
             fused = gm.graph.call_function(torch.ops.i8f.int8_linear_prologue,
-                                           (*new_args, weight, ws_t, ws_v, bias, cdt, rotate, order, eps),
+                                           (h, kind, mod_scale, mod_shift, weight, ws_t, ws_v, bias, cdt, rotate, order, eps),
                                            {} if norm_w is None else {"norm_weight": norm_w})
             n_out, old = _out_features(weight), _meta_val(node)
             if old is not None:   # shapes for the passes that follow (the epilogue rewrite reads them)
@@ -411,6 +454,61 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
     return n_fused
 
 
+def share_quantisation(gm: torch.fx.GraphModule) -> int:
+    """Layers that read the same activations (separate q, k and v projections, the two up-projections of a SwiGLU
+    feed-forward) each quantise them, int8_linear being one operator: give every such group ONE quantize_rowwise and
+    its layers the GEMM operator on the shared int8 rows (bit-identical: the quantiser is a function of its input).
+    Shape-only steps between the shared tensor and the layers (each layer flattens its input) are looked through.
+    Returns the number of layers rewritten."""
+    lin_targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
+    groups = {}
+    for node in gm.graph.nodes:
+        if not _is_call(node, *lin_targets) or not isinstance(node.args[0], torch.fx.Node):
+            continue
+        x_val, y_val = _meta_val(node.args[0]), _meta_val(node)
+        if x_val is None or y_val is None or len(x_val.shape) < 1:
+            continue
+        src = _through_views(node.args[0])
+        groups.setdefault((src, bool(node.args[6])), []).append(node)
+    n_shared = 0
+    for (src, rotate), nodes in groups.items():
+        if len(nodes) < 2:
+            continue
+        first = nodes[0]                                   # (graph order: everything the group reads exists before it)
+        x_in = first.args[0]
+        x_val = _meta_val(x_in)
+        K = int(x_val.shape[-1])
+        rows = int(x_val.numel()) // max(1, K)
+        with gm.graph.inserting_before(first):
+            x2d = x_in
+            if len(x_val.shape) != 2:
+                x2d = _record(gm.graph.call_method("reshape", (x_in, -1, K)), (rows, K), x_val.dtype)
+            qs = gm.graph.call_function(torch.ops.i8f.quantize_rowwise, (x2d, rotate))
+            q = gm.graph.call_function(operator.getitem, (qs, 0))
+            s = gm.graph.call_function(operator.getitem, (qs, 1))
+        for node in nodes:
+            args = list(node.args) + [None] * (10 - len(node.args))
+            _, weight, ws_t, ws_v, bias, cdt, _, order, addend, gate = args[:10]
+            addend = node.kwargs.get("addend", addend)
+            gate = node.kwargs.get("gate", gate)
+            y_val = _meta_val(node)
+            n_out = int(y_val.shape[-1])
+            with gm.graph.inserting_before(node):
+                y = _record(gm.graph.call_function(torch.ops.i8f.linear_w8a8, (q, s, weight, ws_t, ws_v, bias, cdt, order),
+                                                   {"addend": addend, "gate": gate}), (rows, n_out), y_val.dtype)
+                restored = y
+                if tuple(y_val.shape) != (rows, n_out):
+                    restored = _record(gm.graph.call_method("reshape", (y, *(int(d) for d in y_val.shape))), y_val.shape, y_val.dtype)
+            node.replace_all_uses_with(restored)
+            gm.graph.erase_node(node)
+            n_shared += 1
+    if n_shared:
+        gm.graph.eliminate_dead_code()
+        gm.graph.lint()
+        gm.recompile()
+    return n_shared
+
+
 def _sole_user(node):
     return next(iter(node.users)) if len(node.users) == 1 else None
 
@@ -423,7 +521,8 @@ def fuse_epilogues(gm: torch.fx.GraphModule) -> int:
     (a dynamic-LoRA side tensor) are left alone.  Returns the number of layers rewritten."""
     n_fused = 0
     lin_targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default,
-                   torch.ops.i8f.int8_linear_prologue, torch.ops.i8f.int8_linear_prologue.default)
+                   torch.ops.i8f.int8_linear_prologue, torch.ops.i8f.int8_linear_prologue.default,
+                   torch.ops.i8f.linear_w8a8, torch.ops.i8f.linear_w8a8.default)
     for node in list(gm.graph.nodes):
         if not _is_call(node, *lin_targets):
             continue
@@ -492,15 +591,17 @@ def fuse_epilogues(gm: torch.fx.GraphModule) -> int:
 
 
 def _out_features(weight_node):
-    v = weight_node.meta.get("example_value", weight_node.meta.get("val"))
+    v = _meta_val(weight_node)
     if v is None:
         raise RuntimeError("the traced graph carries no shape for the weight")
     return int(v.shape[0])
 
 
 def backend(inner="inductor"):
-    """A torch.compile backend: fuse_prologues and fuse_epilogues, then `inner` (a registered backend name or a callable)."""
+    """A torch.compile backend: share_quantisation, fuse_prologues and fuse_epilogues, then `inner` (a registered backend
+    name or a callable)."""
     def compile_fn(gm, example_inputs):
+        share_quantisation(gm)
         fuse_prologues(gm)
         fuse_epilogues(gm)
         fn = inner

@@ -141,6 +141,60 @@ def forward_pair(layers, xs, gates=None, residuals=None):
                                                   xs[0].dtype, rotate=rot, gates=gates, residuals=residuals)
 
 
+def forward_fanout(layers, x, prologue: int = _lib.PRO_NONE, mod_scale=None, mod_shift=None, eps: float = 1e-6, norm_weight=None):
+    """[layer(x) for layer in layers] for quantised layers that read the same activations (separate q, k and v projections,
+    the two up-projections of a SwiGLU feed-forward): x is quantised ONCE -- with `prologue` and its operands applied
+    inside that quantiser, as forward(x, prologue=...) does for one layer -- and every layer runs its GEMM on the shared
+    int8 rows.  The reference quantises in every Linear.forward (int8_quant.py:703-778); the quantiser being a function
+    of its input, results are bit-identical to the layers' own forward calls, which is also the fall-back where a layer
+    is not on the W8A8 path (16 rows or fewer, dynamic LoRA, managed casting, different rotation flags, tracing)."""
+    layers = list(layers)
+    rot = bool(getattr(layers[0], "_use_quarot", False)) if layers else False
+    ok = len(layers) >= 2 and not torch.compiler.is_compiling() and x.is_cuda and x.dim() >= 2 \
+        and x.numel() // max(1, x.shape[-1]) > SMALL_BATCH_ROWS and x.dtype in (torch.float16, torch.bfloat16)
+    for lin in layers:
+        managed = lin.comfy_cast_weights or len(lin.weight_function) > 0 or len(lin.bias_function) > 0
+        ok = ok and (getattr(lin, "_is_quantized", False) and not managed and lin.lora_A is None and lin.weight.device == x.device
+                     and (lin.bias is None or lin.bias.device == x.device) and bool(getattr(lin, "_use_quarot", False)) == rot)
+    if ok and prologue != _lib.PRO_NONE:
+        # the checks of forward(): operands the quantiser does not take make every layer go alone (torch applies the operation)
+        if prologue == _lib.PRO_CONCAT_GELU:
+            ok = (isinstance(mod_scale, Tensor) and mod_scale.shape[:-1] == x.shape[:-1]
+                  and _lib.concat_gelu_fusable(x.reshape(-1, x.shape[-1]), mod_scale.reshape(-1, mod_scale.shape[-1]))
+                  and not (rot and (x.shape[-1] % 128 or mod_scale.shape[-1] % 128)))
+        elif prologue == _lib.PRO_SILU_GATE:
+            ok = isinstance(mod_scale, Tensor) and mod_scale.shape == x.shape and mod_scale.dtype == x.dtype
+        elif prologue in (_lib.PRO_MODULATE, _lib.PRO_NORM_MODULATE):
+            ok = (isinstance(mod_scale, Tensor) and isinstance(mod_shift, Tensor)
+                  and compile_ops.modulation_broadcasts_over_tokens(x, mod_scale, mod_shift)
+                  and (prologue == _lib.PRO_MODULATE or _lib.norm_modulate_fusable(x.reshape(-1, x.shape[-1]))))
+        elif prologue == _lib.PRO_RMS_NORM:
+            vecs = [v for v in (mod_scale, mod_shift) if v is not None]
+            ok = (_lib.norm_modulate_fusable(x.reshape(-1, x.shape[-1]))
+                  and (norm_weight is None or (norm_weight.dtype == x.dtype and tuple(norm_weight.shape) == (x.shape[-1],)
+                                               and norm_weight.device == x.device))
+                  and all(isinstance(v, Tensor) and v.device == x.device
+                          and compile_ops.modulation_broadcasts_over_tokens(x, v, v) for v in vecs))
+    width = x.shape[-1] + (mod_scale.shape[-1] if ok and prologue == _lib.PRO_CONCAT_GELU else 0)
+    ok = ok and all(lin.weight.shape[1] == width for lin in layers)
+    if not ok:
+        return [lin(x, prologue=prologue, mod_scale=mod_scale, mod_shift=mod_shift, eps=eps, norm_weight=norm_weight) for lin in layers]
+    lead = x.shape[:-1]
+    q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rot, prologue=prologue, mod_scale=mod_scale, mod_shift=mod_shift,
+                              eps=eps, norm_weight=norm_weight)
+    outs = []
+    for lin in layers:
+        ws = lin._get_weight_scale()
+        if isinstance(ws, Tensor):
+            if ws.device != x.device:
+                ws = ws.to(x.device, non_blocking=True)
+            if not lin._is_per_row and ws.numel() != 1:
+                ws = ws.reshape(-1)[:1]
+        y = _lib.linear_w8a8(q, s, lin.weight, ws, lin.bias, x.dtype, int8_fused_kernel.DEFAULT_EPILOGUE)
+        outs.append(y.reshape(*lead, lin.weight.shape[0]))
+    return outs
+
+
 # --------------------------------------------------------------------------- LoRA delta reconstruction
 def reconstruct_lora_diff(weights, target_shape, device, dtype, strength):
     """Float delta of a LoRA / LoHA / LoKr patch and its scalar multiplier (int8_quant.py:128-208).

@@ -52,6 +52,12 @@ def test_shape_only_implementations(pkg):
     y = ops.linear_w8a16_small_m(x[:1, :4], w, ws, 0.0, b, False)
     assert y.shape == (1, 4, 96) and y.dtype == torch.float16
     assert ops.rotate128(x.reshape(21, 256)).shape == (21, 256)
+    q, s = ops.quantize_rowwise_prologue(x, False, pkg._lib.PRO_GELU_ERF, None, None)
+    assert q.shape == (21, 256) and q.dtype == torch.int8 and s.shape == (21, 1)
+    q, s = ops.quantize_rowwise_prologue(x, False, pkg._lib.PRO_CONCAT_GELU, torch.empty(3, 7, 128, dtype=torch.float16, device="meta"), None)
+    assert q.shape == (21, 384)
+    y = ops.linear_w8a8(q[:, :256], s, w, ws, 0.0, None, torch.float16, 0, torch.empty(21, 96, dtype=torch.float16, device="meta"), b)
+    assert y.shape == (21, 96)
     with pytest.raises(Exception):
         ops.quantize_rowwise(x, False)     # 3-D input is rejected by the shape function as by the library
 
@@ -337,6 +343,63 @@ def test_graph_rewrite_moves_concatenation_and_gelu_into_the_quantiser(pkg):
             assert not any(n.target in (torch.cat, F.gelu) for n in gm.graph.nodes if n.op == "call_function")
 
 
+def test_graph_rewrite_gives_layers_that_read_one_tensor_a_single_quantiser(pkg):
+    """Separate q, k, v projections of one tensor: one quantize_rowwise and three GEMM operators instead of three
+    int8_linear.  A SwiGLU feed-forward behind an RMSNorm with modulation, w2(silu(w1(h)) * w3(h)) with
+    h = norm(x) * (1 + scale): w1 and w3 share one quantiser, which takes the norm and the modulation as its prologue
+    (the normalised tensor never exists), and w2 takes the gate as its own; layers with different rotation flags, or a
+    single layer, are left alone."""
+    g = torch.Generator().manual_seed(18)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    def calls(gm, name):
+        return [n for n in gm.graph.nodes if n.op == "call_function" and str(n.target).split(".")[-2 if str(n.target).endswith("default") else -1] == name]
+
+    class Qkv(torch.nn.Module):
+        def __init__(self, rot_k=False):
+            super().__init__()
+            self.q, self.k, self.v = lin(64, 128), lin(64, 128), lin(32, 128)
+            self.k._use_quarot = rot_k
+
+        def forward(self, x):
+            return self.q(x) + self.k(x), self.v(x)
+
+    x = torch.randn(2, 24, 128).bfloat16()
+    gm = torch._dynamo.export(Qkv())(x).graph_module
+    assert pkg.compile_ops.share_quantisation(gm) == 3
+    assert len(calls(gm, "quantize_rowwise")) == 1 and len(calls(gm, "linear_w8a8")) == 3 and not calls(gm, "int8_linear")
+    out = gm.graph.find_nodes(op="output")[0]
+    shapes = [tuple(pkg.compile_ops._meta_val(n).shape) for n in out.args[0]]
+    assert shapes == [(2, 24, 64), (2, 24, 32)]
+    gm = torch._dynamo.export(Qkv(rot_k=True))(x).graph_module     # k reads rotated activations: q and v share, k stays
+    assert pkg.compile_ops.share_quantisation(gm) == 2
+    assert len(calls(gm, "quantize_rowwise")) == 1 and len(calls(gm, "linear_w8a8")) == 2 and len(calls(gm, "int8_linear")) == 1
+
+    class SwiGlu(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = torch.nn.RMSNorm(128, eps=1e-5).bfloat16()
+            self.w1, self.w3, self.w2 = lin(256, 128), lin(256, 128), lin(128, 256)
+
+        def forward(self, x, scale):
+            h = self.norm(x) * (1 + scale)
+            return self.w2(F.silu(self.w1(h)) * self.w3(h))
+
+    gm = torch._dynamo.export(SwiGlu())(x, torch.randn(2, 1, 128).bfloat16()).graph_module
+    assert pkg.compile_ops.share_quantisation(gm) == 2
+    assert pkg.compile_ops.fuse_prologues(gm) == 2
+    quant = calls(gm, "quantize_rowwise_prologue")
+    assert len(quant) == 1 and quant[0].args[2] == pkg._lib.PRO_RMS_NORM and quant[0].args[3] is not None and quant[0].args[6] is not None
+    assert len(calls(gm, "linear_w8a8")) == 2 and not calls(gm, "quantize_rowwise")
+    down = calls(gm, "int8_linear_prologue")
+    assert len(down) == 1 and down[0].args[1] == pkg._lib.PRO_SILU_GATE
+    assert not any("rms_norm" in str(n.target) or n.target in (operator.mul, F.silu) for n in gm.graph.nodes if n.op == "call_function")
+
+
 def test_graph_rewrite_moves_the_gated_residual_into_the_epilogue(pkg):
     """x + gate * proj(h), the residual update of an adaLN-Zero block: multiplication and addition become the layer's
     epilogue (in any operand order); the gate alone and the residual alone are taken too; a gate of another dtype, a
@@ -589,6 +652,59 @@ def test_compiled_rms_norm_producer_and_exact_gelu_equal_eager_bit_for_bit(pkg, 
         assert torch.equal(got, want)
         loose = m(x, scale)
     assert (got.float() - loose.float()).abs().max().item() <= 2.0**-6 * loose.float().abs().max().item()
+
+
+@pytest.mark.gpu
+def test_compiled_swiglu_block_shares_one_quantiser_and_equals_eager(pkg, dev):
+    """x + tanh(gate) * w2(silu(w1(h)) * w3(h)), h = norm(x) * (1 + scale) with an RMSNorm (the feed-forward half of a
+    z-image block) and separate q / k / v projections of the same h, compiled with the rewriting backend over inductor:
+    the five layers that read h share ONE quantiser, which also normalises and modulates (h never exists), w2 takes the
+    gate as its prologue and the residual in its epilogue.  Equal to the eager fused calls bit for bit."""
+    g = torch.Generator().manual_seed(19)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = torch.nn.RMSNorm(256, eps=1e-5).bfloat16()
+            self.q, self.k, self.v = lin(128, 256), lin(64, 256), lin(64, 256)
+            self.w1, self.w3, self.w2 = lin(512, 256), lin(512, 256), lin(256, 512)
+
+        def forward(self, x, scale, gate):
+            h = self.norm(x) * (1 + scale)
+            y = x + gate.tanh() * self.w2(F.silu(self.w1(h)) * self.w3(h))
+            return y, self.q(h), self.k(h), self.v(h)
+
+    m = Block().to(dev)
+    with torch.no_grad():
+        m.norm.weight.copy_((torch.randn(256, generator=g) * 0.2 + 1).bfloat16())
+    x = (torch.randn(2, 40, 256, generator=g) * 2).bfloat16().to(dev)
+    scale, gate = ((torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev) for _ in range(2))
+    seen = []
+
+    def counting(gm, inputs):
+        names = [str(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum("quantize_rowwise" in t for t in names), sum("linear_w8a8" in t for t in names),
+                     sum("int8_linear_prologue" in t for t in names), sum("rms_norm" in t or "silu" in t for t in names)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    with torch.no_grad():
+        got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x, scale, gate)
+        assert seen == [(1, 5, 1, 0)]
+        L = pkg._lib
+        kw = dict(prologue=L.PRO_RMS_NORM, norm_weight=m.norm.weight, mod_scale=scale, eps=1e-5)
+        a, b, q, k, v = pkg.forward_fanout([m.w1, m.w3, m.q, m.k, m.v], x, **kw)
+        y = m.w2(a, prologue=L.PRO_SILU_GATE, mod_scale=b, gate=gate.tanh(), residual=x)
+        for have, want in zip(got, (y, q, k, v)):
+            assert torch.equal(have, want)
+        loose = m(x, scale, gate)
+    for have, want in zip(got, loose):
+        assert (have.float() - want.float()).abs().max().item() <= 2.0**-6 * want.float().abs().max().item()
 
 
 @pytest.mark.gpu

@@ -386,3 +386,40 @@ def test_forward_pair_equals_the_layers_own_forward(pkg, dev, quarot):
     assert torch.equal(o_img, g_img * y_img) and torch.equal(o_txt, r_txt + y_txt)
     o_img, o_small = pkg.forward_pair([img, txt], [x_img, small], gates=[g_img, g_txt[:1]], residuals=[r_img, r_txt[:1, :3]])
     assert torch.equal(o_img, r_img + g_img * y_img) and torch.equal(o_small, r_txt[:1, :3] + g_txt[:1] * txt(small))
+
+
+@pytest.mark.parametrize("quarot", [False, True])
+def test_forward_fanout_equals_the_layers_own_forward(pkg, dev, quarot):
+    """forward_fanout: layers that read the same activations (q, k, v of different widths) on ONE quantisation, bit-identical
+    to calling each layer; with a prologue applied inside that one quantiser (an RMSNorm with scale-only modulation in
+    front of a SwiGLU's two up-projections) bit-identical to each layer's own forward with that prologue; fall-backs
+    (a small batch, a layer with another rotation flag) give the layers' own results."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(37)
+    L = pkg._lib
+
+    def layer(n, k, per_row=True):
+        lin = pkg.Int8TensorwiseOps.Linear(k, n, bias=True)
+        lin._load_from_state_dict({"l.weight": torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g),
+                                   "l.weight_scale": (torch.rand(n, 1, generator=g) * 0.002 + 1e-3) if per_row else torch.tensor(0.0021),
+                                   "l.bias": torch.randn(n, generator=g).bfloat16()}, "l.", {}, True, [], [], [])
+        lin._use_quarot = quarot
+        return lin.to(dev)
+    q, k, v = layer(192, 384), layer(96, 384, per_row=False), layer(64, 384)
+    x = torch.randn(2, 50, 384, generator=g).bfloat16().to(dev)
+    outs = pkg.forward_fanout([q, k, v], x)
+    assert [tuple(o.shape) for o in outs] == [(2, 50, 192), (2, 50, 96), (2, 50, 64)]
+    assert all(torch.equal(o, lin(x)) for o, lin in zip(outs, (q, k, v)))
+    nw = (torch.randn(384, generator=g) * 0.2 + 1).bfloat16().to(dev)
+    sc = (torch.randn(2, 1, 384, generator=g) * 0.3).bfloat16().to(dev)
+    outs = pkg.forward_fanout([q, v], x, prologue=L.PRO_RMS_NORM, norm_weight=nw, mod_scale=sc, eps=1e-5)
+    assert all(torch.equal(o, lin(x, prologue=L.PRO_RMS_NORM, norm_weight=nw, mod_scale=sc, eps=1e-5)) for o, lin in zip(outs, (q, v)))
+    h = F.rms_norm(x, (384,), nw, 1e-5) * (1 + sc)
+    assert all((o.float() - lin(h).float()).abs().max() <= 2.0**-6 * lin(h).float().abs().max() for o, lin in zip(outs, (q, v)))
+    small = x[:1, :5]
+    assert all(torch.equal(o, lin(small)) for o, lin in zip(pkg.forward_fanout([q, k], small), (q, k)))
+    k._use_quarot = not quarot
+    assert all(torch.equal(o, lin(x)) for o, lin in zip(pkg.forward_fanout([q, k], x), (q, k)))
+    per_token = (torch.randn(1, 50, 384, generator=g) * 0.3).bfloat16().to(dev)      # a scale torch would broadcast differently
+    outs = pkg.forward_fanout([q, v], x, prologue=L.PRO_RMS_NORM, norm_weight=nw, mod_scale=per_token, eps=1e-5)
+    assert all(torch.equal(o, lin(F.rms_norm(x, (384,), nw, 1e-5) * (1 + per_token))) for o, lin in zip(outs, (q, v)))
