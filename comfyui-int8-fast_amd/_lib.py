@@ -215,9 +215,9 @@ def quant_rowwise_concat_gelu(a: torch.Tensor, b: torch.Tensor, rotate: bool = F
 
 
 def norm_modulate_fusable(x: torch.Tensor) -> bool:
-    """Whether the quantiser takes PRO_NORM_MODULATE for these rows (one wavefront holds a row): 16-bit elements,
-    a width of at most 4096 in multiples of 16, 16-byte aligned rows."""
-    return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and x.dim() == 2 and 0 < x.shape[1] <= 4096 and x.shape[1] % 16 == 0
+    """Whether the quantiser takes PRO_NORM_MODULATE for these rows (the row stays in the registers of one to four wavefronts): 16-bit elements,
+    a width of at most 16384 in multiples of 16, 16-byte aligned rows."""
+    return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and x.dim() == 2 and 0 < x.shape[1] <= 16384 and x.shape[1] % 16 == 0
             and x.stride(1) == 1 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0)
 
 
@@ -227,7 +227,7 @@ def quant_rowwise_rms_norm(x: torch.Tensor, eps: float = 1e-6, weight=None, mod_
     describes; weight [K]; mod_scale / mod_shift [V,K] (or [K]), M // V consecutive rows to a vector; each optional."""
     _dev(x, "x")
     if not norm_modulate_fusable(x):
-        raise ValueError("the normalising quantiser takes contiguous 16-bit rows of at most 4096 elements in multiples of 16 "
+        raise ValueError("the normalising quantiser takes contiguous 16-bit rows of at most 16384 elements in multiples of 16 "
                          "(see norm_modulate_fusable); normalise with torch")
     M, K = x.shape
     if rotate and K % 128:
@@ -284,7 +284,7 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
     rows_per_vec = 1
     if prologue in (PRO_MODULATE, PRO_SILU_GATE, PRO_NORM_MODULATE):
         if prologue == PRO_NORM_MODULATE and not norm_modulate_fusable(x):
-            raise ValueError("PRO_NORM_MODULATE takes contiguous 16-bit rows of at most 4096 elements in multiples of 16 "
+            raise ValueError("PRO_NORM_MODULATE takes contiguous 16-bit rows of at most 16384 elements in multiples of 16 "
                              "(see norm_modulate_fusable); normalise with torch and use PRO_MODULATE")
         vecs = []
         if prologue == PRO_SILU_GATE:

@@ -289,7 +289,7 @@ def _match_rms_norm(node):
     if v is None or v.dtype not in (torch.bfloat16, torch.float16) or len(v.shape) < 2:
         return None
     K = int(v.shape[-1])
-    if tuple(int(d) for d in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,))) != (K,) or K % 16 or K > 4096:
+    if tuple(int(d) for d in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,))) != (K,) or K % 16 or K > 16384:
         return None
     if w is not None:
         vw = _meta_val(w)
@@ -316,7 +316,7 @@ def _match_plain_layer_norm(node):
     if v is None or v.dtype not in (torch.bfloat16, torch.float16):
         return None
     K = int(v.shape[-1])
-    if tuple(int(d) for d in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,))) != (K,) or K % 16 or K > 4096:
+    if tuple(int(d) for d in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,))) != (K,) or K % 16 or K > 16384:
         return None
     eps = a.get("eps", 1e-5)
     return (h, float(eps)) if isinstance(eps, (int, float)) else None

@@ -501,13 +501,28 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
     {
         float v[RUNS][16];
         float amax = 0.0f;
+        // A row's sum for the normalising prologues: over the wave, then (four waves to a row) over the waves' partial
+        // sums through LDS, always in the same order, so that launches agree bit for bit.  Two slots: the second sum
+        // of a LayerNorm may be written while a slower wave still reads the first.
+        [[maybe_unused]] __shared__ float row_sums[2][ROWS][WPR];
+        [[maybe_unused]] auto row_sum = [&](float part, int slot) {
+            part = wave_sum_all(part);
+            if constexpr (WPR > 1) {
+                if ((t & 63) == 0) row_sums[slot][rb][t / 64] = part;
+                __syncthreads();
+                part = row_sums[slot][rb][0];
+#pragma unroll
+                for (int w = 1; w < WPR; ++w) part += row_sums[slot][rb][w];
+            }
+            return part;
+        };
         [[maybe_unused]] int64_t vrow = 0;  // the row's pair of modulation vectors (M < 2^31: a 32-bit division)
         if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_SILU_GATE || PRO == I8F_PRO_NORM_MODULATE || PRO == I8F_PRO_RMS_NORM)
             vrow = (uint32_t)(FULL || m < M ? m : 0) / (uint32_t)pro.rows_per_vec;
         if constexpr (PRO == I8F_PRO_NORM_MODULATE) {
             // LayerNorm without affine over the row, which this wave holds whole: mean, then the variance of the
             // differences (two passes over registers), y = (x - mean) / sqrt(var + eps) rounded to the dtype.
-            static_assert(WPR == 1 && SEG == 1, "the row's statistics are taken by the one wave that holds it");
+            static_assert(SEG == 1, "the row's statistics are taken by the waves that hold it whole");
             float sum = 0.0f;
 #pragma unroll
             for (int r = 0; r < RUNS; ++r) {
@@ -515,7 +530,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
 #pragma unroll
                 for (int j = 0; j < 16; ++j) sum += v[r][j];
             }
-            const float mean = wave_sum_all(sum) / (float)K;
+            const float mean = row_sum(sum, 0) / (float)K;
             float ss = 0.0f;
 #pragma unroll
             for (int r = 0; r < RUNS; ++r) {
@@ -527,7 +542,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
                     ss += in ? d * d : 0.0f;
                 }
             }
-            const float rstd = 1.0f / sqrtf(wave_sum_all(ss) / (float)K + pro.eps);
+            const float rstd = 1.0f / sqrtf(row_sum(ss, 1) / (float)K + pro.eps);
 #pragma unroll
             for (int r = 0; r < RUNS; ++r)
 #pragma unroll
@@ -536,7 +551,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
         if constexpr (PRO == I8F_PRO_RMS_NORM) {
             // RMSNorm over the row, which this wave holds whole: y = x / sqrt(sum x^2 / K + eps) * w in binary32, rounded
             // once to the dtype (torch's rms_norm); then the modulation's operations, each rounded, where s / t exist.
-            static_assert(WPR == 1 && SEG == 1, "the row's statistics are taken by the one wave that holds it");
+            static_assert(SEG == 1, "the row's statistics are taken by the waves that hold it whole");
             float ss = 0.0f;
 #pragma unroll
             for (int r = 0; r < RUNS; ++r) {
@@ -544,7 +559,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
 #pragma unroll
                 for (int j = 0; j < 16; ++j) ss = __builtin_fmaf(v[r][j], v[r][j], ss);
             }
-            const float rstd = 1.0f / sqrtf(wave_sum_all(ss) / (float)K + pro.eps);
+            const float rstd = 1.0f / sqrtf(row_sum(ss, 0) / (float)K + pro.eps);
 #pragma unroll
             for (int r = 0; r < RUNS; ++r) {
                 const int R = r * TPR + p;
@@ -923,11 +938,11 @@ int dispatch(const void *x, int64_t M, int64_t K, int64_t ldx, int8_t *q, float 
         const int64_t nruns = K / 16;
         if (aligned && K % 16 == 0 && (uintptr_t)q % 16 == 0 && nruns >= 1 && nruns <= 64 * 4 * 4) {
             if (nruns <= 64 * 4) return pick_runs16<DT, ROT, 1, PRO>((int)((nruns + 63) / 64), x, M, K, ldx, q, scale, st, pro);
-            if constexpr (PRO != I8F_PRO_NORM_MODULATE && PRO != I8F_PRO_RMS_NORM) return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
+            return pick_runs16<DT, ROT, 4, PRO>((int)((nruns + 255) / 256), x, M, K, ldx, q, scale, st, pro);
         }
     }
-    // the normalising prologue exists where one wave holds the row: 16-bit rows of up to 4096 aligned elements;
-    // the concatenating one where the row stays in registers: 16-bit rows of up to 16384 aligned elements
+    // the normalising and the concatenating prologues exist where the row stays in registers: 16-bit rows of up to
+    // 16384 aligned elements
     if constexpr (PRO == I8F_PRO_NORM_MODULATE || PRO == I8F_PRO_RMS_NORM || PRO == I8F_PRO_CONCAT_GELU) return I8F_ERR_UNSUPPORTED;
     else {
     if constexpr (PRO == I8F_PRO_NONE) {  // the chunked kernels have no prologue form: such shapes take the generic kernel

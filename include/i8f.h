@@ -172,9 +172,9 @@ int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K,
  * torch's LayerNorm takes its sums in another order and its reciprocal square root from the
  * hardware, so y agrees with it to the last place of the dtype (tests state the tolerance).
  *   mod_scale, mod_shift, rows_per_vec: as for I8F_PRO_MODULATE.
- * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 4096 and x, q and
- * the vectors are 16-byte aligned (one wavefront holds a row): other callers normalise with their
- * own kernel and use I8F_PRO_MODULATE.
+ * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 16384 and x, q and
+ * the vectors are 16-byte aligned (the row stays in the registers of one to four wavefronts): other callers
+ * normalise with their own kernel and use I8F_PRO_MODULATE.
  */
 int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                                     float eps, const void *mod_scale, const void *mod_shift,
@@ -197,8 +197,8 @@ int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64
  * dtype (tests state the tolerance).
  *   weight [K] of x_dtype or NULL; mod_scale, mod_shift [ceil(M / rows_per_vec), K] of x_dtype or NULL each;
  *   rows_per_vec as for I8F_PRO_MODULATE (ignored when both are NULL).
- * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 4096 and x, q and the vectors are
- * 16-byte aligned (one wavefront holds a row): other callers normalise with their own kernel.
+ * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 16384 and x, q and the vectors are
+ * 16-byte aligned (the row stays in the registers of one to four wavefronts): other callers normalise with their own kernel.
  */
 int i8f_quant_rowwise_rms_norm(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, float eps,
                                const void *weight, const void *mod_scale, const void *mod_shift,

@@ -213,7 +213,7 @@ def test_graph_rewrite_moves_the_swiglu_gate_into_the_quantiser(pkg):
 def test_graph_rewrite_moves_layer_norm_and_modulation_into_the_quantiser(pkg):
     """(1 + scale) * LayerNorm(h) + shift -> linear, the adaLN producer of a DiT block: LayerNorm without affine goes into
     the quantiser together with the modulation (with its eps); a LayerNorm with affine parameters, one that is used
-    elsewhere too, or rows wider than a wavefront holds stay torch's and only the modulation is fused."""
+    elsewhere too, or rows wider than the registers hold (16384) stay torch's and only the modulation is fused."""
     g = torch.Generator().manual_seed(13)
 
     def lin(n_out, k_in):
@@ -242,7 +242,7 @@ def test_graph_rewrite_moves_layer_norm_and_modulation_into_the_quantiser(pkg):
 
     node, ln_left = fused_nodes(Block(256), 256)
     assert node.args[1] == pkg._lib.PRO_NORM_MODULATE and not ln_left and abs(node.args[-1] - 1e-6) < 1e-12
-    for mod, k in ((Block(256, affine=True), 256), (Block(256, reuse=True), 256), (Block(8192), 8192)):
+    for mod, k in ((Block(256, affine=True), 256), (Block(256, reuse=True), 256), (Block(16400), 16400)):
         node, ln_left = fused_nodes(mod, k)
         assert node.args[1] == pkg._lib.PRO_MODULATE and ln_left
 
@@ -251,7 +251,7 @@ def test_graph_rewrite_moves_rms_norm_and_exact_gelu_into_the_quantiser(pkg):
     """rms_norm(h, w) * (1 + scale) -> linear (z-image's modulate(norm(x), scale)), (1 + scale) * rms_norm(h) + shift ->
     linear (ltx), a bare rms_norm -> linear, and gelu(h) in its exact form -> linear: all become the layer's prologue,
     the weight of the norm travelling as the operator's norm_weight; an RMSNorm whose weight has another dtype, one used
-    elsewhere too, or rows wider than a wavefront holds stay torch's."""
+    elsewhere too, or rows wider than the registers hold (16384) stay torch's."""
     g = torch.Generator().manual_seed(14)
 
     def lin(n_out, k_in):
@@ -289,7 +289,7 @@ def test_graph_rewrite_moves_rms_norm_and_exact_gelu_into_the_quantiser(pkg):
         assert node.args[1] == pkg._lib.PRO_RMS_NORM and abs(node.args[11] - 1e-5) < 1e-12
         assert (node.kwargs.get("norm_weight") is not None) == has_w
         assert (node.args[2] is not None) == has_s and (node.args[3] is not None) == has_t
-    for mod, k in ((Block(256, "zimage", torch.float32), 256), (Block(256, "reuse"), 256), (Block(8192, "zimage"), 8192)):
+    for mod, k in ((Block(256, "zimage", torch.float32), 256), (Block(256, "reuse"), 256), (Block(16400, "zimage"), 16400)):
         n, nodes, norm_left = rewrite(mod, k)
         assert n == 0 and norm_left
 

@@ -188,7 +188,8 @@ def test_quant_rowwise_silu_gate_prologue_within_tolerance(L, dev, M, K, dt, rot
 @pytest.mark.parametrize("M,K,dt,rot,V,eps", [
     (64, 3072, torch.bfloat16, False, 1, 1e-6), (48, 3072, torch.bfloat16, True, 2, 1e-6), (33, 4096, torch.float16, False, 3, 1e-5),
     (10, 1008, torch.bfloat16, False, 2, 1e-6), (6, 384, torch.float16, True, 1, 1e-5), (5, 16, torch.bfloat16, False, 1, 1e-6),
-    (4608, 3072, torch.bfloat16, False, 1, 1e-6),
+    (4608, 3072, torch.bfloat16, False, 1, 1e-6), (40, 5120, torch.bfloat16, False, 2, 1e-6), (9, 16384, torch.float16, True, 1, 1e-5),
+    (6, 4112, torch.bfloat16, False, 1, 1e-6),
 ])
 def test_quant_rowwise_norm_modulate_prologue_within_tolerance(L, dev, M, K, dt, rot, V, eps):
     """LayerNorm (no affine) and the adaLN modulation inside the quantiser (i8f_quant_rowwise_norm_modulate) against the
@@ -240,7 +241,8 @@ def test_quant_rowwise_gelu_erf_prologue_within_tolerance(L, dev, M, K, dt, rot,
 @pytest.mark.parametrize("M,K,dt,rot,V,eps,parts", [
     (64, 3072, torch.bfloat16, False, 1, 1e-6, "wst"), (48, 3072, torch.bfloat16, True, 2, 1e-6, "ws"), (33, 4096, torch.float16, False, 3, 1e-5, "w"),
     (10, 1008, torch.bfloat16, False, 2, 1e-6, "st"), (6, 384, torch.float16, True, 1, 1e-5, ""), (5, 16, torch.bfloat16, False, 1, 1e-6, "wt"),
-    (4608, 3840, torch.bfloat16, False, 1, 1e-5, "ws"),
+    (4608, 3840, torch.bfloat16, False, 1, 1e-5, "ws"), (40, 5120, torch.bfloat16, False, 2, 1e-6, "wst"), (9, 16384, torch.float16, True, 1, 1e-5, "ws"),
+    (6, 4112, torch.bfloat16, False, 1, 1e-6, "w"),
 ])
 def test_quant_rowwise_rms_norm_prologue_within_tolerance(L, dev, M, K, dt, rot, V, eps, parts):
     """RMSNorm with its weight and the modulation behind it inside the quantiser (i8f_quant_rowwise_rms_norm; each of
@@ -276,13 +278,13 @@ def test_quant_rowwise_rms_norm_prologue_within_tolerance(L, dev, M, K, dt, rot,
 
 
 def test_quant_rowwise_norm_modulate_refuses_rows_it_does_not_take(L, dev):
-    s = torch.zeros(1, 8192, dtype=torch.bfloat16, device=dev)
+    s = torch.zeros(1, 16400, dtype=torch.bfloat16, device=dev)
     with pytest.raises(ValueError):
-        L.quant_rowwise(torch.zeros(4, 8192, dtype=torch.bfloat16, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s, mod_shift=s)
+        L.quant_rowwise(torch.zeros(4, 16400, dtype=torch.bfloat16, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s, mod_shift=s)
     with pytest.raises(ValueError):
         L.quant_rowwise(torch.zeros(4, 256, device=dev), prologue=L.PRO_NORM_MODULATE, mod_scale=s[:, :256].float(), mod_shift=s[:, :256].float())
     with pytest.raises(ValueError):
-        L.quant_rowwise(torch.zeros(4, 8192, dtype=torch.bfloat16, device=dev), prologue=L.PRO_RMS_NORM)
+        L.quant_rowwise(torch.zeros(4, 16400, dtype=torch.bfloat16, device=dev), prologue=L.PRO_RMS_NORM)
     with pytest.raises(ValueError):
         L.quant_rowwise(torch.zeros(4, 256, dtype=torch.bfloat16, device=dev), prologue=L.PRO_RMS_NORM, norm_weight=s[0, :128])
 
