@@ -10,6 +10,7 @@ the namespace `i8f` with a shape-only ("fake") implementation:
     torch.ops.i8f.int8_linear           <- triton_int8_linear[_per_row]         (int8_fused_kernel.py:179-235, 330-372)
     torch.ops.i8f.linear_w8a16_small_m  <- the M <= 16 branch of Linear.forward (int8_quant.py:756-760)
     torch.ops.i8f.rotate128             <- rotate_activation                    (quarot.py:73-102)
+    torch.ops.i8f.int8_linear_lora      <- the same with the dynamic-LoRA side branch formed in the epilogue (int8_quant.py:762-774)
     torch.ops.i8f.int8_linear_prologue  <- int8_linear with the elementwise operation in front of the layer
                                            (adaLN modulation, tanh-GELU) applied inside the quantiser: what
                                            torch.compile's fusion into the Triton quantiser gives the reference
@@ -114,6 +115,25 @@ def _(x, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, 
     return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
 
 
+@torch.library.custom_op(f"{NAMESPACE}::int8_linear_lora", mutates_args=())
+def int8_linear_lora(x: Tensor, weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
+                     bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int,
+                     side_t: Tensor, side_b: Tensor, alpha: Optional[float] = None) -> Tensor:
+    """int8_linear plus the dynamic-LoRA side branch (int8_quant.py:762-774 of the reference): side_t [rows, r] is the
+    first low-rank product x @ A.T, side_b [N, r] the second factor; their product, the scaling by alpha and the sum
+    with the main result happen inside the GEMM epilogue, so the [rows, N] side tensor never exists."""
+    lead = x.shape[:-1]
+    q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate)
+    y = _lib.linear_w8a8_lora(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, side_t, side_b, alpha,
+                              compute_dtype, order)
+    return y.reshape(*lead, weight.shape[0])
+
+
+@int8_linear_lora.register_fake
+def _(x, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, side_t, side_b, alpha=None):
+    return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=compute_dtype)
+
+
 @torch.library.custom_op(f"{NAMESPACE}::linear_w8a16_small_m", mutates_args=())
 def linear_w8a16_small_m(x: Tensor, weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
                          bias: Optional[Tensor], rotate: bool) -> Tensor:
@@ -153,8 +173,8 @@ def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_valu
     return x.new_empty((*x.shape[:-1], width), dtype=compute_dtype)
 
 
-OPS = ("quantize_rowwise", "quantize_rowwise_prologue", "rotate128", "linear_w8a8", "int8_linear", "linear_w8a16_small_m",
-       "int8_linear_prologue")
+OPS = ("quantize_rowwise", "quantize_rowwise_prologue", "rotate128", "linear_w8a8", "int8_linear", "int8_linear_lora",
+       "linear_w8a16_small_m", "int8_linear_prologue")
 
 
 # --------------------------------------------------------------------------- graph rewrite

@@ -633,7 +633,8 @@ class Int8TensorwiseOps(manual_cast):
                     x_side = _lib.rotate128(x_2d)
                 x_side = x_side.to(lA.dtype)
                 rows = x_2d.shape[0]
-                if (not compiling and rows > SMALL_BATCH_ROWS and lB.dtype == lA.dtype
+                if (rows > SMALL_BATCH_ROWS and lB.dtype == lA.dtype
+                        and (self.lora_alpha is None or isinstance(self.lora_alpha, (int, float)))
                         and _lib.lora_side_fusable(rows, weight.shape[0], weight.shape[1], lA.shape[0], compute_dtype, lA.dtype)):
                     # (the first product stays with torch: it is bound by the same per-CU load path whoever issues the
                     # loads, and an own kernel for it measured no faster than the BLAS library's 9.5 us at 4608 x 3072)
@@ -645,10 +646,15 @@ class Int8TensorwiseOps(manual_cast):
 
             if x_2d.shape[0] > SMALL_BATCH_ROWS:
                 addend = None if side is None else side.to(compute_dtype)
-                if compiling:  # under torch.compile the call goes through the registered operator
+                if compiling:  # under torch.compile the call goes through the registered operators
                     ws_t, ws_v = compile_ops.split_scale(w_scale)
-                    y = torch.ops.i8f.int8_linear(x_2d, weight, ws_t, ws_v, bias, compute_dtype, rotate,
-                                                  int8_fused_kernel.DEFAULT_EPILOGUE, addend)
+                    if side_factors is not None:
+                        alpha = None if self.lora_alpha is None else float(self.lora_alpha)
+                        y = torch.ops.i8f.int8_linear_lora(x_2d, weight, ws_t, ws_v, bias, compute_dtype, rotate,
+                                                           int8_fused_kernel.DEFAULT_EPILOGUE, side_factors[0], lB, alpha)
+                    else:
+                        y = torch.ops.i8f.int8_linear(x_2d, weight, ws_t, ws_v, bias, compute_dtype, rotate,
+                                                      int8_fused_kernel.DEFAULT_EPILOGUE, addend)
                 else:
                     fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
                     pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift, eps, norm_weight)

@@ -52,6 +52,9 @@ def test_shape_only_implementations(pkg):
     y = ops.linear_w8a16_small_m(x[:1, :4], w, ws, 0.0, b, False)
     assert y.shape == (1, 4, 96) and y.dtype == torch.float16
     assert ops.rotate128(x.reshape(21, 256)).shape == (21, 256)
+    y = ops.int8_linear_lora(x, w, ws, 0.0, b, torch.float16, False, 0, torch.empty(21, 8, dtype=torch.float16, device="meta"),
+                             torch.empty(96, 8, dtype=torch.float16, device="meta"), 0.5)
+    assert y.shape == (3, 7, 96) and y.dtype == torch.float16
     q, s = ops.quantize_rowwise_prologue(x, False, pkg._lib.PRO_GELU_ERF, None, None)
     assert q.shape == (21, 256) and q.dtype == torch.int8 and s.shape == (21, 1)
     q, s = ops.quantize_rowwise_prologue(x, False, pkg._lib.PRO_CONCAT_GELU, torch.empty(3, 7, 128, dtype=torch.float16, device="meta"), None)
@@ -705,6 +708,39 @@ def test_compiled_swiglu_block_shares_one_quantiser_and_equals_eager(pkg, dev):
         loose = m(x, scale, gate)
     for have, want in zip(got, loose):
         assert (have.float() - want.float()).abs().max().item() <= 2.0**-6 * want.float().abs().max().item()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quarot", [False, True])
+def test_compiled_dynamic_lora_takes_the_side_branch_in_the_epilogue(pkg, dev, quarot):
+    """A layer with dynamic LoRA factors under torch.compile: the traced graph holds the first low-rank product and ONE
+    operator that forms the second product, the scaling and the sum inside the GEMM epilogue (no [rows, N] side tensor),
+    as the eager path does; result equal to eager's, which the module tests hold to the reference's expression."""
+    g = torch.Generator().manual_seed(23)
+    lin = pkg.Int8TensorwiseOps.Linear(384, 256, bias=True)
+    _load(lin, {"weight": torch.randint(-127, 128, (256, 384), dtype=torch.int8, generator=g),
+                "weight_scale": torch.rand(256, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(256, generator=g) * 0.1).bfloat16()})
+    lin = lin.to(dev)
+    lin._use_quarot = quarot
+    lin.lora_A = (torch.randn(16, 384, generator=g) * 0.05).bfloat16().to(dev)
+    lin.lora_B = (torch.randn(256, 16, generator=g) * 0.05).bfloat16().to(dev)
+    lin.lora_alpha = 0.5
+    x = torch.randn(2, 30, 384, generator=g).bfloat16().to(dev)
+    seen = []
+
+    def counting(gm, inputs):
+        names = [str(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum("int8_linear_lora" in t for t in names), sum(t.endswith("int8_linear.default") or t.endswith("int8_linear") for t in names)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    with torch.no_grad():
+        got = torch.compile(lin, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x)
+        want = lin(x)
+    assert seen == [(1, 0)]
+    assert got.shape == (2, 30, 256)
+    assert (got.float() - want.float()).abs().max().item() <= 2.0**-8 * want.float().abs().max().item()
+    assert (got != want).float().mean().item() < 0.01      # (the first product is the BLAS library's in both runs)
 
 
 @pytest.mark.gpu
