@@ -363,6 +363,33 @@ def modulation_broadcasts_over_tokens(x, scale, shift) -> bool:
     return len(ss) == len(xs) and ss[-1] == xs[-1] and ss[-2] == 1 and ss[:-2] == xs[:-2]
 
 
+_INPLACE_FUNCTIONS = tuple(getattr(operator, n) for n in ("iadd", "isub", "imul", "itruediv", "ifloordiv", "imod", "ipow", "iand", "ior",
+                                                          "ixor", "ilshift", "irshift", "imatmul", "setitem"))
+
+
+def _writes_in_place(node) -> bool:
+    """Whether a traced node may overwrite one of its tensor operands: an in-place method (name ending in an underscore),
+    an augmented assignment or an item assignment, or an `out=` argument."""
+    if node.op == "call_method":
+        return node.target.endswith("_") and not node.target.endswith("__")
+    if node.op == "call_function":
+        name = getattr(node.target, "__name__", "")
+        return node.target in _INPLACE_FUNCTIONS or (name.endswith("_") and not name.endswith("__")) or "out" in node.kwargs
+    return False
+
+
+def _in_place_write_between(first, last) -> bool:
+    """True if a node that may write in place sits between `first` and `last` in graph order.  The rewrites move a read of
+    a tensor from where the model reads it to where the fused operator runs; with a write in between they would read
+    another value, so they leave such stretches alone (inference graphs rarely have any)."""
+    node = first.next
+    while node is not last and node.op != "root":
+        if _writes_in_place(node):
+            return True
+        node = node.next
+    return False
+
+
 def _match_producer(src, rotate):
     """The producer of a layer's activations as a prologue kind -> (h, kind, mod_scale, mod_shift, eps, norm_weight)
     nodes / values, or None.  Every node matched is used nowhere else."""
@@ -409,6 +436,7 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
     n_fused = 0
     lin_targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default)
     quant_targets = (torch.ops.i8f.quantize_rowwise, torch.ops.i8f.quantize_rowwise.default)
+    order_of = {n: i for i, n in enumerate(gm.graph.nodes)}
     for node in list(gm.graph.nodes):
         is_lin = _is_call(node, *lin_targets)
         if not is_lin and not _is_call(node, *quant_targets):
@@ -430,6 +458,9 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         if found is None:
             continue
         h, kind, mod_scale, mod_shift, eps, norm_w = found
+        earliest = min((n for n in (h, mod_scale, mod_shift, norm_w) if isinstance(n, torch.fx.Node)), key=lambda n: order_of.get(n, 1 << 30))   # (nodes this pass created sit where a later node was)
+        if _in_place_write_between(earliest, node):
+            continue
         # The fused operator returns the leading shape of h, the original one that of x_in: the same when nothing
         # sat between them; a layer that flattened h to 2-D gets its 2-D result back by a reshape; anything else
         # (a direct caller with another regrouping of the rows) is left alone.
@@ -495,6 +526,8 @@ def share_quantisation(gm: torch.fx.GraphModule) -> int:
         if len(nodes) < 2:
             continue
         first = nodes[0]                                   # (graph order: everything the group reads exists before it)
+        if _in_place_write_between(first, nodes[-1]):      # the later layers might read another value than the first
+            continue
         x_in = first.args[0]
         x_val = _meta_val(x_in)
         K = int(x_val.shape[-1])
@@ -593,6 +626,8 @@ def fuse_epilogues(gm: torch.fx.GraphModule) -> int:
             continue
         final_shape = _meta_shape(last)
         if final_shape is None or final_shape[-1] != y_val.shape[-1]:
+            continue
+        if _in_place_write_between(node, last):   # the layer would run later than the model ran it
             continue
         with gm.graph.inserting_before(last):
             kwargs = dict(node.kwargs)

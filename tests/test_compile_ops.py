@@ -403,6 +403,48 @@ def test_graph_rewrite_gives_layers_that_read_one_tensor_a_single_quantiser(pkg)
     assert not any("rms_norm" in str(n.target) or n.target in (operator.mul, F.silu) for n in gm.graph.nodes if n.op == "call_function")
 
 
+def test_graph_rewrites_keep_away_from_in_place_writes(pkg):
+    """A tensor overwritten in place between the point where the model reads it and the layer that would read it inside
+    a fused operator: the rewrites leave that stretch of the graph alone (the fused read would see the new value)."""
+    g = torch.Generator().manual_seed(20)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Mlp(torch.nn.Module):
+        def __init__(self, clobber):
+            super().__init__()
+            self.up, self.down, self.clobber = lin(128, 64), lin(64, 128), clobber
+
+        def forward(self, x):
+            h = self.up(x)
+            a = F.gelu(h, approximate="tanh")
+            if self.clobber:
+                h.mul_(2.0)
+            return self.down(a), h
+
+    class Qk(torch.nn.Module):
+        def __init__(self, clobber):
+            super().__init__()
+            self.q, self.k, self.clobber = lin(64, 64), lin(64, 64), clobber
+
+        def forward(self, x):
+            x = x * 1.0
+            a = self.q(x)
+            if self.clobber:
+                x += 1.0
+            return a, self.k(x)
+
+    x = torch.randn(2, 24, 64).bfloat16()
+    for clobber, fused in ((False, 1), (True, 0)):
+        gm = torch._dynamo.export(Mlp(clobber))(x).graph_module
+        assert pkg.compile_ops.fuse_prologues(gm) == fused
+        gm = torch._dynamo.export(Qk(clobber))(x).graph_module
+        assert pkg.compile_ops.share_quantisation(gm) == 2 * fused
+
+
 def test_graph_rewrite_moves_the_gated_residual_into_the_epilogue(pkg):
     """x + gate * proj(h), the residual update of an adaLN-Zero block: multiplication and addition become the layer's
     epilogue (in any operand order); the gate alone and the residual alone are taken too; a gate of another dtype, a
