@@ -786,6 +786,48 @@ def test_compiled_dynamic_lora_takes_the_side_branch_in_the_epilogue(pkg, dev, q
 
 
 @pytest.mark.gpu
+def test_compiled_shared_quantiser_with_a_gated_residual_on_one_layer(pkg, dev):
+    """Two layers read one tensor and the first one's result goes into res + gate * y: the rewriting backend shares the
+    quantiser (two GEMM operators) and still folds the gated residual into the first GEMM's epilogue; equal to the
+    eager calls bit for bit."""
+    g = torch.Generator().manual_seed(21)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+
+    class Two(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.b = lin(256, 256), lin(128, 256)
+
+        def forward(self, x, res, gate):
+            return res + gate * self.a(x), self.b(x)
+
+    m = Two().to(dev)
+    x = torch.randn(2, 40, 256, generator=g).bfloat16().to(dev)
+    res = torch.randn(2, 40, 256, generator=g).bfloat16().to(dev)
+    gate = (torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev)
+    seen = []
+
+    def counting(gm, inputs):
+        calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum("quantize_rowwise" in str(n.target) for n in calls),
+                     sum("linear_w8a8" in str(n.target) and n.kwargs.get("gate") is not None and n.kwargs.get("addend") is not None for n in calls),
+                     sum("linear_w8a8" in str(n.target) for n in calls),
+                     sum(n.target in (operator.mul, operator.add) for n in calls)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    with torch.no_grad():
+        got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x, res, gate)
+        assert seen == [(1, 1, 2, 0)]
+        assert torch.equal(got[0], m.a(x, gate=gate, residual=res)) and torch.equal(got[1], m.b(x))
+        assert torch.equal(got[0], res + gate * m.a(x))
+
+
+@pytest.mark.gpu
 def test_compiled_single_stream_block_equals_eager_bit_for_bit(pkg, dev):
     """x + gate * linear2(cat((a, gelu(mlp)), -1)) with a and mlp split from linear1's output, the shape of a
     single-stream block: the split halves reach the quantiser as strided views, neither the activated tensor nor the
