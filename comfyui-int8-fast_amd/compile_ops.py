@@ -656,9 +656,7 @@ def backend(inner="inductor"):
     """A torch.compile backend: share_quantisation, fuse_prologues and fuse_epilogues, then `inner` (a registered backend
     name or a callable)."""
     def compile_fn(gm, example_inputs):
-        share_quantisation(gm)
-        fuse_prologues(gm)
-        fuse_epilogues(gm)
+        rewrite(gm)
         fn = inner
         if isinstance(inner, str):
             from torch._dynamo.backends.registry import lookup_backend
@@ -666,6 +664,46 @@ def backend(inner="inductor"):
             fn = lookup_backend(inner)
         return fn(gm, example_inputs)
     return compile_fn
+
+
+LAST_PASS_COUNTS = None   # (layers sharing a quantiser, prologues, epilogues) of the most recent graph the installed pass saw
+
+
+def rewrite(gm: torch.fx.GraphModule):
+    """The three rewrites in the order in which they build on each other -> their counts."""
+    return share_quantisation(gm), fuse_prologues(gm), fuse_epilogues(gm)
+
+
+def install_inductor_pass() -> bool:
+    """Make plain `torch.compile(model)` -- the inductor backend, what ComfyUI's compile nodes call, as the reference's
+    README has its users do (README.md:4,56) -- apply the rewrites without `backend=compile_ops.backend()`: they are
+    registered as inductor's pre-grad custom pass, behind a pass that is already registered there.  Idempotent;
+    returns False where this torch has no such hook."""
+    global _installed
+    try:
+        import torch._inductor.config as inductor_config
+    except ImportError:
+        return False
+    if not hasattr(inductor_config, "pre_grad_custom_pass"):
+        return False
+    if _installed:
+        return True
+    before = inductor_config.pre_grad_custom_pass
+
+    def i8f_pre_grad_pass(graph: torch.fx.Graph):
+        global LAST_PASS_COUNTS
+        if before is not None:
+            before(graph)
+        gm = graph.owning_module
+        if gm is not None and any("i8f" in str(n.target) for n in graph.nodes if n.op == "call_function"):
+            LAST_PASS_COUNTS = rewrite(gm)
+
+    inductor_config.pre_grad_custom_pass = i8f_pre_grad_pass
+    _installed = True
+    return True
+
+
+_installed = False
 
 
 def split_scale(weight_scale):

@@ -11,9 +11,11 @@ when this module is imported, so that the logic underneath (`configure_ops`, `up
 from __future__ import annotations
 
 import logging
+import os
 
 import torch
 
+from . import compile_ops
 from .dynamic_lora import DynamicLoRAHook, append_entry
 from .int8_quant import INT8LoRAPatchAdapter, INT8MergedLoRAPatchAdapter, Int8TensorwiseOps
 
@@ -187,6 +189,10 @@ class UNetLoaderINTW8A8:
         from comfy.sd import load_diffusion_model
 
         ops = configure_ops(model_type, on_the_fly_quantization, enable_quarot)
+        # a model loaded here may be handed to torch.compile later (ComfyUI's compile nodes use the inductor backend):
+        # have inductor apply the graph rewrites to graphs that hold this package's operators
+        if not os.environ.get("I8F_NO_INDUCTOR_PASS"):
+            compile_ops.install_inductor_pass()
         path = folder_paths.get_full_path("diffusion_models", unet_name)
         return (load_diffusion_model(path, model_options={"custom_operations": ops}),)
 

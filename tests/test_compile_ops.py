@@ -828,6 +828,47 @@ def test_compiled_shared_quantiser_with_a_gated_residual_on_one_layer(pkg, dev):
 
 
 @pytest.mark.gpu
+def test_plain_torch_compile_applies_the_rewrites_once_the_pass_is_installed(pkg, dev):
+    """torch.compile(model) with the default backend, after compile_ops.install_inductor_pass(): the adaLN-Zero MLP is
+    rewritten by inductor's pre-grad hook exactly as by compile_ops.backend() -- two prologues, one gated residual --
+    and the result is that of the eager fused calls bit for bit."""
+    import torch._inductor.config as inductor_config
+    g = torch.Generator().manual_seed(22)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = torch.nn.LayerNorm(256, elementwise_affine=False, eps=1e-6)
+            self.up, self.down = lin(512, 256), lin(256, 512)
+
+        def forward(self, x, scale, shift, gate):
+            h = self.up((1 + scale) * self.norm(x) + shift)
+            return x + gate * self.down(F.gelu(h, approximate="tanh"))
+
+    m = Block().to(dev)
+    x = (torch.randn(2, 40, 256, generator=g) * 2).bfloat16().to(dev)
+    sc, sh, gate = ((torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev) for _ in range(3))
+    before = inductor_config.pre_grad_custom_pass
+    try:
+        assert pkg.compile_ops.install_inductor_pass() and pkg.compile_ops.install_inductor_pass()
+        pkg.compile_ops.LAST_PASS_COUNTS = None
+        with torch.no_grad():
+            got = torch.compile(m, fullgraph=True)(x, sc, sh, gate)
+        assert pkg.compile_ops.LAST_PASS_COUNTS == (0, 2, 1)
+        L = pkg._lib
+        h = m.up(x, prologue=L.PRO_NORM_MODULATE, mod_scale=sc, mod_shift=sh, eps=1e-6)
+        assert torch.equal(got, m.down(h, prologue=L.PRO_GELU_TANH, gate=gate, residual=x))
+    finally:
+        inductor_config.pre_grad_custom_pass = before
+        pkg.compile_ops._installed = False
+
+
+@pytest.mark.gpu
 def test_compiled_single_stream_block_equals_eager_bit_for_bit(pkg, dev):
     """x + gate * linear2(cat((a, gelu(mlp)), -1)) with a and mlp split from linear1's output, the shape of a
     single-stream block: the split halves reach the quantiser as strided views, neither the activated tensor nor the

@@ -218,7 +218,10 @@ def fake_comfy(monkeypatch, pkg):
     return types.SimpleNamespace(calls=calls, model=model, files=lora_files)
 
 
-def test_loader_node_passes_the_ops_class(pkg, fake_comfy):
+def test_loader_node_passes_the_ops_class(pkg, fake_comfy, monkeypatch):
+    import torch._inductor.config as inductor_config
+    monkeypatch.setattr(inductor_config, "pre_grad_custom_pass", None)       # (restored when the test ends)
+    monkeypatch.setattr(pkg.compile_ops, "_installed", False)
     node = pkg.NODE_CLASS_MAPPINGS["OTUNetLoaderW8A8"]()
     inputs = node.INPUT_TYPES()["required"]
     assert inputs["unet_name"] == (["unet.safetensors"],) and inputs["model_type"][0][0] == "flux2"
@@ -229,6 +232,13 @@ def test_loader_node_passes_the_ops_class(pkg, fake_comfy):
     assert options == {"custom_operations": pkg.Int8TensorwiseOps}
     assert pkg.Int8TensorwiseOps.excluded_names == ["time_text_embed", "img_in", "norm_out", "proj_out", "txt_in"]
     assert pkg.Int8TensorwiseOps.dynamic_quantize and pkg.Int8TensorwiseOps.enable_quarot
+    # a model from this loader may be compiled later: inductor has been given the graph rewrites as its pre-grad pass
+    assert inductor_config.pre_grad_custom_pass is not None and pkg.compile_ops._installed
+    monkeypatch.setenv("I8F_NO_INDUCTOR_PASS", "1")
+    monkeypatch.setattr(inductor_config, "pre_grad_custom_pass", None)
+    monkeypatch.setattr(pkg.compile_ops, "_installed", False)
+    node.load_unet("unet.safetensors", "default", "qwen", True)
+    assert inductor_config.pre_grad_custom_pass is None
 
 
 def test_lora_node_upgrades_and_registers(pkg, fake_comfy):
