@@ -566,13 +566,41 @@ def _sole_user(node):
     return next(iter(node.users)) if len(node.users) == 1 else None
 
 
+_FRESH_TENSOR_FUNCTIONS = (operator.add, operator.sub, operator.mul, operator.truediv, operator.iadd, operator.isub, operator.imul,
+                           torch.add, torch.sub, torch.mul, torch.cat, torch.nn.functional.linear, torch.nn.functional.layer_norm,
+                           torch.nn.functional.rms_norm, torch.nn.functional.gelu, torch.nn.functional.silu)
+
+
+def _update_in_place_is_private(res, update, order_of) -> bool:
+    """`update` is `res += v` (operator.iadd).  Replacing it by an operator that RETURNS res + v leaves res itself as it
+    was, which nobody can tell if (a) everything else that reads res does so before the update, and (b) res is not a
+    window onto storage that something else reads: it is the result of an operation that makes a new tensor (arithmetic,
+    a layer, one of this package's operators), possibly behind shape-only steps that have no other user.  Graph inputs,
+    parameters, slices and anything unknown fail (b)."""
+    pos = order_of.get(update, 1 << 30)
+    for user in res.users:
+        if user is not update and order_of.get(user, 1 << 30) > pos:
+            return False
+    base = res
+    while (base.op == "call_method" and base.target in _VIEW_METHODS) or _is_call(base, torch.reshape, torch.flatten):
+        src = base.args[0]
+        if not isinstance(src, torch.fx.Node) or len(src.users) != 1:
+            return False
+        base = src
+    if base.op == "call_module":
+        return True
+    return base.op == "call_function" and (base.target in _FRESH_TENSOR_FUNCTIONS or "i8f" in str(base.target))
+
+
 def fuse_epilogues(gm: torch.fx.GraphModule) -> int:
     """Rewrite res + gate * int8_linear(...) -- the gated residual behind the projections of an adaLN-Zero block, gate
     one vector per leading index broadcast over the tokens, res of the result's shape, all of the compute dtype, in any
     operand order, with shape-only steps between the layer and the multiplication -- into the layer's own epilogue
-    (addend=res, gate=gate); also gate * linear(...) and res + linear(...) alone.  Layers that already carry an addend
-    (a dynamic-LoRA side tensor) are left alone.  Returns the number of layers rewritten."""
+    (addend=res, gate=gate); also gate * linear(...) and res + linear(...) alone, and the in-place spelling
+    `res += gate * linear(...)` where nobody can tell the difference (_update_in_place_is_private).  Layers that already
+    carry an addend (a dynamic-LoRA side tensor) are left alone.  Returns the number of layers rewritten."""
     n_fused = 0
+    order_of = {n: i for i, n in enumerate(gm.graph.nodes)}
     lin_targets = (torch.ops.i8f.int8_linear, torch.ops.i8f.int8_linear.default,
                    torch.ops.i8f.int8_linear_prologue, torch.ops.i8f.int8_linear_prologue.default,
                    torch.ops.i8f.linear_w8a8, torch.ops.i8f.linear_w8a8.default)
@@ -616,6 +644,19 @@ def fuse_epilogues(gm: torch.fx.GraphModule) -> int:
                 r_val = _meta_val(r_node)
                 if r_val is not None and tuple(r_val.shape) == tuple(_meta_shape(u)) and r_val.dtype == cur_val.dtype and r_node is not u:
                     res, last = r_node, a
+            elif a is not None and _is_call(a, operator.iadd) and len(a.args) == 2 and a.args[1] is u and isinstance(a.args[0], torch.fx.Node):
+                r_node = a.args[0]                                   # res += gate * y
+                r_val = _meta_val(r_node)
+                if (r_val is not None and tuple(r_val.shape) == tuple(_meta_shape(u)) and r_val.dtype == cur_val.dtype
+                        and _update_in_place_is_private(r_node, a, order_of)):
+                    res, last = r_node, a
+        elif _is_call(u, operator.iadd) and len(u.args) == 2 and u.args[1] is cur and isinstance(u.args[0], torch.fx.Node):
+            r_node = u.args[0]                                       # res += y
+            r_val = _meta_val(r_node)
+            if (r_val is None or cur_val is None or tuple(r_val.shape) != tuple(cur_val.shape) or r_val.dtype != cur_val.dtype
+                    or not _update_in_place_is_private(r_node, u, order_of)):
+                continue
+            res, last = r_node, u
         elif _is_call(u, operator.add, torch.add) and len(u.args) == 2 and not u.kwargs:
             r_node = other(u, cur)
             r_val = _meta_val(r_node)

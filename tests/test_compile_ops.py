@@ -403,6 +403,46 @@ def test_graph_rewrite_gives_layers_that_read_one_tensor_a_single_quantiser(pkg)
     assert not any("rms_norm" in str(n.target) or n.target in (operator.mul, F.silu) for n in gm.graph.nodes if n.op == "call_function")
 
 
+def test_graph_rewrite_takes_the_in_place_residual_update_where_nobody_can_tell(pkg):
+    """`txt += gate * proj(h)`, the in-place spelling of the residual update: folded into the layer's epilogue when txt is
+    an intermediate of the graph that nothing reads afterwards except through the update's result; left to torch (with
+    only the gate folded in) when txt is a graph input, a slice of something else, or read again after the update."""
+    g = torch.Generator().manual_seed(24)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Block(torch.nn.Module):
+        def __init__(self, form):
+            super().__init__()
+            self.proj, self.form = lin(64, 64), form
+
+        def forward(self, x, h, gate):
+            if self.form == "input":
+                txt = x
+            elif self.form == "slice":
+                txt = torch.cat((x, x), 1)[:, :24]
+            else:
+                txt = x + 1.0
+            before = txt.sum() if self.form == "read_before" else None
+            keep = txt                                   # the same tensor: sees the update in eager mode
+            txt += gate * self.proj(h)
+            out = txt * 2.0
+            if self.form == "read_after":
+                return out, keep.mean()
+            return (out, before) if before is not None else out
+
+    x, h, gate = torch.randn(2, 24, 64).bfloat16(), torch.randn(2, 24, 64).bfloat16(), torch.randn(2, 1, 64).bfloat16()
+    for form, with_residual in (("fresh", True), ("read_before", True), ("input", False), ("slice", False), ("read_after", False)):
+        gm = torch._dynamo.export(Block(form))(x, h, gate).graph_module
+        assert pkg.compile_ops.fuse_epilogues(gm) == 1
+        node = [n for n in gm.graph.nodes if n.op == "call_function" and "int8_linear" in str(n.target)][0]
+        assert node.kwargs.get("gate") is not None and (node.kwargs.get("addend") is not None) == with_residual, form
+        assert any(n.target is operator.iadd for n in gm.graph.nodes if n.op == "call_function") == (not with_residual), form
+
+
 def test_graph_rewrites_keep_away_from_in_place_writes(pkg):
     """A tensor overwritten in place between the point where the model reads it and the layer that would read it inside
     a fused operator: the rewrites leave that stretch of the graph alone (the fused read would see the new value)."""
@@ -866,6 +906,49 @@ def test_plain_torch_compile_applies_the_rewrites_once_the_pass_is_installed(pkg
     finally:
         inductor_config.pre_grad_custom_pass = before
         pkg.compile_ops._installed = False
+
+
+@pytest.mark.gpu
+def test_compiled_in_place_residual_update_equals_eager(pkg, dev):
+    """The residual updates of a double-stream block as the model code spells them, `img = img + g * proj(a)` and
+    `txt += g * proj(a)`: both end up in their layer's epilogue under the rewriting backend, and the results are those
+    of eager mode bit for bit (torch's two rounded operations either way)."""
+    g = torch.Generator().manual_seed(25)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+
+    class Pair(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.img_proj, self.txt_proj, self.embed = lin(256, 256), lin(256, 256), lin(256, 128)
+
+        def forward(self, img, txt_tokens, a_img, a_txt, g_img, g_txt):
+            txt = self.embed(txt_tokens)
+            img = img + g_img * self.img_proj(a_img)
+            txt += g_txt * self.txt_proj(a_txt)
+            return img, txt
+
+    m = Pair().to(dev)
+    img, a_img = (torch.randn(2, 64, 256, generator=g).bfloat16().to(dev) for _ in range(2))
+    tok, a_txt = torch.randn(2, 24, 128, generator=g).bfloat16().to(dev), torch.randn(2, 24, 256, generator=g).bfloat16().to(dev)
+    g_img, g_txt = ((torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev) for _ in range(2))
+    seen = []
+
+    def counting(gm, inputs):
+        calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum(n.kwargs.get("gate") is not None and n.kwargs.get("addend") is not None for n in calls),
+                     sum(n.target in (operator.mul, operator.add, operator.iadd) for n in calls)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    with torch.no_grad():
+        got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(img, tok, a_img, a_txt, g_img, g_txt)
+        assert seen == [(2, 0)]
+        want = m(img, tok, a_img, a_txt, g_img, g_txt)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
 
 
 @pytest.mark.gpu
