@@ -342,7 +342,7 @@ def extras(L, dev, quick=False):
 
     # the whole adaLN producer of a DiT block, LayerNorm without affine and the modulation, inside the quantiser
     def norm_fused(i):
-        rc = lib.i8f_quant_rowwise_norm_modulate(ptr(xs[i]), L.BF16, M, K, K, 1e-6, ptr(sc), ptr(sh), M, 0, ptr(qs[i]), ptr(ss[i]), stream)
+        rc = lib.i8f_quant_rowwise_norm_modulate(ptr(xs[i]), L.BF16, M, K, K, 1e-6, ptr(sc), ptr(sh), M, 0, 0, ptr(qs[i]), ptr(ss[i]), stream)
         assert rc == 0, rc
 
     def norm_unfused(i):
@@ -380,7 +380,7 @@ def extras(L, dev, quick=False):
     nw, zsc = (torch.randn(Kz, device=dev) * 0.2 + 1).bfloat16(), (torch.randn(1, Kz, device=dev) * 0.3).bfloat16()
 
     def rms_fused(i):
-        rc = lib.i8f_quant_rowwise_rms_norm(ptr(zs[i]), L.BF16, M, Kz, Kz, 1e-5, ptr(nw), ptr(zsc), None, M, 0, ptr(zq[i]), ptr(ss[i]), stream)
+        rc = lib.i8f_quant_rowwise_rms_norm(ptr(zs[i]), L.BF16, M, Kz, Kz, 1e-5, ptr(nw), ptr(zsc), None, M, 0, 0, ptr(zq[i]), ptr(ss[i]), stream)
         assert rc == 0, rc
 
     def rms_unfused(i):

@@ -19,6 +19,7 @@ BF16, F16, F32 = 0, 1, 2
 SCALE_TENSOR, SCALE_ROW = 0, 1
 EPI_TORCH, EPI_FUSED = 0, 1
 PRO_NONE, PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE, PRO_CONCAT_GELU, PRO_GELU_ERF, PRO_RMS_NORM = 0, 1, 2, 3, 4, 5, 6, 7
+PRO_MODULATE_FUSED = 8   # the modulation as torch.addcmul(shift, x, 1 + scale): product and sum rounded once
 
 _DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
 
@@ -55,8 +56,8 @@ def lib() -> ctypes.CDLL:
     L.i8f_rotate128.argtypes = [vp, i32, i64, i64, i64, vp, vp]
     L.i8f_quant_rowwise_grouped.argtypes = [vp, i32, i32, i64, i32, vp]
     L.i8f_quant_rowwise_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, i32, vp, vp, vp]
-    L.i8f_quant_rowwise_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, i32, vp, vp, vp]
-    L.i8f_quant_rowwise_rms_norm.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, vp, i64, i32, vp, vp, vp]
+    L.i8f_quant_rowwise_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, i32, i32, vp, vp, vp]
+    L.i8f_quant_rowwise_rms_norm.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, vp, i64, i32, i32, vp, vp, vp]
     L.i8f_quant_rowwise_concat_gelu.argtypes = [vp, i32, i64, i64, i64, vp, i64, i64, i32, vp, vp, vp]
     L.i8f_quant_tensorwise_workspace_bytes.argtypes = [i64]
     L.i8f_quant_tensorwise_workspace_bytes.restype = i64
@@ -221,7 +222,8 @@ def norm_modulate_fusable(x: torch.Tensor) -> bool:
             and x.stride(1) == 1 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0)
 
 
-def quant_rowwise_rms_norm(x: torch.Tensor, eps: float = 1e-6, weight=None, mod_scale=None, mod_shift=None, rotate: bool = False):
+def quant_rowwise_rms_norm(x: torch.Tensor, eps: float = 1e-6, weight=None, mod_scale=None, mod_shift=None, rotate: bool = False,
+                           fused_add: bool = False):
     """quant_rowwise of rms_norm(x, weight, eps) [* (1 + mod_scale)] [+ mod_shift] with no intermediate tensor in memory:
     the producer of the projections of blocks that normalise with an RMSNorm.  x [M,K] as norm_modulate_fusable
     describes; weight [K]; mod_scale / mod_shift [V,K] (or [K]), M // V consecutive rows to a vector; each optional."""
@@ -253,13 +255,13 @@ def quant_rowwise_rms_norm(x: torch.Tensor, eps: float = 1e-6, weight=None, mod_
     with _on(x.device):
         _check(lib().i8f_quant_rowwise_rms_norm(_ptr(x), dtype_code(x.dtype), M, K, x.stride(0) if M > 1 else K, float(eps),
                                                 _ptr(weight) if weight is not None else None, *(None if v is None else _ptr(v) for v in vecs),
-                                                rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s), _stream(x)),
+                                                rows_per_vec, int(bool(fused_add)), 128 if rotate else 0, _ptr(q), _ptr(s), _stream(x)),
                "i8f_quant_rowwise_rms_norm")
     return q, s
 
 
 def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NONE, mod_scale=None, mod_shift=None, eps: float = 1e-6,
-                  norm_weight=None):
+                  norm_weight=None, fused_add: bool = False):
     """x [M,K] (bf16/fp16/fp32, cuda) -> (int8 [M,K], float32 [M,1]); rotate=True applies the 128-block Hadamard first.
     prologue applies an elementwise operation while the rows are read: PRO_GELU_TANH, or PRO_MODULATE with
     mod_scale / mod_shift of x's dtype, [V,K] (or [K]): (1 + mod_scale) * x + mod_shift, M // V consecutive rows
@@ -268,10 +270,11 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
     parameters (see norm_modulate_fusable for the rows it takes), or PRO_CONCAT_GELU with a second tensor [M,Kb] as
     mod_scale: cat((x, gelu(mod_scale)), -1) (see quant_rowwise_concat_gelu), or PRO_GELU_ERF, GELU in its exact form, or
     PRO_RMS_NORM: rms_norm(x, norm_weight, eps), then the modulation's operations where mod_scale / mod_shift are given
-    (see quant_rowwise_rms_norm)."""
+    (see quant_rowwise_rms_norm).  fused_add (or PRO_MODULATE_FUSED): the modulation as torch.addcmul(mod_shift, x, 1 + mod_scale)
+    computes it, product and sum rounded once (16-bit tensors), in the three kinds that modulate."""
     _dev(x, "x")
     if prologue == PRO_RMS_NORM:
-        return quant_rowwise_rms_norm(x, eps, norm_weight, mod_scale, mod_shift, rotate=rotate)
+        return quant_rowwise_rms_norm(x, eps, norm_weight, mod_scale, mod_shift, rotate=rotate, fused_add=fused_add)
     if prologue == PRO_CONCAT_GELU:   # x followed by gelu(mod_scale) along the row
         return quant_rowwise_concat_gelu(x, mod_scale, rotate=rotate)
     x = _rows(x, "x")
@@ -282,7 +285,11 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
     s = torch.empty((M, 1), dtype=torch.float32, device=x.device)
     ldx = x.stride(0) if M > 1 else K
     rows_per_vec = 1
-    if prologue in (PRO_MODULATE, PRO_SILU_GATE, PRO_NORM_MODULATE):
+    if prologue == PRO_MODULATE and fused_add:
+        prologue = PRO_MODULATE_FUSED
+    if prologue == PRO_MODULATE_FUSED and x.dtype == torch.float32:
+        raise ValueError("the fused form of the modulation exists for 16-bit tensors")
+    if prologue in (PRO_MODULATE, PRO_MODULATE_FUSED, PRO_SILU_GATE, PRO_NORM_MODULATE):
         if prologue == PRO_NORM_MODULATE and not norm_modulate_fusable(x):
             raise ValueError("PRO_NORM_MODULATE takes contiguous 16-bit rows of at most 16384 elements in multiples of 16 "
                              "(see norm_modulate_fusable); normalise with torch and use PRO_MODULATE")
@@ -309,8 +316,8 @@ def quant_rowwise(x: torch.Tensor, rotate: bool = False, prologue: int = PRO_NON
                                            _stream(x)), "i8f_quant_rowwise")
         elif prologue == PRO_NORM_MODULATE:
             _check(lib().i8f_quant_rowwise_norm_modulate(_ptr(x), dtype_code(x.dtype), M, K, ldx, float(eps), _ptr(mod_scale),
-                                                         _ptr(mod_shift), rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s),
-                                                         _stream(x)), "i8f_quant_rowwise_norm_modulate")
+                                                         _ptr(mod_shift), rows_per_vec, int(bool(fused_add)), 128 if rotate else 0, _ptr(q),
+                                                         _ptr(s), _stream(x)), "i8f_quant_rowwise_norm_modulate")
         else:
             _check(lib().i8f_quant_rowwise_prologue(_ptr(x), dtype_code(x.dtype), M, K, ldx, prologue, _ptr(mod_scale),
                                                     _ptr(mod_shift), rows_per_vec, 128 if rotate else 0, _ptr(q), _ptr(s),

@@ -57,16 +57,16 @@ def _(x, rotate):
 
 @torch.library.custom_op(f"{NAMESPACE}::quantize_rowwise_prologue", mutates_args=())
 def quantize_rowwise_prologue(x: Tensor, rotate: bool, prologue: int, mod_scale: Optional[Tensor], mod_shift: Optional[Tensor],
-                              eps: float = 1e-6, norm_weight: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+                              eps: float = 1e-6, norm_weight: Optional[Tensor] = None, fused_add: bool = False) -> Tuple[Tensor, Tensor]:
     """quantize_rowwise on prologue(x) (the kinds of int8_linear_prologue), x with any leading dimensions:
     -> int8 [rows, K'] and float32 [rows, 1], K' the width behind the prologue.  What the layers that read one
     activation tensor share when the graph rewrite gives them a single quantiser."""
     return _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
-                              mod_shift=mod_shift, eps=eps, norm_weight=norm_weight)
+                              mod_shift=mod_shift, eps=eps, norm_weight=norm_weight, fused_add=fused_add)
 
 
 @quantize_rowwise_prologue.register_fake
-def _(x, rotate, prologue, mod_scale, mod_shift, eps=1e-6, norm_weight=None):
+def _(x, rotate, prologue, mod_scale, mod_shift, eps=1e-6, norm_weight=None, fused_add=False):
     rows = x.numel() // max(1, x.shape[-1])
     width = x.shape[-1] + (mod_scale.shape[-1] if prologue == _lib.PRO_CONCAT_GELU else 0)
     return (x.new_empty((rows, width), dtype=torch.int8), x.new_empty((rows, 1), dtype=torch.float32))
@@ -154,21 +154,22 @@ def int8_linear_prologue(x: Tensor, prologue: int, mod_scale: Optional[Tensor], 
                          weight: Tensor, weight_scale: Optional[Tensor], weight_scale_value: float,
                          bias: Optional[Tensor], compute_dtype: torch.dtype, rotate: bool, order: int, eps: float = 1e-6,
                          addend: Optional[Tensor] = None, gate: Optional[Tensor] = None,
-                         norm_weight: Optional[Tensor] = None) -> Tensor:
+                         norm_weight: Optional[Tensor] = None, fused_add: bool = False) -> Tensor:
     """int8_linear on prologue(x): GELU (tanh or exact form), (1 + mod_scale) * x + mod_shift with one pair of vectors per
     group of consecutive rows (PRO_NORM_MODULATE: of layer_norm(x, eps) without affine parameters; PRO_RMS_NORM: of
-    rms_norm(x, norm_weight, eps), scale and shift each optional), silu(x) * mod_scale with a gate operand of x's shape,
+    rms_norm(x, norm_weight, eps), scale and shift each optional; fused_add: product and sum rounded once, as
+    torch.addcmul(mod_shift, x, 1 + mod_scale)), silu(x) * mod_scale with a gate operand of x's shape,
     or cat((x, gelu(mod_scale)), -1); the transformed activations exist only inside the quantiser."""
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rotate, prologue=prologue, mod_scale=mod_scale,
-                              mod_shift=mod_shift, eps=eps, norm_weight=norm_weight)
+                              mod_shift=mod_shift, eps=eps, norm_weight=norm_weight, fused_add=fused_add)
     y = _lib.linear_w8a8(q, s, weight, _scale_arg(weight_scale, weight_scale_value), bias, compute_dtype, order, addend=addend, gate=gate)
     return y.reshape(*lead, weight.shape[0])
 
 
 @int8_linear_prologue.register_fake
 def _(x, prologue, mod_scale, mod_shift, weight, weight_scale, weight_scale_value, bias, compute_dtype, rotate, order, eps=1e-6,
-      addend=None, gate=None, norm_weight=None):
+      addend=None, gate=None, norm_weight=None, fused_add=False):
     width = weight.shape[0]
     return x.new_empty((*x.shape[:-1], width), dtype=compute_dtype)
 
@@ -321,6 +322,25 @@ def _match_rms_norm(node):
     return (h, w, float(eps)) if isinstance(eps, (int, float)) else None
 
 
+def _match_modulate_addcmul(node):
+    """torch.addcmul(shift, x, 1 + scale) (the two factors in either order, value 1) on 16-bit tensors -> (x, scale, shift)."""
+    if not (_is_call(node, torch.addcmul) and len(node.users) == 1):
+        return None
+    a = dict(zip(("input", "tensor1", "tensor2"), node.args))
+    a.update(node.kwargs)
+    if a.get("value", 1) != 1 or a.get("out") is not None:
+        return None
+    shift, f1, f2 = a.get("input"), a.get("tensor1"), a.get("tensor2")
+    for gain, x in ((f1, f2), (f2, f1)):
+        if isinstance(gain, torch.fx.Node) and _is_call(gain, operator.add, torch.add) and len(gain.users) == 1 and len(gain.args) == 2:
+            for one, scale in (gain.args, gain.args[::-1]):
+                if isinstance(one, (int, float)) and one == 1 and all(isinstance(n, torch.fx.Node) for n in (scale, x, shift)):
+                    v = _meta_val(x)
+                    if v is not None and v.dtype in (torch.bfloat16, torch.float16):
+                        return x, scale, shift
+    return None
+
+
 def _match_plain_layer_norm(node):
     """layer_norm(h, (K,), eps=...) over the last dimension without weight and bias, used nowhere else, on 16-bit rows
     of a width the normalising quantiser takes -> (h, eps)."""
@@ -391,39 +411,41 @@ def _in_place_write_between(first, last) -> bool:
 
 
 def _match_producer(src, rotate):
-    """The producer of a layer's activations as a prologue kind -> (h, kind, mod_scale, mod_shift, eps, norm_weight)
-    nodes / values, or None.  Every node matched is used nowhere else."""
+    """The producer of a layer's activations as a prologue kind -> (h, kind, mod_scale, mod_shift, eps, norm_weight,
+    fused_add) nodes / values, or None.  Every node matched is used nowhere else."""
     h = _match_gelu(src)
     if h is not None:
-        return h, _lib.PRO_GELU_TANH, None, None, 1e-6, None
+        return h, _lib.PRO_GELU_TANH, None, None, 1e-6, None, False
     h = _match_gelu_erf(src)
     if h is not None:
-        return h, _lib.PRO_GELU_ERF, None, None, 1e-6, None
+        return h, _lib.PRO_GELU_ERF, None, None, 1e-6, None, False
     r = _match_rms_norm(src)
     if r is not None:                                               # the norm alone
-        return r[0], _lib.PRO_RMS_NORM, None, None, r[2], r[1]
+        return r[0], _lib.PRO_RMS_NORM, None, None, r[2], r[1], False
     so = _match_scale_only(src)
     if so is not None:                                              # modulate(norm(x), scale) = norm(x) * (1 + scale)
         r = _match_rms_norm(so[0])
         if r is not None and _vectors_broadcast_over_tokens(r[0], so[1], so[1]):
-            return r[0], _lib.PRO_RMS_NORM, so[1], None, r[2], r[1]
-    m = _match_modulate(src)
+            return r[0], _lib.PRO_RMS_NORM, so[1], None, r[2], r[1], False
+    m, fused = _match_modulate(src), False
+    if m is None:
+        m, fused = _match_modulate_addcmul(src), True               # the one-kernel spelling: product and sum rounded once
     if m is not None:
         if not _vectors_broadcast_over_tokens(*m):
             return None
         ln = _match_plain_layer_norm(m[0])   # the modulated tensor is a LayerNorm without affine: that goes in too
         if ln is not None:
-            return ln[0], _lib.PRO_NORM_MODULATE, m[1], m[2], ln[1], None
+            return ln[0], _lib.PRO_NORM_MODULATE, m[1], m[2], ln[1], None, fused
         rn = _match_rms_norm(m[0])           # or an RMSNorm
         if rn is not None and _vectors_broadcast_over_tokens(rn[0], m[1], m[2]):
-            return rn[0], _lib.PRO_RMS_NORM, m[1], m[2], rn[2], rn[1]
-        return m[0], _lib.PRO_MODULATE, m[1], m[2], 1e-6, None
+            return rn[0], _lib.PRO_RMS_NORM, m[1], m[2], rn[2], rn[1], fused
+        return m[0], _lib.PRO_MODULATE, m[1], m[2], 1e-6, None, fused
     g = _match_silu_gate(src)
     if g is not None:
-        return g[0], _lib.PRO_SILU_GATE, g[1], None, 1e-6, None
+        return g[0], _lib.PRO_SILU_GATE, g[1], None, 1e-6, None, False
     c = _match_concat_gelu(src)
     if c is not None and not (rotate and (_meta_shape(c[0])[-1] % 128 or _meta_shape(c[1])[-1] % 128)):
-        return c[0], _lib.PRO_CONCAT_GELU, c[1], None, 1e-6, None
+        return c[0], _lib.PRO_CONCAT_GELU, c[1], None, 1e-6, None, False
     return None
 
 
@@ -457,7 +479,7 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         found = _match_producer(src, rotate)
         if found is None:
             continue
-        h, kind, mod_scale, mod_shift, eps, norm_w = found
+        h, kind, mod_scale, mod_shift, eps, norm_w, fused_add = found
         earliest = min((n for n in (h, mod_scale, mod_shift, norm_w) if isinstance(n, torch.fx.Node)), key=lambda n: order_of.get(n, 1 << 30))   # (nodes this pass created sit where a later node was)
         if _in_place_write_between(earliest, node):
             continue
@@ -478,7 +500,7 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         if not is_lin:   # the shared quantiser: its outputs are 2-D whatever h's leading dimensions are
             with gm.graph.inserting_before(node):
                 fused = gm.graph.call_function(torch.ops.i8f.quantize_rowwise_prologue,
-                                               (h, rotate, kind, mod_scale, mod_shift, eps, norm_w))
+                                               (h, rotate, kind, mod_scale, mod_shift, eps, norm_w, fused_add))
             node.replace_all_uses_with(fused)
             gm.graph.erase_node(node)
             n_fused += 1
@@ -486,7 +508,7 @@ def fuse_prologues(gm: torch.fx.GraphModule) -> int:
         with gm.graph.inserting_before(node):
             fused = gm.graph.call_function(torch.ops.i8f.int8_linear_prologue,
                                            (h, kind, mod_scale, mod_shift, weight, ws_t, ws_v, bias, cdt, rotate, order, eps),
-                                           {} if norm_w is None else {"norm_weight": norm_w})
+                                           {k: v for k, v in (("norm_weight", norm_w), ("fused_add", fused_add)) if v})
             n_out, old = _out_features(weight), _meta_val(node)
             if old is not None:   # shapes for the passes that follow (the epilogue rewrite reads them)
                 _record(fused, (*h_shape[:-1], n_out), old.dtype)

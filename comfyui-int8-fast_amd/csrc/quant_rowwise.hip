@@ -59,6 +59,7 @@ struct Prologue {
     int64_t ldb_bytes;
     int runs_a;
     const void *w;           // RMS_NORM: the norm's weight vector [K] (or nullptr)
+    int fused_add;           // the modulation's product and sum with ONE rounding, round((1 + s) * x + t): torch.addcmul
 };
 
 // the sum over the wave in a fixed order (the same in every lane)
@@ -97,13 +98,16 @@ __device__ __forceinline__ float gelu_erf_f32(float x) {
     return x * (x >= 0.0f ? 1.0f - h : h);
 }
 
+// (fused: torch.addcmul(t, x, 1 + s) -- the gain still a rounded tensor of its own, its product with x, exact in binary32
+// for 16-bit operands, added to t and rounded once)
 template <int DT, int PRO>
-__device__ __forceinline__ float apply_prologue(float x, float s, float t) {
+__device__ __forceinline__ float apply_prologue(float x, float s, float t, bool fused = false) {
     if constexpr (PRO == I8F_PRO_SILU_GATE) {
         return round_to_dtype<DT>(round_to_dtype<DT>(silu_f32(x)) * s);
     } else if constexpr (PRO == I8F_PRO_MODULATE || PRO == I8F_PRO_NORM_MODULATE) {
         const float a = round_to_dtype<DT>(1.0f + s);
-        const float b = round_to_dtype<DT>(a * x);
+        const float p = a * x;
+        const float b = fused ? p : round_to_dtype<DT>(p);
         return round_to_dtype<DT>(b + t);
     } else if constexpr (PRO == I8F_PRO_GELU_TANH) {
         return round_to_dtype<DT>(gelu_tanh_f32(x));
@@ -578,7 +582,10 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
                 if (pro.s) {
                     expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), wv);
 #pragma unroll
-                    for (int j = 0; j < 16; ++j) v[r][j] = round_to_dtype<DT>(round_to_dtype<DT>(1.0f + wv[j]) * v[r][j]);
+                    for (int j = 0; j < 16; ++j) {
+                        const float pr = round_to_dtype<DT>(1.0f + wv[j]) * v[r][j];
+                        v[r][j] = (pro.fused_add && pro.t) ? pr : round_to_dtype<DT>(pr);   // (fused: rounded with the sum below)
+                    }
                 }
                 if (pro.t) {
                     expand16<DT>(*(const uint4 *)((const char *)pro.t + off), *(const uint4 *)((const char *)pro.t + off + 16), wv);
@@ -602,7 +609,7 @@ __device__ __forceinline__ void quant16_body(const char *__restrict__ x, int64_t
                 expand16<DT>(*(const uint4 *)((const char *)pro.s + off), *(const uint4 *)((const char *)pro.s + off + 16), sv);
                 expand16<DT>(*(const uint4 *)((const char *)pro.t + off), *(const uint4 *)((const char *)pro.t + off + 16), tv);
 #pragma unroll
-                for (int j = 0; j < 16; ++j) v[r][j] = FULL || R < nruns ? apply_prologue<DT, PRO>(v[r][j], sv[j], tv[j]) : 0.0f;
+                for (int j = 0; j < 16; ++j) v[r][j] = FULL || R < nruns ? apply_prologue<DT, PRO>(v[r][j], sv[j], tv[j], pro.fused_add != 0) : 0.0f;
             } else if constexpr (PRO == I8F_PRO_SILU_GATE) {
                 const int R = r * TPR + p;
                 const int64_t off = (vrow * K + (seg_run + (FULL || R < nruns ? R : 0)) * 16) * 2;
@@ -795,7 +802,7 @@ __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__r
     auto element = [&](int64_t k) {
         const float xv = load_as_f32<DT>(x, base + k);
         if constexpr (PRO == I8F_PRO_SILU_GATE) return apply_prologue<DT, PRO>(xv, load_as_f32<DT>(pro.s, vbase + k), 0.0f);
-        else if constexpr (PRO == I8F_PRO_MODULATE) return apply_prologue<DT, PRO>(xv, load_as_f32<DT>(pro.s, vbase + k), load_as_f32<DT>(pro.t, vbase + k));
+        else if constexpr (PRO == I8F_PRO_MODULATE) return apply_prologue<DT, PRO>(xv, load_as_f32<DT>(pro.s, vbase + k), load_as_f32<DT>(pro.t, vbase + k), pro.fused_add != 0);
         else return apply_prologue<DT, PRO>(xv, 0.0f, 0.0f);
     };
 
@@ -1064,8 +1071,11 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
                                           int rotate_block, int8_t *q, float *scale, void *stream) {
     using namespace i8f;
     if (prologue == I8F_PRO_NONE) return i8f_quant_rowwise(x, x_dtype, M, K, ldx, rotate_block, q, scale, stream);
+    const bool fused_add = prologue == I8F_PRO_MODULATE_FUSED;   // the modulation with torch.addcmul's single rounding
+    if (fused_add) prologue = I8F_PRO_MODULATE;
     if (prologue != I8F_PRO_MODULATE && prologue != I8F_PRO_GELU_TANH && prologue != I8F_PRO_SILU_GATE && prologue != I8F_PRO_GELU_ERF)
         return I8F_ERR_INVALID;
+    if (fused_add && x_dtype == I8F_F32) return I8F_ERR_UNSUPPORTED;   // (a binary32 product is not exact: torch's result depends on contraction)
     if (M < 0 || K < 0 || !valid_dtype(x_dtype)) return I8F_ERR_INVALID;
     if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
     if (rotate_block && K % rotate_block) return I8F_ERR_INVALID;
@@ -1078,6 +1088,7 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
     if (int rc = check_device()) return rc;
     if (rows_per_vec > 0x7fffffff) rows_per_vec = 0x7fffffff;  // M itself is below 2^31
     Prologue pro{prologue, mod_scale, mod_shift, rows_per_vec > 0 ? rows_per_vec : 1, 0.0f};
+    pro.fused_add = fused_add ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     const bool rot = rotate_block != 0;
     switch (x_dtype) {
@@ -1088,8 +1099,8 @@ extern "C" int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M,
 }
 
 extern "C" int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, float eps,
-                                               const void *mod_scale, const void *mod_shift, int64_t rows_per_vec, int rotate_block,
-                                               int8_t *q, float *scale, void *stream) {
+                                               const void *mod_scale, const void *mod_shift, int64_t rows_per_vec, int modulate_fused,
+                                               int rotate_block, int8_t *q, float *scale, void *stream) {
     using namespace i8f;
     if (M < 0 || K < 0 || !valid_dtype(x_dtype) || !(eps >= 0.0f)) return I8F_ERR_INVALID;
     if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
@@ -1100,6 +1111,7 @@ extern "C" int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64
     if (int rc = check_device()) return rc;
     if (rows_per_vec > 0x7fffffff) rows_per_vec = 0x7fffffff;
     Prologue pro{I8F_PRO_NORM_MODULATE, mod_scale, mod_shift, rows_per_vec, eps};
+    pro.fused_add = modulate_fused ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     const bool rot = rotate_block != 0;
     switch (x_dtype) {
@@ -1110,8 +1122,8 @@ extern "C" int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64
 }
 
 extern "C" int i8f_quant_rowwise_rms_norm(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, float eps, const void *weight,
-                                          const void *mod_scale, const void *mod_shift, int64_t rows_per_vec, int rotate_block,
-                                          int8_t *q, float *scale, void *stream) {
+                                          const void *mod_scale, const void *mod_shift, int64_t rows_per_vec, int modulate_fused,
+                                          int rotate_block, int8_t *q, float *scale, void *stream) {
     using namespace i8f;
     if (M < 0 || K < 0 || !valid_dtype(x_dtype) || !(eps >= 0.0f)) return I8F_ERR_INVALID;
     if (rotate_block != 0 && rotate_block != 128) return I8F_ERR_UNSUPPORTED;
@@ -1122,7 +1134,7 @@ extern "C" int i8f_quant_rowwise_rms_norm(const void *x, int x_dtype, int64_t M,
     if (M > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
     if (int rc = check_device()) return rc;
     if (rows_per_vec > 0x7fffffff || rows_per_vec <= 0) rows_per_vec = 0x7fffffff;
-    Prologue pro{I8F_PRO_RMS_NORM, mod_scale, mod_shift, rows_per_vec, eps, nullptr, 0, 0, weight};
+    Prologue pro{I8F_PRO_RMS_NORM, mod_scale, mod_shift, rows_per_vec, eps, nullptr, 0, 0, weight, modulate_fused ? 1 : 0};
     hipStream_t st = (hipStream_t)stream;
     const bool rot = rotate_block != 0;
     switch (x_dtype) {

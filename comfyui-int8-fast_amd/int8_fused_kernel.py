@@ -34,8 +34,10 @@ def hip_quantize_rowwise(x: torch.Tensor, rotate: bool = False):
 def _linear(x, weight, weight_scale, bias, compute_dtype, rotate, order, addend=None, prologue=None, side=None, gate=None):
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
-    kind, mod_scale, mod_shift, eps, norm_weight = (tuple(prologue) + (1e-6, None)[len(prologue) - 3:])[:5] if prologue else (_lib.PRO_NONE, None, None, 1e-6, None)
-    q, s = _lib.quant_rowwise(x2, rotate=rotate, prologue=kind, mod_scale=mod_scale, mod_shift=mod_shift, eps=eps, norm_weight=norm_weight)
+    kind, mod_scale, mod_shift, eps, norm_weight, fused_add = \
+        (tuple(prologue) + (1e-6, None, False)[len(prologue) - 3:])[:6] if prologue else (_lib.PRO_NONE, None, None, 1e-6, None, False)
+    q, s = _lib.quant_rowwise(x2, rotate=rotate, prologue=kind, mod_scale=mod_scale, mod_shift=mod_shift, eps=eps, norm_weight=norm_weight,
+                              fused_add=fused_add)
     order = DEFAULT_EPILOGUE if order is None else order
     if side is not None:   # (side_t [M,r], side_b [N,r], alpha or None): the low-rank branch formed inside the epilogue
         if gate is not None or addend is not None:
@@ -50,7 +52,7 @@ def hip_int8_linear(x, weight, weight_scale, bias=None, compute_dtype=torch.floa
                     addend=None, prologue=None, side=None, gate=None):
     """W8A8 linear with ONE weight scale (Python float or 1-element tensor).  `addend`, a tensor of the
     output's shape and dtype, is added to the result inside the epilogue (and the sum rounded again).
-    `prologue` = (kind, mod_scale, mod_shift[, eps[, norm_weight]]) applies _lib.PRO_GELU_TANH, _lib.PRO_GELU_ERF, _lib.PRO_MODULATE,
+    `prologue` = (kind, mod_scale, mod_shift[, eps[, norm_weight[, fused_add]]]) applies _lib.PRO_GELU_TANH, _lib.PRO_GELU_ERF, _lib.PRO_MODULATE,
     _lib.PRO_SILU_GATE, _lib.PRO_NORM_MODULATE, _lib.PRO_RMS_NORM or _lib.PRO_CONCAT_GELU to x inside the quantiser.  `side` = (side_t [M,r], side_b [N,r], alpha or None) adds the low-rank product side_t @ side_b.T,
     formed inside the epilogue (see _lib.linear_w8a8_lora), instead of a ready-made addend.  `gate` ([.., 1, N] or [N],
     one vector per group of consecutive rows) multiplies the rounded result before the addend is added:

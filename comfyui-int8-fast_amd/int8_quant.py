@@ -141,7 +141,8 @@ def forward_pair(layers, xs, gates=None, residuals=None):
                                                   xs[0].dtype, rotate=rot, gates=gates, residuals=residuals)
 
 
-def forward_fanout(layers, x, prologue: int = _lib.PRO_NONE, mod_scale=None, mod_shift=None, eps: float = 1e-6, norm_weight=None):
+def forward_fanout(layers, x, prologue: int = _lib.PRO_NONE, mod_scale=None, mod_shift=None, eps: float = 1e-6, norm_weight=None,
+                   fused_add: bool = False):
     """[layer(x) for layer in layers] for quantised layers that read the same activations (separate q, k and v projections,
     the two up-projections of a SwiGLU feed-forward): x is quantised ONCE -- with `prologue` and its operands applied
     inside that quantiser, as forward(x, prologue=...) does for one layer -- and every layer runs its GEMM on the shared
@@ -149,6 +150,8 @@ def forward_fanout(layers, x, prologue: int = _lib.PRO_NONE, mod_scale=None, mod
     of its input, results are bit-identical to the layers' own forward calls, which is also the fall-back where a layer
     is not on the W8A8 path (16 rows or fewer, dynamic LoRA, managed casting, different rotation flags, tracing)."""
     layers = list(layers)
+    if prologue == _lib.PRO_MODULATE_FUSED:
+        prologue, fused_add = _lib.PRO_MODULATE, True
     rot = bool(getattr(layers[0], "_use_quarot", False)) if layers else False
     ok = len(layers) >= 2 and not torch.compiler.is_compiling() and x.is_cuda and x.dim() >= 2 \
         and x.numel() // max(1, x.shape[-1]) > SMALL_BATCH_ROWS and x.dtype in (torch.float16, torch.bfloat16)
@@ -178,10 +181,11 @@ def forward_fanout(layers, x, prologue: int = _lib.PRO_NONE, mod_scale=None, mod
     width = x.shape[-1] + (mod_scale.shape[-1] if ok and prologue == _lib.PRO_CONCAT_GELU else 0)
     ok = ok and all(lin.weight.shape[1] == width for lin in layers)
     if not ok:
-        return [lin(x, prologue=prologue, mod_scale=mod_scale, mod_shift=mod_shift, eps=eps, norm_weight=norm_weight) for lin in layers]
+        return [lin(x, prologue=prologue, mod_scale=mod_scale, mod_shift=mod_shift, eps=eps, norm_weight=norm_weight, fused_add=fused_add)
+                for lin in layers]
     lead = x.shape[:-1]
     q, s = _lib.quant_rowwise(x.reshape(-1, x.shape[-1]), rotate=rot, prologue=prologue, mod_scale=mod_scale, mod_shift=mod_shift,
-                              eps=eps, norm_weight=norm_weight)
+                              eps=eps, norm_weight=norm_weight, fused_add=fused_add)
     outs = []
     for lin in layers:
         ws = lin._get_weight_scale()
@@ -507,7 +511,7 @@ class Int8TensorwiseOps(manual_cast):
         # -- forward ------------------------------------------------------------------------
         def forward(self, x: Tensor, prologue: int = _lib.PRO_NONE, mod_scale: Tensor | None = None,
                     mod_shift: Tensor | None = None, eps: float = 1e-6, gate: Tensor | None = None,
-                    residual: Tensor | None = None, norm_weight: Tensor | None = None) -> Tensor:
+                    residual: Tensor | None = None, norm_weight: Tensor | None = None, fused_add: bool = False) -> Tensor:
             """The reference's forward(x) (int8_quant.py:703-778).  The optional arguments name the elementwise
             operation the caller would otherwise apply to x first -- _lib.PRO_GELU_TANH, _lib.PRO_MODULATE with
             (1 + mod_scale) * x + mod_shift, vectors broadcast over the token dimension, _lib.PRO_NORM_MODULATE with
@@ -515,7 +519,8 @@ class Int8TensorwiseOps(manual_cast):
             block), _lib.PRO_CONCAT_GELU with cat((x, gelu(mod_scale)), -1), the input of the second projection of a
             single-stream block, _lib.PRO_GELU_ERF (GELU in its exact form), _lib.PRO_RMS_NORM with
             rms_norm(x, norm_weight, eps) followed by * (1 + mod_scale) and + mod_shift where those are given (the
-            producer in blocks that normalise with an RMSNorm), or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
+            producer in blocks that normalise with an RMSNorm; fused_add=True in the three modulating kinds: product and
+            sum rounded once, as torch.addcmul(mod_shift, x, 1 + mod_scale) computes them), or _lib.PRO_SILU_GATE with silu(x) * mod_scale, the gate operand of x's shape -- which the W8A8
             path then applies inside its quantiser instead of in passes of their own (under torch.compile the graph
             rewrite of compile_ops does this without the caller's help).  `gate` / `residual` name what the caller would
             apply to the result: forward(h, gate=g, residual=x) returns x + g * linear(h), the gated residual of an
@@ -533,7 +538,7 @@ class Int8TensorwiseOps(manual_cast):
                                  and (gate is None or (gate.device == x.device and compile_ops.modulation_broadcasts_over_tokens(
                                      _ShapeAndDtype(out_shape, cdt), gate, gate))))
                 if not fuse_epilogue:   # torch applies the two operations, as the caller would have
-                    y = self.forward(x, prologue, mod_scale, mod_shift, eps, norm_weight=norm_weight)
+                    y = self.forward(x, prologue, mod_scale, mod_shift, eps, norm_weight=norm_weight, fused_add=fused_add)
                     if gate is not None:
                         y = gate * y
                     return y if residual is None else residual + y
@@ -541,6 +546,10 @@ class Int8TensorwiseOps(manual_cast):
                 rows = x.numel() // max(1, x.shape[-1])
                 fusable = (self._is_quantized and rows > SMALL_BATCH_ROWS and self.lora_A is None
                            and not torch.compiler.is_compiling())
+                if prologue == _lib.PRO_MODULATE_FUSED:
+                    prologue, fused_add = _lib.PRO_MODULATE, True
+                if fused_add and x.dtype not in (torch.float16, torch.bfloat16):
+                    fusable = False                      # (the one-rounding form exists for 16-bit tensors)
                 if fusable and prologue == _lib.PRO_CONCAT_GELU:   # x followed by gelu(mod_scale) along the feature dimension
                     fusable = (isinstance(mod_scale, Tensor) and mod_scale.shape[:-1] == x.shape[:-1]
                                and x.shape[-1] + mod_scale.shape[-1] == self.weight.shape[1]
@@ -572,14 +581,19 @@ class Int8TensorwiseOps(manual_cast):
                         x = F.gelu(x)
                     elif prologue == _lib.PRO_RMS_NORM:
                         x = F.rms_norm(x, (x.shape[-1],), norm_weight, eps)
-                        if mod_scale is not None:
-                            x = x * (1 + mod_scale)
-                        if mod_shift is not None:
-                            x = x + mod_shift
+                        if fused_add and mod_scale is not None and mod_shift is not None:
+                            x = torch.addcmul(mod_shift, x, 1 + mod_scale)
+                        else:
+                            if mod_scale is not None:
+                                x = x * (1 + mod_scale)
+                            if mod_shift is not None:
+                                x = x + mod_shift
                     elif prologue == _lib.PRO_CONCAT_GELU:
                         x = torch.cat((x, F.gelu(mod_scale, approximate="tanh")), -1)
                     elif prologue == _lib.PRO_SILU_GATE:
                         x = F.silu(x) * mod_scale
+                    elif fused_add:
+                        x = torch.addcmul(mod_shift, x, 1 + mod_scale)
                     else:
                         x = (1 + mod_scale) * x + mod_shift
                     prologue = _lib.PRO_NONE
@@ -657,7 +671,7 @@ class Int8TensorwiseOps(manual_cast):
                                                       int8_fused_kernel.DEFAULT_EPILOGUE, addend)
                 else:
                     fwd = int8_forward_dynamic_per_row if self._is_per_row else int8_forward_dynamic
-                    pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift, eps, norm_weight)
+                    pro = None if prologue == _lib.PRO_NONE else (prologue, mod_scale, mod_shift, eps, norm_weight, fused_add)
                     if fuse_epilogue:   # (no dynamic LoRA here: the addend slot is free for the residual stream)
                         addend = None if residual is None else residual.reshape(-1, residual.shape[-1])
                     y = fwd(x_2d, weight, w_scale, bias, compute_dtype, rotate=rotate, addend=addend, prologue=pro,

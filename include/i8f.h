@@ -84,12 +84,15 @@ typedef enum i8f_epilogue { I8F_EPI_TORCH = 0, I8F_EPI_FUSED = 1 } i8f_epilogue;
  *   I8F_PRO_CONCAT_GELU  cat(a, gelu(b, approximate="tanh")) along the row; taken by
  *                      i8f_quant_rowwise_concat_gelu only, which carries the second tensor
  *   I8F_PRO_GELU_ERF   gelu(x) in its exact form, 0.5 x (1 + erf(x / sqrt 2)), in binary32, rounded once to x's dtype
+ *   I8F_PRO_MODULATE_FUSED  the same modulation as torch.addcmul(t, x, 1 + s) computes it: the gain 1 + s rounded to x's
+ *                      dtype, its product with x (exact in binary32) added to t and rounded ONCE; 16-bit dtypes only.
+ *                      The norm entry points below take the same choice as their modulate_fused argument.
  *   I8F_PRO_RMS_NORM   rms_norm(x, weight, eps), optionally followed by (1 + s[k]) * y and + t[k]; taken by
  *                      i8f_quant_rowwise_rms_norm only, which carries the epsilon and the weight
  */
 typedef enum i8f_prologue {
     I8F_PRO_NONE = 0, I8F_PRO_MODULATE = 1, I8F_PRO_GELU_TANH = 2, I8F_PRO_SILU_GATE = 3, I8F_PRO_NORM_MODULATE = 4,
-    I8F_PRO_CONCAT_GELU = 5, I8F_PRO_GELU_ERF = 6, I8F_PRO_RMS_NORM = 7
+    I8F_PRO_CONCAT_GELU = 5, I8F_PRO_GELU_ERF = 6, I8F_PRO_RMS_NORM = 7, I8F_PRO_MODULATE_FUSED = 8
 } i8f_prologue;
 
 /* Library version (I8F_VERSION of the build). */
@@ -172,14 +175,16 @@ int i8f_quant_rowwise_prologue(const void *x, int x_dtype, int64_t M, int64_t K,
  * torch's LayerNorm takes its sums in another order and its reciprocal square root from the
  * hardware, so y agrees with it to the last place of the dtype (tests state the tolerance).
  *   mod_scale, mod_shift, rows_per_vec: as for I8F_PRO_MODULATE.
+ *   modulate_fused   0: three rounded operations; 1: z = round((1 + s[k]) * y + t[k]) with the gain rounded and the
+ *                    product and sum rounded once, as torch.addcmul(shift, y, 1 + scale) (I8F_PRO_MODULATE_FUSED)
  * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 16384 and x, q and
  * the vectors are 16-byte aligned (the row stays in the registers of one to four wavefronts): other callers
  * normalise with their own kernel and use I8F_PRO_MODULATE.
  */
 int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                                     float eps, const void *mod_scale, const void *mod_shift,
-                                    int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale,
-                                    void *stream);
+                                    int64_t rows_per_vec, int modulate_fused, int rotate_block, int8_t *q,
+                                    float *scale, void *stream);
 
 /*
  * The quantiser with an RMSNorm, and optionally the modulation behind it, in front of it:
@@ -196,13 +201,15 @@ int i8f_quant_rowwise_norm_modulate(const void *x, int x_dtype, int64_t M, int64
  * The row's sum is taken in this kernel's order, torch's in its own: y agrees with torch's to the last place of the
  * dtype (tests state the tolerance).
  *   weight [K] of x_dtype or NULL; mod_scale, mod_shift [ceil(M / rows_per_vec), K] of x_dtype or NULL each;
- *   rows_per_vec as for I8F_PRO_MODULATE (ignored when both are NULL).
+ *   rows_per_vec as for I8F_PRO_MODULATE (ignored when both are NULL); modulate_fused as for
+ *   i8f_quant_rowwise_norm_modulate (it matters only when both scale and shift are given).
  * I8F_ERR_UNSUPPORTED unless x_dtype is I8F_BF16 or I8F_F16, K % 16 == 0, K <= 16384 and x, q and the vectors are
  * 16-byte aligned (the row stays in the registers of one to four wavefronts): other callers normalise with their own kernel.
  */
 int i8f_quant_rowwise_rms_norm(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, float eps,
                                const void *weight, const void *mod_scale, const void *mod_shift,
-                               int64_t rows_per_vec, int rotate_block, int8_t *q, float *scale, void *stream);
+                               int64_t rows_per_vec, int modulate_fused, int rotate_block, int8_t *q, float *scale,
+                               void *stream);
 
 /*
  * The quantiser on the concatenation of two tensors along the row, the second through tanh-GELU:

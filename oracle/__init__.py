@@ -45,8 +45,8 @@ def lib() -> ctypes.CDLL:
         L.orc_quant_rowwise.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp]
         L.orc_quant_tensorwise.argtypes = [vp, i32, i64, vp, vp]
         L.orc_prologue.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i64, vp]
-        L.orc_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, vp]
-        L.orc_rms_norm.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, vp, i64, vp]
+        L.orc_norm_modulate.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, i64, i32, vp]
+        L.orc_rms_norm.argtypes = [vp, i32, i64, i64, i64, f32, vp, vp, vp, i64, i32, vp]
         L.orc_gemm_i32.argtypes = [vp, vp, i64, i64, i64, vp]
         L.orc_epilogue.argtypes = [vp, vp, vp, i32, vp, i32, vp, i32, i64, i64, i32]
         L.orc_linear_w8a8.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, i32, vp, i32, vp, i32, i64, i32]
@@ -169,7 +169,7 @@ def quant_tensorwise(x, dtype_code):
     return q, s
 
 
-PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE, PRO_GELU_ERF = 1, 2, 3, 4, 6
+PRO_MODULATE, PRO_GELU_TANH, PRO_SILU_GATE, PRO_NORM_MODULATE, PRO_GELU_ERF, PRO_MODULATE_FUSED = 1, 2, 3, 4, 6, 8
 
 
 def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
@@ -177,7 +177,7 @@ def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
     torch's eager kernels do; returns the storage array of dtype_code, shape of x."""
     x = _arr(x, dtype_code)
     M, K = x.shape
-    if kind == PRO_MODULATE:
+    if kind in (PRO_MODULATE, PRO_MODULATE_FUSED):
         s, t = _arr(s, dtype_code).reshape(-1, K), _arr(t, dtype_code).reshape(-1, K)
         assert s.shape == t.shape and s.shape[0] * rows_per_vec >= M
     elif kind == PRO_SILU_GATE:
@@ -189,19 +189,20 @@ def prologue(x, dtype_code, kind, s=None, t=None, rows_per_vec=1):
     return out
 
 
-def norm_modulate(x, dtype_code, eps, s, t, rows_per_vec=1):
+def norm_modulate(x, dtype_code, eps, s, t, rows_per_vec=1, fused=False):
     """(1 + s) * layer_norm(x, eps) + t without affine parameters, every tensor operation rounded to the dtype as
-    torch's eager kernels do; returns the storage array of dtype_code, shape of x."""
+    torch's eager kernels do (fused: the product and the sum as torch.addcmul, one rounding); returns the storage array
+    of dtype_code, shape of x."""
     x = _arr(x, dtype_code)
     M, K = x.shape
     s, t = _arr(s, dtype_code).reshape(-1, K), _arr(t, dtype_code).reshape(-1, K)
     assert s.shape == t.shape and s.shape[0] * rows_per_vec >= M
     out = np.empty((M, K), dtype=x.dtype)
-    _chk(lib().orc_norm_modulate(_p(x), dtype_code, M, K, K, float(eps), _p(s), _p(t), rows_per_vec, _p(out)), "norm_modulate")
+    _chk(lib().orc_norm_modulate(_p(x), dtype_code, M, K, K, float(eps), _p(s), _p(t), rows_per_vec, int(bool(fused)), _p(out)), "norm_modulate")
     return out
 
 
-def rms_norm(x, dtype_code, eps, w=None, s=None, t=None, rows_per_vec=1):
+def rms_norm(x, dtype_code, eps, w=None, s=None, t=None, rows_per_vec=1, fused=False):
     """rms_norm(x, w, eps) rounded once to the dtype as torch's kernel does, then (1 + s) * y and + t where given, each
     rounded; returns the storage array of dtype_code, shape of x."""
     x = _arr(x, dtype_code)
@@ -213,7 +214,7 @@ def rms_norm(x, dtype_code, eps, w=None, s=None, t=None, rows_per_vec=1):
         assert v is None or v.shape[0] * rows_per_vec >= M
     out = np.empty((M, K), dtype=x.dtype)
     _chk(lib().orc_rms_norm(_p(x), dtype_code, M, K, K, float(eps), *(None if v is None else _p(v) for v in (w, s, t)),
-                            rows_per_vec, _p(out)), "rms_norm")
+                            rows_per_vec, int(bool(fused)), _p(out)), "rms_norm")
     return out
 
 

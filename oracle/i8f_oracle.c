@@ -262,23 +262,26 @@ int orc_quant_rowwise(const void *x, int dtype, int64_t M, int64_t K, int64_t ld
  *           library's: a tolerance reference like kind 2
  *   kind 6  gelu(x) in its exact form, x * 0.5 * (1 + erf(x / sqrt 2)) in binary32 as torch's kernel writes it,
  *           rounded once to dtype (erff is the C library's: a tolerance reference)
+ *   kind 8  torch.addcmul(t, x, 1 + s): the gain 1 + s rounded to dtype (a tensor of its own), then t + x * gain in
+ *           binary32 (the product of two 16-bit values is exact there) rounded once to dtype
  * out is [M,K] of dtype, contiguous.  Followed by orc_quant_rowwise it is the
  * oracle of the fused quantiser.
  */
 int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, int kind,
                  const void *s, const void *t, int64_t rows_per_vec, void *out) {
-    if (M < 0 || K < 0 || ldx < K || (kind != 1 && kind != 2 && kind != 3 && kind != 6)) return -1;
-    if (kind == 1 && (rows_per_vec <= 0 || !s || !t)) return -1;
+    if (M < 0 || K < 0 || ldx < K || (kind != 1 && kind != 2 && kind != 3 && kind != 6 && kind != 8)) return -1;
+    if ((kind == 1 || kind == 8) && (rows_per_vec <= 0 || !s || !t)) return -1;
     if (kind == 3 && (rows_per_vec <= 0 || !s)) return -1;
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; ++m) {
         for (int64_t k = 0; k < K; ++k) {
             const float xv = load_as_f32(x, dtype, (size_t)(m * ldx + k));
             float v;
-            if (kind == 1) {
+            if (kind == 1 || kind == 8) {
                 const size_t vi = (size_t)((m / rows_per_vec) * K + k);
                 const float a = round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype);
-                const float b = round_to_dtype(a * xv, dtype);
+                const float p = a * xv;
+                const float b = kind == 8 ? p : round_to_dtype(p, dtype);
                 v = b + load_as_f32(t, dtype, vi);
             } else if (kind == 3) {
                 /* silu(x) * g as two tensor operations: x / (1 + exp(-x)) in binary32, rounded to the dtype, then
@@ -309,7 +312,7 @@ int orc_prologue(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, in
  * The row's sum is taken in double (torch takes it in binary32 in its own order).
  */
 int orc_rms_norm(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, float eps, const void *w,
-                 const void *s, const void *t, int64_t rows_per_vec, void *out) {
+                 const void *s, const void *t, int64_t rows_per_vec, int fused, void *out) {
     if (M < 0 || K <= 0 || ldx < K || ((s || t) && rows_per_vec <= 0)) return -1;
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; ++m) {
@@ -324,7 +327,10 @@ int orc_rms_norm(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, fl
             float y = load_as_f32(x, dtype, (size_t)(m * ldx + k)) * rstd;
             if (w) y = y * load_as_f32(w, dtype, (size_t)k);
             y = round_to_dtype(y, dtype);
-            if (s) y = round_to_dtype(round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype) * y, dtype);
+            if (s) {
+                y = round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype) * y;
+                if (!(fused && t)) y = round_to_dtype(y, dtype);   /* fused with a shift: torch.addcmul(t, y, 1 + s) */
+            }
             if (t) y = y + load_as_f32(t, dtype, vi);
             store_from_f32(out, dtype, (size_t)(m * K + k), y);
         }
@@ -342,7 +348,7 @@ int orc_rms_norm(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, fl
  * mean and rstd are then binary32 values and the elementwise part runs in binary32 as torch's does.
  */
 int orc_norm_modulate(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, float eps,
-                      const void *s, const void *t, int64_t rows_per_vec, void *out) {
+                      const void *s, const void *t, int64_t rows_per_vec, int fused, void *out) {
     if (M < 0 || K <= 0 || ldx < K || rows_per_vec <= 0 || !s || !t) return -1;
 #pragma omp parallel for schedule(static)
     for (int64_t m = 0; m < M; ++m) {
@@ -359,7 +365,7 @@ int orc_norm_modulate(const void *x, int dtype, int64_t M, int64_t K, int64_t ld
             const size_t vi = (size_t)((m / rows_per_vec) * K + k);
             const float y = round_to_dtype((load_as_f32(x, dtype, (size_t)(m * ldx + k)) - mean) * rstd, dtype);
             const float a = round_to_dtype(1.0f + load_as_f32(s, dtype, vi), dtype);
-            const float b = round_to_dtype(a * y, dtype);
+            const float b = fused ? a * y : round_to_dtype(a * y, dtype);   /* fused: torch.addcmul(t, y, 1 + s), one rounding */
             store_from_f32(out, dtype, (size_t)(m * K + k), b + load_as_f32(t, dtype, vi));
         }
     }

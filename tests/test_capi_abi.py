@@ -96,16 +96,16 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 24, 0, 0.0, one, L.BF16, 32, 32, 128, 0, null) == UNSUPPORTED
     assert lib.i8f_linear_w8a8_lora(one, one, one, one, 1.0, 1, null, 0, one, one, 80, 0, 0.0, one, L.BF16, 32, 32, 128, 0, null) == UNSUPPORTED
     # normalising quantiser: operands missing, negative eps, binary32 rows
-    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 256, 256, 1e-6, null, one, 4, 0, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 256, 256, -1.0, one, one, 4, 0, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 256, 256, 1e-6, one, one, 0, 0, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 200, 200, 1e-6, one, one, 4, 128, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_norm_modulate(null, L.BF16, 0, 256, 256, 1e-6, null, null, 1, 0, null, null, null) == 0
-    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 256, 256, -1.0, null, null, null, 1, 0, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 256, 256, 1e-6, null, one, null, 0, 0, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 200, 200, 1e-6, null, null, null, 1, 128, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 256, 128, 1e-6, null, null, null, 1, 0, one, one, null) == INVALID
-    assert lib.i8f_quant_rowwise_rms_norm(null, L.BF16, 0, 256, 256, 1e-6, null, null, null, 1, 0, null, null, null) == 0
+    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 256, 256, 1e-6, null, one, 4, 0, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 256, 256, -1.0, one, one, 4, 0, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 256, 256, 1e-6, one, one, 0, 0, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_norm_modulate(one, L.BF16, 4, 200, 200, 1e-6, one, one, 4, 0, 128, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_norm_modulate(null, L.BF16, 0, 256, 256, 1e-6, null, null, 1, 0, 0, null, null, null) == 0
+    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 256, 256, -1.0, null, null, null, 1, 0, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 256, 256, 1e-6, null, one, null, 0, 0, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 200, 200, 1e-6, null, null, null, 1, 0, 128, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 256, 128, 1e-6, null, null, null, 1, 0, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_rms_norm(null, L.BF16, 0, 256, 256, 1e-6, null, null, null, 1, 0, 0, null, null, null) == 0
     assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, 8, null, null, 1, 0, one, one, null) == INVALID
     assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, L.PRO_NORM_MODULATE, one, one, 4, 0, one, one, null) == INVALID  # needs its own entry point: it carries eps
     # concatenating quantiser: negative widths, operands missing, a rotation block that would straddle the seam, binary32,

@@ -311,6 +311,51 @@ def test_graph_rewrite_moves_rms_norm_and_exact_gelu_into_the_quantiser(pkg):
     assert not any(n_.target is F.gelu for n_ in gm.graph.nodes if n_.op == "call_function")
 
 
+def test_graph_rewrite_takes_the_addcmul_spelling_of_the_modulation(pkg):
+    """torch.addcmul(shift, norm(x), 1 + scale) -> linear, the modulation as one torch kernel (product and sum rounded once):
+    fused with the flag that keeps that rounding, behind a LayerNorm without affine, an RMSNorm or no norm at all, the
+    factors in either order; another `value`, binary32 tensors or a gain that is not 1 + scale stay torch's."""
+    g = torch.Generator().manual_seed(26)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=False)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3})
+
+    class Block(torch.nn.Module):
+        def __init__(self, norm, form="plain"):
+            super().__init__()
+            self.norm = {"ln": torch.nn.LayerNorm(128, elementwise_affine=False, eps=1e-6), "rms": torch.nn.RMSNorm(128, eps=1e-5).bfloat16(),
+                         "none": torch.nn.Identity()}[norm]
+            self.qkv, self.form = lin(64, 128), form
+
+        def forward(self, x, scale, shift):
+            h = self.norm(x)
+            if self.form == "swapped":
+                z = torch.addcmul(shift, 1 + scale, h)
+            elif self.form == "value":
+                z = torch.addcmul(shift, h, 1 + scale, value=2)
+            elif self.form == "gain":
+                z = torch.addcmul(shift, h, scale)
+            else:
+                z = torch.addcmul(shift, h, 1 + scale)
+            return self.qkv(z)
+
+    x, v = torch.randn(2, 24, 128).bfloat16(), torch.randn(2, 1, 128).bfloat16()
+    for norm, form, kind in (("ln", "plain", "PRO_NORM_MODULATE"), ("rms", "plain", "PRO_RMS_NORM"), ("none", "plain", "PRO_MODULATE"),
+                             ("ln", "swapped", "PRO_NORM_MODULATE")):
+        gm = torch._dynamo.export(Block(norm, form))(x, v, v).graph_module
+        assert pkg.compile_ops.fuse_prologues(gm) == 1
+        node = [n for n in gm.graph.nodes if n.op == "call_function" and "int8_linear_prologue" in str(n.target)][0]
+        assert node.args[1] == getattr(pkg._lib, kind) and node.kwargs.get("fused_add") is True
+        assert not any(n.target is torch.addcmul for n in gm.graph.nodes if n.op == "call_function")
+    for norm, form in (("ln", "value"), ("ln", "gain")):
+        gm = torch._dynamo.export(Block(norm, form))(x, v, v).graph_module
+        assert pkg.compile_ops.fuse_prologues(gm) == 0
+    gm = torch._dynamo.export(Block("none"))(x.float(), v.float(), v.float()).graph_module
+    assert pkg.compile_ops.fuse_prologues(gm) == 0
+
+
 def test_graph_rewrite_moves_concatenation_and_gelu_into_the_quantiser(pkg):
     """linear2(cat((attn, gelu(mlp)), -1)), the second projection of a single-stream block: both producers become the
     layer's prologue; a concatenation along another dimension, of three tensors, or with an exact GELU stays torch's."""
@@ -949,6 +994,68 @@ def test_compiled_in_place_residual_update_equals_eager(pkg, dev):
         assert seen == [(2, 0)]
         want = m(img, tok, a_img, a_txt, g_img, g_txt)
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+@pytest.mark.gpu
+def test_compiled_block_in_the_spelling_of_the_model_code_equals_eager(pkg, dev):
+    """One stream of a double-stream block as the model's Python writes it -- apply_mod(t, m, a) = torch.addcmul(a, t, m),
+    apply_mod(t, m) = t * m: qkv(apply_mod(norm1(x), 1 + scale1, shift1)), x = x + apply_mod(proj(a), gate1),
+    x += apply_mod(mlp(apply_mod(norm2(x), 1 + scale2, shift2)), gate2) -- under the rewriting backend: every layer
+    carries its producer or its residual update, nothing elementwise is left for inductor but the attention stand-in,
+    and the result is that of the eager fused calls bit for bit (and that of the module in eager mode up to the
+    roundings of the in-quantiser LayerNorm, carried through four layers)."""
+    g = torch.Generator().manual_seed(27)
+
+    def lin(n_out, k_in):
+        l = pkg.Int8TensorwiseOps.Linear(k_in, n_out, bias=True)
+        return _load(l, {"weight": torch.randint(-127, 128, (n_out, k_in), dtype=torch.int8, generator=g),
+                         "weight_scale": torch.rand(n_out, 1, generator=g) * 0.002 + 1e-3, "bias": (torch.randn(n_out, generator=g) * 0.1).bfloat16()})
+
+    def apply_mod(tensor, m_mult, m_add=None):
+        return torch.addcmul(m_add, tensor, m_mult) if m_add is not None else tensor * m_mult
+
+    class Stream(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm1 = torch.nn.LayerNorm(256, elementwise_affine=False, eps=1e-6)
+            self.norm2 = torch.nn.LayerNorm(256, elementwise_affine=False, eps=1e-6)
+            self.qkv, self.proj, self.up, self.down = lin(768, 256), lin(256, 256), lin(1024, 256), lin(256, 1024)
+
+        def forward(self, x, shift1, scale1, gate1, shift2, scale2, gate2):
+            x = x * 1.0                                                   # (an intermediate, as inside a model)
+            q, k, v = self.qkv(apply_mod(self.norm1(x), 1 + scale1, shift1)).chunk(3, dim=-1)
+            attn = q + v                                                  # (stands in for the attention: ONE rounded operation, as inductor keeps chains in binary32)
+            x = x + apply_mod(self.proj(attn), gate1)
+            x += apply_mod(self.down(F.gelu(self.up(apply_mod(self.norm2(x), 1 + scale2, shift2)), approximate="tanh")), gate2)
+            return x
+
+    m = Stream().to(dev)
+    x = (torch.randn(2, 48, 256, generator=g) * 2).bfloat16().to(dev)
+    mods = [(torch.randn(2, 1, 256, generator=g) * 0.3).bfloat16().to(dev) for _ in range(6)]
+    seen = []
+
+    def counting(gm, inputs):
+        calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+        seen.append((sum("int8_linear_prologue" in str(n.target) for n in calls),
+                     sum(n.kwargs.get("gate") is not None and n.kwargs.get("addend") is not None for n in calls),
+                     sum(n.target in (torch.addcmul, operator.iadd) or "layer_norm" in str(n.target) or "gelu" in str(n.target) for n in calls)))
+        from torch._dynamo.backends.registry import lookup_backend
+        return lookup_backend("inductor")(gm, inputs)
+
+    with torch.no_grad():
+        got = torch.compile(m, backend=pkg.compile_ops.backend(counting), fullgraph=True)(x, *mods)
+        assert seen == [(3, 2, 0)]            # qkv, up, down carry a prologue; proj and down the gated residual
+        L = pkg._lib
+        shift1, scale1, gate1, shift2, scale2, gate2 = mods
+        x0 = x * 1.0
+        q, k, v = m.qkv(x0, prologue=L.PRO_NORM_MODULATE, mod_scale=scale1, mod_shift=shift1, eps=1e-6, fused_add=True).chunk(3, dim=-1)
+        x1 = m.proj(q + v, gate=gate1, residual=x0)
+        h = m.up(x1, prologue=L.PRO_NORM_MODULATE, mod_scale=scale2, mod_shift=shift2, eps=1e-6, fused_add=True)
+        want = m.down(h, prologue=L.PRO_GELU_TANH, gate=gate2, residual=x1)
+        assert torch.equal(got, want)
+        loose = m(x, *mods)
+    diff = (got.float() - loose.float()).abs()
+    assert diff.max().item() <= 2.0**-4 * loose.float().abs().max().item() and diff.mean().item() <= 2.0**-9 * loose.float().abs().max().item()
 
 
 @pytest.mark.gpu

@@ -289,6 +289,11 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
         b = lin((1 + sc) * F.layer_norm(x, (384,), eps=1e-6) + sh)
         assert a.shape == (2, 20, 96) and (a.float() - b.float()).abs().max() <= 2.0**-6 * b.float().abs().max()
         assert (a != b).float().mean().item() <= 0.2
+        a = lin(x, prologue=L.PRO_MODULATE, mod_scale=sc, mod_shift=sh, fused_add=True)     # the one-kernel spelling of the modulation
+        assert torch.equal(a, lin(torch.addcmul(sh, x, 1 + sc))) and torch.equal(a, lin(x, prologue=L.PRO_MODULATE_FUSED, mod_scale=sc, mod_shift=sh))
+        a = lin(x, prologue=L.PRO_NORM_MODULATE, mod_scale=sc, mod_shift=sh, eps=1e-6, fused_add=True)
+        b = lin(torch.addcmul(sh, F.layer_norm(x, (384,), eps=1e-6), 1 + sc))
+        assert (a.float() - b.float()).abs().max() <= 2.0**-6 * b.float().abs().max() and (a != b).float().mean().item() <= 0.2
         a = lin(x, prologue=L.PRO_GELU_ERF)
         b = lin(F.gelu(x))
         assert (a.float() - b.float()).abs().max() <= 2.0**-7 * b.float().abs().max()
@@ -315,6 +320,9 @@ def test_forward_with_a_prologue_equals_the_unfused_sequence(pkg, dev):
                        lin(F.rms_norm(small, (384,), nw, 1e-5) * (1 + sc[:1])))
     assert torch.equal(lin(x, prologue=L.PRO_RMS_NORM, norm_weight=nw.float(), eps=1e-5), lin(F.rms_norm(x, (384,), nw.float(), 1e-5)))
     assert torch.equal(lin(small, prologue=L.PRO_GELU_ERF), lin(F.gelu(small)))
+    assert torch.equal(lin(small, prologue=L.PRO_MODULATE, mod_scale=sc[:1], mod_shift=sh[:1], fused_add=True), lin(torch.addcmul(sh[:1], small, 1 + sc[:1])))
+    assert torch.equal(lin(x.float(), prologue=L.PRO_MODULATE_FUSED, mod_scale=sc.float(), mod_shift=sh.float()),
+                       lin(torch.addcmul(sh.float(), x.float(), 1 + sc.float())))
     # rows that the normalising quantiser does not take (binary32 here): torch normalises, and the result is that of
     # the unfused expression
     x32, sc_, sh_ = x.float(), sc.float(), sh.float()

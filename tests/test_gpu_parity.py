@@ -142,6 +142,17 @@ def test_quant_rowwise_modulate_prologue_bit_exact(L, dev, M, K, dt, rot, V):
     t = ((1 + sc.to(dev)[:, None, :]) * xd.view(V, M // V, K) + sh.to(dev)[:, None, :]).reshape(M, K)
     q2, s2 = L.quant_rowwise(t, rotate=rot)
     assert torch.equal(q, q2) and torch.equal(s, s2)
+    if dt != torch.float32:   # the one-kernel spelling, torch.addcmul(shift, x, 1 + scale): product and sum rounded once
+        modf = O.prologue(xa, code, O.PRO_MODULATE_FUSED, O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=M // V)
+        qo, so = O.quant_rowwise(modf, code, 128 if rot else 0)
+        q, s = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_MODULATE_FUSED, mod_scale=sc.to(dev), mod_shift=sh.to(dev))
+        assert np.array_equal(q.cpu().numpy(), qo) and np.array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+        t = torch.addcmul(sh.to(dev)[:, None, :], xd.view(V, M // V, K), 1 + sc.to(dev)[:, None, :]).reshape(M, K)
+        q2, s2 = L.quant_rowwise(t, rotate=rot)
+        assert torch.equal(q, q2) and torch.equal(s, s2)
+    else:
+        with pytest.raises(ValueError):
+            L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_MODULATE_FUSED, mod_scale=sc.to(dev), mod_shift=sh.to(dev))
 
 
 @pytest.mark.parametrize("M,K,dt,rot,V", PROLOGUE_CASES)
@@ -215,6 +226,16 @@ def test_quant_rowwise_norm_modulate_prologue_within_tolerance(L, dev, M, K, dt,
         assert (np.abs(sc.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
     again = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_NORM_MODULATE, mod_scale=s.to(dev), mod_shift=t.to(dev), eps=eps)
     assert torch.equal(again[0], q) and torch.equal(again[1], sc)     # fixed order of the sums: launches agree bit for bit
+    # the modulation as torch.addcmul (one rounding for product and sum): same bar against the oracle's fused form and torch's
+    zf = O.norm_modulate(xa, code, eps, O.from_torch(s)[0], O.from_torch(t)[0], rows_per_vec=rows // V, fused=True)
+    qo, so = O.quant_rowwise(zf, code, 128 if rot else 0)
+    q, sc = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_NORM_MODULATE, mod_scale=s.to(dev), mod_shift=t.to(dev), eps=eps, fused_add=True)
+    zt = torch.addcmul(t.to(dev)[:, None], torch.nn.functional.layer_norm(xd, (K,), eps=eps), 1 + s.to(dev)[:, None]).reshape(rows, K)
+    q2, s2 = L.quant_rowwise(zt, rotate=rot)
+    for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+        d = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() <= (2e-2 if rot else 5e-3)
+        assert (np.abs(sc.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
 
 
 @pytest.mark.parametrize("M,K,dt,rot,V", PROLOGUE_CASES)
@@ -272,6 +293,16 @@ def test_quant_rowwise_rms_norm_prologue_within_tolerance(L, dev, M, K, dt, rot,
         assert (np.abs(sc.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
     again = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_RMS_NORM, norm_weight=d(w), mod_scale=d(s), mod_shift=d(t), eps=eps)
     assert torch.equal(again[0], q) and torch.equal(again[1], sc)
+    if s is not None and t is not None:   # with both: the fused spelling, torch.addcmul(shift, norm(x), 1 + scale)
+        zf = O.rms_norm(xa, code, eps, *(None if v is None else O.from_torch(v)[0] for v in (w, s, t)), rows_per_vec=rows // V, fused=True)
+        qo, so = O.quant_rowwise(zf, code, 128 if rot else 0)
+        q, sc = L.quant_rowwise(x.to(dev), rotate=rot, prologue=L.PRO_RMS_NORM, norm_weight=d(w), mod_scale=d(s), mod_shift=d(t), eps=eps, fused_add=True)
+        zt = torch.addcmul(d(t)[:, None], torch.nn.functional.rms_norm(x.to(dev), (K,), d(w), eps).reshape(V, rows // V, K), 1 + d(s)[:, None])
+        q2, s2 = L.quant_rowwise(zt.reshape(rows, K), rotate=rot)
+        for qr, sr in ((qo, so), (q2.cpu().numpy(), s2.cpu().numpy())):
+            df = np.abs(q.cpu().numpy().astype(np.int32) - qr.astype(np.int32))
+            assert df.max() <= 1 and (df != 0).mean() <= (2e-2 if rot else 5e-3)
+            assert (np.abs(sc.cpu().numpy() - sr) <= 2 * ulp * np.abs(sr)).all()
     if parts == "":      # nothing but the normalisation: invariant under a positive power-of-two factor (eps scaled with it)
         q4, s4 = L.quant_rowwise((x.float() * 4).to(dt).to(dev), rotate=rot, prologue=L.PRO_RMS_NORM, eps=eps * 16)
         assert torch.equal(q4, q) and torch.equal(s4, sc)

@@ -566,6 +566,38 @@ def test_norm_modulate_agrees_with_torch(dt):
     assert torch.equal(got3.view(torch.int16), tv[:1, :64].contiguous().view(torch.int16))
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_prologue_fused_modulation_equals_torch_addcmul(dt):
+    """torch.addcmul(shift, x, 1 + scale), the one-kernel spelling of the modulation (the gain a rounded tensor of its
+    own, product and sum rounded once): bit-equal on 16-bit CPU tensors, vectors dealt over groups of rows; it differs
+    from the three-operation form exactly where the extra rounding of the product matters; and the two normalising
+    oracles' fused forms equal this kind applied to their own normalised tensor."""
+    g = torch.Generator().manual_seed(35)
+    x = (torch.randn(2 * 6, 200, generator=g) * 3).to(dt)
+    sc, sh = (torch.randn(2, 200, generator=g) * 0.3).to(dt), torch.randn(2, 200, generator=g).to(dt)
+    want = torch.addcmul(sh[:, None, :], x.view(2, 6, 200), 1 + sc[:, None, :]).reshape(12, 200)
+    xa, code = O.from_torch(x)
+    got = O.prologue(xa, code, O.PRO_MODULATE_FUSED, O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=6)
+    assert np.array_equal(got, O.from_torch(want)[0])
+    three = O.prologue(xa, code, O.PRO_MODULATE, O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=6)
+    assert 0.01 < (got != three).mean() < 0.6
+    w = (torch.randn(200, generator=g) * 0.2 + 1).to(dt)
+    y = O.rms_norm(xa, code, 1e-5, O.from_torch(w)[0])
+    fused = O.rms_norm(xa, code, 1e-5, O.from_torch(w)[0], O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=6, fused=True)
+    assert np.array_equal(fused, O.prologue(y, code, O.PRO_MODULATE_FUSED, O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=6))
+    only_s = O.rms_norm(xa, code, 1e-5, O.from_torch(w)[0], O.from_torch(sc)[0], None, rows_per_vec=6, fused=True)   # no shift: nothing to fuse
+    assert np.array_equal(only_s, O.rms_norm(xa, code, 1e-5, O.from_torch(w)[0], O.from_torch(sc)[0], None, rows_per_vec=6))
+    # LayerNorm form: against torch end to end within the tolerance of the normalised value, and tighter than the
+    # three-operation form is to the same target
+    want_ln = torch.addcmul(sh[:, None, :], torch.nn.functional.layer_norm(x, (200,), eps=1e-6).view(2, 6, 200), 1 + sc[:, None, :]).reshape(12, 200)
+    got_ln = O.to_f32(O.norm_modulate(xa, code, 1e-6, O.from_torch(sc)[0], O.from_torch(sh)[0], rows_per_vec=6, fused=True), code)
+    wl = want_ln.float().numpy()
+    ulp = {torch.bfloat16: 2.0**-7, torch.float16: 2.0**-10}[dt]
+    yl = torch.nn.functional.layer_norm(x.float(), (200,), eps=1e-6).numpy()
+    gain = np.abs(1 + sc.float().numpy()).repeat(6, 0)
+    assert (np.abs(got_ln - wl) <= ulp * (np.abs(yl) * gain + np.abs(wl)) + 1e-30).all() and (got_ln != wl).mean() < 2e-2
+
+
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
 def test_prologue_gelu_erf_agrees_with_torch_and_with_the_normal_distribution(dt):
     """GELU in its exact form, x Phi(x): against torch's gelu (same binary32 expression, its own vectorised erf: at most
