@@ -28,6 +28,8 @@ hands the graph to `inner` ("inductor" by default):
 
     model = torch.compile(model, backend=compile_ops.backend())
 """
+import copy
+import logging
 import operator
 from typing import Optional, Tuple
 
@@ -758,8 +760,16 @@ def install_inductor_pass() -> bool:
         if before is not None:
             before(graph)
         gm = graph.owning_module
-        if gm is not None and any("i8f" in str(n.target) for n in graph.nodes if n.op == "call_function"):
-            LAST_PASS_COUNTS = rewrite(gm)
+        if gm is None or not any("i8f" in str(n.target) for n in graph.nodes if n.op == "call_function"):
+            return
+        # Somebody else's compile must not fail over a graph these rewrites were not written for: they are tried on a
+        # copy first, and a graph on which they raise is compiled as it is.
+        try:
+            rewrite(copy.deepcopy(gm))
+        except Exception as e:  # noqa: BLE001
+            logging.getLogger(__name__).warning("INT8 Fast: graph rewrites skipped for this graph (%s: %s)", type(e).__name__, e)
+            return
+        LAST_PASS_COUNTS = rewrite(gm)
 
     inductor_config.pre_grad_custom_pass = i8f_pre_grad_pass
     _installed = True

@@ -488,6 +488,48 @@ def test_graph_rewrite_takes_the_in_place_residual_update_where_nobody_can_tell(
         assert any(n.target is operator.iadd for n in gm.graph.nodes if n.op == "call_function") == (not with_residual), form
 
 
+def test_installed_pass_rewrites_a_graph_and_steps_aside_when_a_rewrite_raises(pkg, monkeypatch):
+    """compile_ops.install_inductor_pass(): the function it registers with inductor rewrites a graph that holds this
+    package's operators, leaves other graphs alone, chains to a pass that was registered before it, and compiles a graph
+    as it is when a rewrite raises on it (tried on a copy first)."""
+    import torch._inductor.config as inductor_config
+    g = torch.Generator().manual_seed(28)
+    lin = pkg.Int8TensorwiseOps.Linear(64, 128, bias=False)
+    _load(lin, {"weight": torch.randint(-127, 128, (128, 64), dtype=torch.int8, generator=g), "weight_scale": torch.rand(128, 1, generator=g) * 0.002 + 1e-3})
+
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = lin
+
+        def forward(self, x):
+            return self.up(F.gelu(x, approximate="tanh"))
+
+    seen = []
+    monkeypatch.setattr(inductor_config, "pre_grad_custom_pass", lambda graph: seen.append("earlier pass"))
+    monkeypatch.setattr(pkg.compile_ops, "_installed", False)
+    assert pkg.compile_ops.install_inductor_pass()
+    hook = inductor_config.pre_grad_custom_pass
+    x = torch.randn(2, 24, 64).bfloat16()
+    gm = torch._dynamo.export(Mlp())(x).graph_module
+    hook(gm.graph)
+    assert seen == ["earlier pass"] and pkg.compile_ops.LAST_PASS_COUNTS == (0, 1, 0)
+    assert any("int8_linear_prologue" in str(n.target) for n in gm.graph.nodes)
+    other = torch._dynamo.export(torch.nn.GELU())(x).graph_module           # no operator of this package: untouched
+    before = [str(n.target) for n in other.graph.nodes]
+    hook(other.graph)
+    assert [str(n.target) for n in other.graph.nodes] == before
+    gm = torch._dynamo.export(Mlp())(x).graph_module
+    before = [str(n.target) for n in gm.graph.nodes]
+
+    def broken(_gm):
+        raise RuntimeError("a graph this rewrite was not written for")
+
+    monkeypatch.setattr(pkg.compile_ops, "fuse_prologues", broken)
+    hook(gm.graph)
+    assert [str(n.target) for n in gm.graph.nodes] == before
+
+
 def test_graph_rewrites_keep_away_from_in_place_writes(pkg):
     """A tensor overwritten in place between the point where the model reads it and the layer that would read it inside
     a fused operator: the rewrites leave that stretch of the graph alone (the fused read would see the new value)."""
