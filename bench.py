@@ -640,8 +640,8 @@ def extras(L, dev, quick=False):
     bufs = {(m, n): torch.empty(m, n, dtype=torch.bfloat16, device=dev) for m in (4096, 512) for n in (9216, 3072, 12288)}
 
     def block(_i):
-        for m in (4096, 512):   # image stream, text stream: the modulation vectors of each
-            L.linear_w8a16_small_m(vec, *lin[m]["adaln"])
+        # image stream, text stream: the modulation vectors of each, both small-batch layers in one launch
+        L.linear_w8a16_small_m_grouped([(vec,) + lin[m]["adaln"] for m in (4096, 512)])
         # each projection for both streams: their activations are quantised by one launch (they share the width,
         # not the weights), and their GEMMs go out together where the text stream's tiles fit into the CUs that the
         # image stream's last round leaves idle (the two projections into 3072 columns), else one launch per stream
@@ -675,6 +675,10 @@ def extras(L, dev, quick=False):
     out["adaln_w8a16_m1_18432x3072"] = {"median_us": round(t["median_us"], 2), "gbs": round(abytes / t["median_us"] / 1e3, 1),
                                         "frac_of_hbm_peak": round(abytes / t["median_us"] / 1e3 / PEAK_HBM_GBS, 4), "bytes": abytes,
                                         "note": "two 56.6 MB weights in turn: partly served by the 256 MB memory-side cache"}
+    tg = time_kernel(lambda i: L.linear_w8a16_small_m_grouped([(vec,) + a_ for a_ in ada]), max(10, iters // 4))
+    out["adaln_w8a16_m1_pair_in_one_launch"] = {"median_us": round(tg["median_us"], 2), "gbs": round(2 * abytes / tg["median_us"] / 1e3, 1),
+                                                "frac_of_hbm_peak": round(2 * abytes / tg["median_us"] / 1e3 / PEAK_HBM_GBS, 4), "bytes": 2 * abytes,
+                                                "note": "the modulation projections of both streams of a block (113 MB of weights) as one grid"}
 
     t_sep = time_kernel(block_separate, max(10, iters // 4))
     t_qg = time_kernel(block_quant_grouped, max(10, iters // 4))

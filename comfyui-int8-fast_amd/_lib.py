@@ -75,10 +75,11 @@ def lib() -> ctypes.CDLL:
     L.i8f_linear_w8a8_workspace_bytes.restype = i64
     L.i8f_linear_w8a8_lora.argtypes = [vp, vp, vp, vp, f32, i32, vp, i32, vp, vp, i64, i32, f32, vp, i32, i64, i64, i64, i32, vp]
     L.i8f_linear_w8a16_small_m.argtypes = [vp, i32, i64, i64, i64, vp, vp, f32, i32, vp, i32, vp, i64, vp]
+    L.i8f_linear_w8a16_small_m_grouped.argtypes = [vp, i32, i32, i32, i32, vp]
     L.i8f_sr_quant_delta.argtypes = [vp, vp, f32, i32, vp, i64, i64, vp, vp]
     L.i8f_lora_merge_sr.argtypes = [vp, vp, f32, i32, vp, vp, vp, i64, f32, vp, i64, i64, vp, vp]
     for name in ("i8f_quant_rowwise_concat_gelu", "i8f_quant_rowwise_rms_norm", "i8f_linear_w8a8_gated", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_rotate128", "i8f_gemm_i32", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora",
-                 "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
+                 "i8f_linear_w8a16_small_m", "i8f_linear_w8a16_small_m_grouped", "i8f_sr_quant_delta", "i8f_lora_merge_sr"):
         getattr(L, name).restype = i32
     _lib = L
     return L
@@ -88,7 +89,7 @@ EXPORTS = (
     "i8f_version", "i8f_status_string", "i8f_last_hip_error", "i8f_quant_rowwise", "i8f_quant_rowwise_grouped", "i8f_rotate128",
     "i8f_quant_tensorwise_workspace_bytes", "i8f_quant_tensorwise", "i8f_quant_tensorwise_static", "i8f_quant_rowwise_prologue", "i8f_quant_rowwise_norm_modulate", "i8f_quant_rowwise_concat_gelu",
     "i8f_quant_rowwise_rms_norm",
-    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_gated", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
+    "i8f_gemm_i32", "i8f_gemm_tile", "i8f_linear_w8a8", "i8f_linear_w8a8_add", "i8f_linear_w8a8_workspace_bytes", "i8f_linear_w8a8_splitk", "i8f_linear_w8a8_gated", "i8f_linear_w8a8_grouped", "i8f_linear_w8a8_lora", "i8f_linear_w8a16_small_m", "i8f_linear_w8a16_small_m_grouped", "i8f_sr_quant_delta", "i8f_lora_merge_sr",
 )
 
 
@@ -664,6 +665,52 @@ def linear_w8a16_small_m(x, w, w_scale, bias=None):
         _check(lib().i8f_linear_w8a16_small_m(_ptr(x), dtype_code(x.dtype), M, K, ldx, _ptr(w), _ptr(ws), ws_host, mode,
                                               _ptr(bias), bcode, _ptr(out), N, _stream(x)), "i8f_linear_w8a16_small_m")
     return out
+
+
+class _SmallMGroup(ctypes.Structure):
+    _fields_ = [("a", ctypes.c_void_p), ("M", ctypes.c_int64), ("K", ctypes.c_int64), ("ldx", ctypes.c_int64), ("w", ctypes.c_void_p),
+                ("w_scale", ctypes.c_void_p), ("w_scale_host", ctypes.c_float), ("bias", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("N", ctypes.c_int64)]
+
+
+def linear_w8a16_small_m_grouped(problems):
+    """[linear_w8a16_small_m(x, w, w_scale, bias) for (x, w, w_scale, bias) in problems] with all layers in one launch
+    where the library has a grouped kernel for them (up to 4 layers, 16-bit activations of one dtype, one scale mode and
+    one bias dtype); anything else goes layer by layer.  Results are those of the separate calls bit for bit."""
+    problems = [tuple(p) + (None,) * (4 - len(p)) for p in problems]
+    if not problems:
+        return []
+    x0 = problems[0][0]
+    _dev(x0, "x")
+    prepared, keep = [], []
+    for x, w, w_scale, bias in problems:
+        _dev(x, "x")
+        x = _rows(x, "x")
+        w = _i8_matrix(w, "w")
+        if x.shape[1] != w.shape[1]:
+            raise ValueError(f"K mismatch: x has {x.shape[1]}, w has {w.shape[1]}")
+        ws, ws_host, mode = _scale(w_scale, w.shape[0], x.device)
+        b, bcode = _bias_arg(bias, w.shape[0], x.device)
+        prepared.append((x, w, ws, ws_host, mode, b, bcode))
+    modes = {p[4] for p in prepared}
+    bcodes = {p[6] for p in prepared if p[5] is not None}
+    same = (len(problems) <= MAX_LINEAR_GROUPS and len(modes) == 1 and len(bcodes) <= 1
+            and all(p[0].dtype == x0.dtype and p[0].device == x0.device for p in prepared))
+    if not same:
+        return [linear_w8a16_small_m(x, w, w_scale, bias) for x, w, w_scale, bias in problems]
+    groups = (_SmallMGroup * len(prepared))()
+    outs = []
+    for g, (x, w, ws, ws_host, mode, b, bcode) in zip(groups, prepared):
+        M, K = x.shape
+        out = torch.empty((M, w.shape[0]), dtype=x.dtype, device=x.device)
+        g.a, g.M, g.K, g.ldx, g.w = _addr(x), M, K, (x.stride(0) if M > 1 else K), _addr(w)
+        g.w_scale, g.w_scale_host, g.bias, g.out, g.N = _addr(ws), ws_host, _addr(b), _addr(out), w.shape[0]
+        outs.append(out)
+        keep.append((x, w, ws, b))
+    with _on(x0.device):
+        _check(lib().i8f_linear_w8a16_small_m_grouped(groups, len(prepared), dtype_code(x0.dtype), modes.pop(),
+                                                      bcodes.pop() if bcodes else BF16, _stream(x0)), "i8f_linear_w8a16_small_m_grouped")
+    return outs
 
 
 def _f32_matrix(t, name, device):

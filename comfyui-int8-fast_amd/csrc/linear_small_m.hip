@@ -165,8 +165,10 @@ __device__ __forceinline__ v4f_t mma8(uint32_t wlo, uint32_t whi, v4u_t xk, floa
 // the wave, so no barrier is involved.  Fetching straight into the operand layout (16 rows per
 // instruction, 16 or more cache lines) measured 12 % slower, and slower still the more lines an
 // instruction touched.
+// (The body is shared by the kernel of one layer and the kernel of several layers in one launch: `block` is the
+// workgroup's number within its layer.)
 template <int DT, int NB, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void small_m_lds_kernel(const SmallMArgs a) {
+__device__ __forceinline__ void small_m_lds_body(const SmallMArgs &a, const int64_t block) {
     constexpr int COLS = NB * 16;
     constexpr int PITCH = 144;
     __shared__ float red[WAVES][COLS][16];
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(WAVES * 64) void small_m_lds_kernel(const SmallMArg
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
     const int lr = lane >> 3, lc = lane & 7;   // fetch layout: row within 8, 16-byte column
-    const int64_t n0 = (int64_t)blockIdx.x * COLS;
+    const int64_t n0 = block * COLS;
     const int K = (int)a.K;
     const int nsteps = (K + 127) / 128;
     const bool xrow = r < (int)a.M;
@@ -274,6 +276,35 @@ __global__ __launch_bounds__(WAVES * 64) void small_m_lds_kernel(const SmallMArg
 }
 
 template <int DT, int NB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void small_m_lds_kernel(const SmallMArgs a) {
+    small_m_lds_body<DT, NB, WAVES>(a, (int64_t)blockIdx.x);
+}
+
+// Several layers in one launch (the modulation projections of the image and of the text stream of a double-stream
+// block read the same conditioning vector through their own weights): a weight stream of 57 MB lasts 13 us, of which
+// ramp-up and drain are a good part; two of them back to back in one grid keep the memory system busy through the seam.
+constexpr int MAX_SMALL_M_GROUPS = 4;
+struct SmallMGroups {
+    SmallMArgs a[MAX_SMALL_M_GROUPS];
+    int first_block[MAX_SMALL_M_GROUPS + 1];
+    int n;
+};
+
+template <int DT, int NB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void small_m_lds_grouped_kernel(const SmallMGroups gg) {
+    int grp = 0;
+#pragma unroll
+    for (int i = 1; i < MAX_SMALL_M_GROUPS; ++i)
+        if (i < gg.n && (int)blockIdx.x >= gg.first_block[i]) grp = i;
+    // (selected with constant indices: the argument structure then stays in scalar registers)
+    SmallMArgs a = gg.a[0];
+#pragma unroll
+    for (int i = 1; i < MAX_SMALL_M_GROUPS; ++i)
+        if (grp == i) a = gg.a[i];
+    small_m_lds_body<DT, NB, WAVES>(a, (int64_t)((int)blockIdx.x - gg.first_block[grp]));
+}
+
+template <int DT, int NB, int WAVES>
 int launch_lds(const SmallMArgs &a, hipStream_t st) {
     const int64_t cols = NB * 16;
     hipLaunchKernelGGL((small_m_lds_kernel<DT, NB, WAVES>), dim3((unsigned)((a.N + cols - 1) / cols)), dim3(WAVES * 64), 0, st, a);
@@ -301,8 +332,72 @@ int launch(const SmallMArgs &a, hipStream_t st) {
     return check_launch();
 }
 
+// the layers of a group launch: all of them on the fast path, with the same block form
+template <int DT>
+int launch_grouped(const SmallMArgs *as, int n, hipStream_t st) {
+    SmallMGroups gg{};
+    gg.n = n;
+    int64_t total_blocks16 = 0;
+    for (int i = 0; i < n; ++i) total_blocks16 += (as[i].N + 15) / 16;
+    const bool two = (total_blocks16 + 1) / 2 >= 256;     // as for one layer: two 16-column blocks per workgroup once every CU has one
+    const int64_t cols = two ? 32 : 16;
+    int64_t first = 0;
+    for (int i = 0; i < n; ++i) {
+        gg.a[i] = as[i];
+        gg.first_block[i] = (int)first;
+        first += (as[i].N + cols - 1) / cols;
+    }
+    for (int i = n; i <= MAX_SMALL_M_GROUPS; ++i) gg.first_block[i] = (int)first;
+    if (first > 0x7fffffff) return I8F_ERR_UNSUPPORTED;
+    if (two) hipLaunchKernelGGL((small_m_lds_grouped_kernel<DT, 2, 8>), dim3((unsigned)first), dim3(512), 0, st, gg);
+    else hipLaunchKernelGGL((small_m_lds_grouped_kernel<DT, 1, 8>), dim3((unsigned)first), dim3(512), 0, st, gg);
+    return check_launch();
+}
+
 }  // namespace
 }  // namespace i8f
+
+extern "C" int i8f_linear_w8a16_small_m_grouped(const i8f_small_m_group *groups, int n_groups, int x_dtype, int scale_mode,
+                                                int bias_dtype, void *stream) {
+    using namespace i8f;
+    if (n_groups < 0 || (n_groups > 0 && !groups) || !valid_dtype(x_dtype)) return I8F_ERR_INVALID;
+    if (scale_mode != I8F_SCALE_TENSOR && scale_mode != I8F_SCALE_ROW) return I8F_ERR_INVALID;
+    bool one_launch = n_groups >= 2 && n_groups <= MAX_SMALL_M_GROUPS && x_dtype != I8F_F32;
+    bool any_bias = false;
+    for (int i = 0; i < n_groups; ++i) {
+        const i8f_small_m_group &g = groups[i];
+        if (g.M < 0 || g.N < 0 || g.K < 0) return I8F_ERR_INVALID;
+        if (g.M > 16) return I8F_ERR_UNSUPPORTED;
+        if (g.M > 0 && g.N > 0) {
+            if (!g.out || g.ldx < g.K || (g.K > 0 && (!g.a || !g.w)) || (scale_mode == I8F_SCALE_ROW && !g.w_scale)) return I8F_ERR_INVALID;
+        }
+        any_bias = any_bias || g.bias;
+        // what the fast kernel asks of a layer (as the single-layer entry point checks it)
+        one_launch = one_launch && g.M > 0 && g.N > 0 && g.K % 16 == 0 && g.K > 0 && g.K < (1ll << 30) && (uintptr_t)g.w % 16 == 0 &&
+                     (uintptr_t)g.a % 16 == 0 && (g.ldx * 2) % 16 == 0;
+    }
+    if (any_bias && !valid_dtype(bias_dtype)) return I8F_ERR_INVALID;
+    if (!one_launch) {   // shapes without a grouped kernel: one launch per layer, same results
+        for (int i = 0; i < n_groups; ++i) {
+            const i8f_small_m_group &g = groups[i];
+            if (int rc = i8f_linear_w8a16_small_m(g.a, x_dtype, g.M, g.K, g.ldx, g.w, g.w_scale, g.w_scale_host, scale_mode, g.bias,
+                                                  bias_dtype, g.out, g.N, stream))
+                return rc;
+        }
+        return I8F_OK;
+    }
+    if (int rc = check_device()) return rc;
+    SmallMArgs as[MAX_SMALL_M_GROUPS];
+    for (int i = 0; i < n_groups; ++i) {
+        const i8f_small_m_group &g = groups[i];
+        as[i] = SmallMArgs{};
+        as[i].x = g.a, as[i].M = g.M, as[i].K = g.K, as[i].ldx = g.ldx, as[i].N = g.N, as[i].w = g.w, as[i].ws = g.w_scale;
+        as[i].ws_host = g.w_scale_host, as[i].row_scale = scale_mode == I8F_SCALE_ROW, as[i].bias = g.bias, as[i].bias_dtype = bias_dtype;
+        as[i].out = g.out;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    return x_dtype == I8F_BF16 ? launch_grouped<I8F_BF16>(as, n_groups, st) : launch_grouped<I8F_F16>(as, n_groups, st);
+}
 
 extern "C" int i8f_linear_w8a16_small_m(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                                         const int8_t *w, const float *w_scale, float w_scale_host, int scale_mode,

@@ -148,11 +148,32 @@ def forward_fanout(layers, x, prologue: int = _lib.PRO_NONE, mod_scale=None, mod
     inside that quantiser, as forward(x, prologue=...) does for one layer -- and every layer runs its GEMM on the shared
     int8 rows.  The reference quantises in every Linear.forward (int8_quant.py:703-778); the quantiser being a function
     of its input, results are bit-identical to the layers' own forward calls, which is also the fall-back where a layer
-    is not on the W8A8 path (16 rows or fewer, dynamic LoRA, managed casting, different rotation flags, tracing)."""
+    is not on the W8A8 path (dynamic LoRA, managed casting, different rotation flags, tracing).  With 16 rows or fewer
+    (no prologue) the layers' small-batch W8A16 kernels go out as one launch instead."""
     layers = list(layers)
     if prologue == _lib.PRO_MODULATE_FUSED:
         prologue, fused_add = _lib.PRO_MODULATE, True
     rot = bool(getattr(layers[0], "_use_quarot", False)) if layers else False
+    # 16 rows or fewer (the modulation projections of a block, which read the conditioning vector): the small-batch
+    # W8A16 kernel of all the layers in one launch
+    if (len(layers) >= 2 and prologue == _lib.PRO_NONE and not torch.compiler.is_compiling() and x.is_cuda and x.dim() >= 1
+            and 0 < x.numel() // max(1, x.shape[-1]) <= SMALL_BATCH_ROWS and x.dtype in (torch.float16, torch.bfloat16)
+            and all(getattr(lin, "_is_quantized", False) and lin.lora_A is None and lin.weight.device == x.device
+                    and not (lin.comfy_cast_weights or len(lin.weight_function) > 0 or len(lin.bias_function) > 0)
+                    and (lin.bias is None or lin.bias.device == x.device) and bool(getattr(lin, "_use_quarot", False)) == rot
+                    and lin.weight.shape[1] == x.shape[-1] for lin in layers)):
+        x_2d = x.reshape(-1, x.shape[-1])
+        x_in = _lib.rotate128(x_2d) if rot else x_2d
+        problems = []
+        for lin in layers:
+            ws = lin._get_weight_scale()
+            if isinstance(ws, Tensor):
+                if ws.device != x.device:
+                    ws = ws.to(x.device, non_blocking=True)
+                if not lin._is_per_row and ws.numel() != 1:
+                    ws = ws.reshape(-1)[:1]
+            problems.append((x_in, lin.weight, ws, lin.bias))
+        return [y.reshape(*x.shape[:-1], y.shape[-1]) for y in _lib.linear_w8a16_small_m_grouped(problems)]
     ok = len(layers) >= 2 and not torch.compiler.is_compiling() and x.is_cuda and x.dim() >= 2 \
         and x.numel() // max(1, x.shape[-1]) > SMALL_BATCH_ROWS and x.dtype in (torch.float16, torch.bfloat16)
     for lin in layers:

@@ -437,6 +437,30 @@ int i8f_linear_w8a16_small_m(const void *x, int x_dtype, int64_t M, int64_t K, i
                              int64_t N, void *stream);
 
 /*
+ * i8f_linear_w8a16_small_m for several layers in one launch: the modulation projections of the image and of the
+ * text stream of a double-stream block, each Linear.forward(vec) with M <= 16 on its own weight (int8_quant.py:756-760
+ * called once per layer).  No counterpart in the reference, whose operator takes one layer; results are those of the
+ * separate calls bit for bit.  Why: a weight stream of tens of megabytes lasts little longer than the memory system
+ * takes to ramp up and drain, and two of them in one grid keep it busy through the seam.
+ *   groups[i]: a [M,K] of x_dtype (row stride ldx), w int8 [N,K], w_scale / w_scale_host as above, bias [N] of
+ *   bias_dtype or NULL, out [M,N] of x_dtype.  x_dtype, scale_mode and bias_dtype are shared.
+ * Up to 4 layers with 16-bit activations, K % 16 == 0 and 16-byte aligned operands take one launch; anything else is
+ * launched layer by layer.  The array is read on the host during the call.
+ */
+typedef struct i8f_small_m_group {
+    const void *a;
+    int64_t M, K, ldx;
+    const int8_t *w;
+    const float *w_scale;
+    float w_scale_host;
+    const void *bias;
+    void *out;
+    int64_t N;
+} i8f_small_m_group;
+int i8f_linear_w8a16_small_m_grouped(const i8f_small_m_group *groups, int n_groups, int x_dtype, int scale_mode,
+                                     int bias_dtype, void *stream);
+
+/*
  * Stochastic rounding of a float delta to int8 with SUPPLIED uniform noise.
  * Replaces stochastic_round_int8_delta (int8_quant.py:36-62); the reference
  * draws the noise from a device generator (:41,55), which no other device can

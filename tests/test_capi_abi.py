@@ -18,7 +18,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points(L):
     names = declared_functions()
     assert set(names) == set(L.EXPORTS)
-    assert len(names) == 25
+    assert len(names) == 26
 
 
 def test_library_exports_every_declared_symbol(L):
@@ -106,7 +106,16 @@ def test_bad_arguments_are_rejected_before_any_launch(L):
     assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 200, 200, 1e-6, null, null, null, 1, 0, 128, one, one, null) == INVALID
     assert lib.i8f_quant_rowwise_rms_norm(one, L.BF16, 4, 256, 128, 1e-6, null, null, null, 1, 0, 0, one, one, null) == INVALID
     assert lib.i8f_quant_rowwise_rms_norm(null, L.BF16, 0, 256, 256, 1e-6, null, null, null, 1, 0, 0, null, null, null) == 0
-    assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, 8, null, null, 1, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, 9, null, null, 1, 0, one, one, null) == INVALID
+    assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, 8, null, null, 1, 0, one, one, null) == INVALID   # fused modulation without vectors
+    grp = (L._SmallMGroup * 2)()
+    assert lib.i8f_linear_w8a16_small_m_grouped(grp, 0, L.BF16, 1, 0, null) == 0
+    assert lib.i8f_linear_w8a16_small_m_grouped(null, 2, L.BF16, 1, 0, null) == INVALID
+    assert lib.i8f_linear_w8a16_small_m_grouped(grp, 2, 9, 1, 0, null) == INVALID
+    grp[0].M, grp[0].N, grp[0].K, grp[0].ldx = 17, 16, 16, 16
+    assert lib.i8f_linear_w8a16_small_m_grouped(grp, 2, L.BF16, 1, 0, null) == UNSUPPORTED
+    grp[0].M = 4
+    assert lib.i8f_linear_w8a16_small_m_grouped(grp, 2, L.BF16, 1, 0, null) == INVALID   # no pointers
     assert lib.i8f_quant_rowwise_prologue(one, L.BF16, 4, 256, 256, L.PRO_NORM_MODULATE, one, one, 4, 0, one, one, null) == INVALID  # needs its own entry point: it carries eps
     # concatenating quantiser: negative widths, operands missing, a rotation block that would straddle the seam, binary32,
     # widths that are not whole runs of 16, more than 16384 columns

@@ -426,6 +426,9 @@ def test_forward_fanout_equals_the_layers_own_forward(pkg, dev, quarot):
     assert all((o.float() - lin(h).float()).abs().max() <= 2.0**-6 * lin(h).float().abs().max() for o, lin in zip(outs, (q, v)))
     small = x[:1, :5]
     assert all(torch.equal(o, lin(small)) for o, lin in zip(pkg.forward_fanout([q, k], small), (q, k)))
+    vec = x[:, 0]                                      # [2, 384]: the small-batch kernels of all three layers in one launch
+    outs = pkg.forward_fanout([q, k, v], vec)
+    assert [tuple(o.shape) for o in outs] == [(2, 192), (2, 96), (2, 64)] and all(torch.equal(o, lin(vec)) for o, lin in zip(outs, (q, k, v)))
     k._use_quarot = not quarot
     assert all(torch.equal(o, lin(x)) for o, lin in zip(pkg.forward_fanout([q, k], x), (q, k)))
     per_token = (torch.randn(1, 50, 384, generator=g) * 0.3).bfloat16().to(dev)      # a scale torch would broadcast differently

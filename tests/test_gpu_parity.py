@@ -1237,3 +1237,30 @@ def test_linear_w8a8_k_split_flags_sweep(L, dev):
             fused = L.linear_w8a8(q, s, wq.to(dev), ws.to(dev) if row else float(ws[0]), None if bias is None else bias.to(dev), odt, order, addend=add)
             assert torch.equal(fused, (got + add).to(odt))
 
+
+
+@pytest.mark.parametrize("dt,M,shapes,bias,per_row", [
+    (torch.bfloat16, 1, [(18432, 3072), (18432, 3072)], True, True), (torch.float16, 16, [(512, 1024), (96, 1024), (2048, 1024)], False, True),
+    (torch.bfloat16, 5, [(33, 272), (17, 272)], True, False), (torch.bfloat16, 3, [(64, 256)] * 4, True, True),
+    (torch.float32, 4, [(64, 256), (32, 256)], True, True), (torch.bfloat16, 2, [(64, 256)] * 5, False, True),
+    (torch.bfloat16, 2, [(64, 200), (64, 264)], True, True),
+])
+def test_linear_w8a16_small_m_grouped_equals_separate_calls(L, dev, dt, M, shapes, bias, per_row):
+    """Several small-batch layers in one launch (the modulation projections of both streams of a block) == the
+    separate calls bit for bit: layers of different widths and depths, with and without bias, one weight scale or one
+    per row, and the shapes without a grouped kernel (binary32 activations, more than four layers, K % 16 != 0), which
+    go layer by layer."""
+    g = torch.Generator().manual_seed(71)
+    problems = []
+    for (N, K) in shapes:
+        x = torch.randn(M, K, generator=g).to(dt).to(dev)
+        w = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g).to(dev)
+        ws = (torch.rand(N, 1, generator=g) * 0.002 + 1e-3).to(dev) if per_row else 0.0017
+        b = torch.randn(N, generator=g).to(dt).to(dev) if bias else None
+        problems.append((x, w, ws, b))
+    outs = L.linear_w8a16_small_m_grouped(problems)
+    assert len(outs) == len(problems)
+    for (x, w, ws, b), y in zip(problems, outs):
+        want = L.linear_w8a16_small_m(x, w, ws, b)
+        assert y.shape == want.shape and y.dtype == want.dtype
+        assert torch.equal(y.view(torch.int32) if dt == torch.float32 else y.view(torch.int16), want.view(torch.int32) if dt == torch.float32 else want.view(torch.int16))
